@@ -1,0 +1,79 @@
+/*
+ * titanic_moe.h -- C ABI of libtitanic_moe_hip.so, the MI355X (gfx950) implementation of Titanic Flash's MoE FFN layer.
+ *
+ * The library is the drop-in for the native objects the reference's Rust FFN operators bind:
+ *   libcanada_ffn.so              (src/ffn.rs:42-84:        ca_ffn_abi, ca_router_logits, ca_shared_swiglu, ca_ffn_add)
+ *   libcanada_moe_primitives.so   (src/primitives.rs:45-182: ca_primitives_abi / open / close / launch / launch2)
+ *   core.cubin / shared.cubin     (kernels resolved by name and launched through src/cuda.rs Function::launch)
+ * Conventions are the reference's (runtime/kernels/moe-runtime-m6-cache-ca-v1/bridge.cc): 0 = success, negative =
+ * argument validation (-1 null / range, -2 arity, -3 unknown index, -4 unsupported geometry), positive = hipError_t.
+ * No entry point allocates, frees or synchronizes; every launch goes to the stream passed in (a hipStream_t as void*),
+ * so calls can be captured into a HIP graph.  All pointers are device pointers unless stated otherwise.
+ *
+ * Shapes are not compiled in: ca_ffn_configure() sets the process geometry used by the fixed-signature entry points,
+ * and ca_primitives_open() snapshots it into the context it returns.
+ */
+#ifndef TITANIC_MOE_H
+#define TITANIC_MOE_H
+#include <stddef.h>
+#include <stdint.h>
+#ifdef __cplusplus
+extern "C" {
+#endif
+
+typedef struct ca_geometry {
+    int32_t hidden;               /* H, multiple of 512 */
+    int32_t experts;              /* E <= 512 */
+    int32_t topk;                 /* K <= 8 */
+    int32_t intermediate;         /* routed expert intermediate I, multiple of 512 */
+    int32_t shared_intermediate;  /* shared expert intermediate, multiple of 512 */
+    int32_t scoring;              /* 0 sigmoid, 1 sqrt(softplus) (reference: 1, src/ffn.rs:249) */
+    float route_scale;            /* routed_scaling_factor (reference: 1.5, src/ffn.rs:250) */
+    int32_t act_block;            /* activation quantization block: 32 (reference) or 128 */
+    int32_t shared_bn, shared_bk; /* shared-expert weight scale block (reference: 32 x 32, src/blockscaled.rs:161-171) */
+    int64_t alt_token;            /* token id that selects the alternative bias (reference: 129264), -1 none */
+    float swiglu_limit;           /* 10 (src/ffn.rs:66) */
+} ca_geometry;
+
+/* ---- libcanada_ffn.so surface (runtime/kernels/ffn-native-v1/ffn.cu:259-276) ----------------------------------- */
+int ca_ffn_abi(void);                                   /* ffn.cu:259: returns 1 */
+int ca_ffn_configure(const ca_geometry* geometry);      /* additive: replaces the reference's compiled-in 5120/384/576 */
+int ca_ffn_geometry(ca_geometry* out);                  /* additive: reads the process geometry back */
+/* ffn.cu:260-265.  logits[rows][E] (f32) = x[rows][H] (bf16) . w[E][H]^T (bf16), rows 1..16. */
+int ca_router_logits(int rows, const void* x, const void* w, void* out, void* stream);
+/* ffn.cu:266-271.  out[rows][Is] (bf16) = clipped SwiGLU of in[rows][gate | up] (bf16), rows 1..65536. */
+int ca_shared_swiglu(int rows, const void* input, void* output, void* stream);
+/* ffn.cu:272-276.  out = bf16(f32(routed) + f32(shared)) over rows x H, rows 1..65536. */
+int ca_ffn_add(int rows, const void* routed, const void* shared, void* out, void* stream);
+/* Additive: the gate product for any row count (rows > 16 use the matrix-core kernel, whose summation order differs). */
+int ca_router_logits_wide(int rows, const void* x, const void* w, void* out, void* stream);
+
+/* ---- kernels the reference resolves by name from a code module (src/cuda.rs:199-226 Module::function + launch) -- */
+/* Launches the `extern "C" __global__` kernel `name` with the reference's launch tuple ([grid;3], [block;3], dynamic
+ * shared bytes, stream, argument pointers).  -3 for an unknown name.  The same kernels are in titanic_moe_gfx950.hsaco
+ * for hosts that load code objects with hipModuleLoadData / hipModuleGetFunction. */
+int ca_kernel_launch(const char* name, const uint32_t grid[3], const uint32_t block[3], uint32_t shared_bytes, void** args,
+                     void* stream);
+int ca_kernel_count(void);
+const char* ca_kernel_name(int index);
+
+/* kernels/moe_nibble_layout_probe.cu:17-21 */
+int ca_moe_nibble_permute(void* data, uint64_t bytes, int inverse, void* stream);
+
+/* ---- operator ABI (src/primitives.rs:45-60, 91-182; bridge.cc) ------------------------------------------------- */
+int32_t ca_primitives_abi(void);                /* returns 1 */
+void* ca_primitives_open(int32_t* status);      /* host handle; snapshots the process geometry and the device's CU count */
+void ca_primitives_close(void* context);
+/* Entries, pointer and scalar lists: titanic-flash-41_amd/contracts/bindings.json (same schema as the reference's). */
+int32_t ca_primitives_launch(void* context, int32_t index, const uint64_t* pointers, size_t pointer_count,
+                             const int32_t* scalars, size_t scalar_count, void* stream);
+/* words = pointers followed by scalars widened to 64 bits (src/primitives.rs:153-182). */
+int32_t ca_primitives_launch2(void* context, int32_t index, const uint64_t* words, size_t word_count, void* stream);
+int32_t ca_primitives_entries(void);            /* additive: number of entries */
+/* additive: scratch bytes entry `index` needs for `rows` token rows (the role "scratch" of the runtime contract). */
+int64_t ca_primitives_scratch_bytes(void* context, int32_t index, int32_t rows);
+
+#ifdef __cplusplus
+}
+#endif
+#endif

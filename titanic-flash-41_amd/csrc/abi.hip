@@ -1,0 +1,396 @@
+// C ABI of libtitanic_moe_hip.so: the entry points the reference's Rust FFN operators bind (see include/titanic_moe.h).
+// Nothing here allocates, frees or synchronizes; every entry point only enqueues kernels on the caller's stream.
+#include "../../include/titanic_moe.h"
+#include "combine.cuh"
+#include "experts_gemm.cuh"
+#include "experts_stream.cuh"
+#include "packing.cuh"
+#include "shared.cuh"
+#include <cstdlib>
+#include <cstring>
+
+namespace {
+
+ca_geometry g_geometry = {5120, 384, 6, 576, 576, 1, 1.5f, 32, 32, 32, 129264, 10.f};   // src/ffn.rs:65-66, 245-258
+
+bool supported_k(int k) { return k == 512 || k == 1024 || k == 2048 || k == 4096 || k == 8192; }
+int check_geometry(const ca_geometry& g) {
+    if (g.hidden <= 0 || g.hidden % 512 || g.experts <= 0 || g.experts > 512 || g.topk <= 0 || g.topk > 8 ||
+        g.topk > g.experts || g.intermediate <= 0 || g.intermediate % 512 || g.shared_intermediate <= 0 ||
+        g.shared_intermediate % 512 || (g.scoring != 0 && g.scoring != 1) || (g.act_block != 32 && g.act_block != 128) ||
+        g.shared_bn <= 0 || g.shared_bk <= 0 || g.shared_bk % 32 || g.hidden % g.shared_bk || g.shared_intermediate % g.shared_bk ||
+        g.hidden % g.shared_bn || (2 * g.shared_intermediate) % g.shared_bn)
+        return -4;
+    return 0;
+}
+int launch_status() { return (int)hipGetLastError(); }
+
+struct Context {
+    ca_geometry g;
+    int cus;
+    int stream_wgs;    // persistent workgroups of the streaming kernels
+};
+
+template <bool FP8>
+int launch_fc1_stream(const StreamArgs& a, int wgs, hipStream_t s) {
+    switch (a.k) {
+        case 512: tf_fc1_stream<FP8, 1><<<wgs, 256, 0, s>>>(a); break;
+        case 1024: tf_fc1_stream<FP8, 2><<<wgs, 256, 0, s>>>(a); break;
+        case 2048: tf_fc1_stream<FP8, 4><<<wgs, 256, 0, s>>>(a); break;
+        case 4096: tf_fc1_stream<FP8, 8><<<wgs, 256, 0, s>>>(a); break;
+        case 8192: tf_fc1_stream<FP8, 16><<<wgs, 256, 0, s>>>(a); break;
+        default: return -4;
+    }
+    return launch_status();
+}
+template <bool FP8>
+int launch_fc2_stream(const StreamArgs& a, int wgs, hipStream_t s) {
+    const size_t lds = 16 * (size_t)a.k + 16 * (size_t)(a.k / a.act_block);
+    switch (a.k) {
+        case 512: tf_fc2_stream<FP8, 1><<<wgs, 256, lds, s>>>(a); break;
+        case 1024: tf_fc2_stream<FP8, 2><<<wgs, 256, lds, s>>>(a); break;
+        case 2048: tf_fc2_stream<FP8, 4><<<wgs, 256, lds, s>>>(a); break;
+        case 4096: tf_fc2_stream<FP8, 8><<<wgs, 256, lds, s>>>(a); break;
+        default: return -4;
+    }
+    return launch_status();
+}
+
+// ---- entry 0 / 1: integration.tp_moe.dynamic -----------------------------------------------------------------------
+enum DynPtr {
+    P_A, P_IDS, P_WEIGHTS, P_PACKED, P_SCALES, P_PACKED_MIN, P_SCALES_MIN, P_INTER, P_INTER_CODES, P_INTER_SCALES,
+    P_TASK_EXPERT, P_TASK_VALID, P_TILE_BASE, P_TOKEN_MAP, P_TOKEN_WEIGHTS, P_W13, P_S13, P_W2, P_S2, P_SCATTER,
+    P_PLAN_SCRATCH, P_DYN_COUNT,
+    P_LOGITS = P_DYN_COUNT, P_BIAS, P_BIAS_ALT, P_TOKENS, P_LIVE, P_PADDING, P_ROUTE_COUNT
+};
+enum DynScalar { S_TOKENS, S_MAX_ROWS, S_ROWS_PADDED, S_MAX_TILES, S_TILE_M, S_GROUPS, S_DYN_COUNT, S_OWNER_ROWS = S_DYN_COUNT, S_ROUTE_COUNT };
+
+int launch_dynamic(const Context& c, bool route, const uint64_t* p, const int32_t* sc, hipStream_t s) {
+    const ca_geometry& g = c.g;
+    const int rows = sc[S_TOKENS], tile_m = sc[S_TILE_M], groups = sc[S_GROUPS], max_tiles = sc[S_MAX_TILES];
+    if (rows < 1 || rows > sc[S_MAX_ROWS] || groups < 1 || max_tiles < 1 || sc[S_ROWS_PADDED] != max_tiles * tile_m) return -1;
+    for (int i = 0; i < P_DYN_COUNT; ++i)
+        if (!p[i] && i != P_PACKED_MIN && i != P_SCALES_MIN && i != P_INTER_CODES && i != P_INTER_SCALES && i != P_PLAN_SCRATCH) return -1;
+    if (!supported_k(g.hidden) || !supported_k(g.intermediate)) return -4;
+    const long long pairs = (long long)rows * g.topk;
+    // worst case tiles: every expert opens one partial tile
+    const long long need_tiles = (pairs / tile_m) + (g.experts < pairs ? g.experts : pairs);
+    if (need_tiles > max_tiles) return -1;
+    const bool few = rows <= TF_STREAM_MAX_ROWS;
+    if (few ? tile_m != 16 : tile_m != TF_GEMM_TILE_M) return -1;
+
+    const uint16_t* x = (const uint16_t*)p[P_A];
+    int32_t* ids = (int32_t*)p[P_IDS];
+    float* weights = (float*)p[P_WEIGHTS];
+    if (pairs <= 1024 && g.experts < 1024) {
+        const int quant_blocks = (int)((((long long)rows * (g.hidden >> 3)) + 1023) / 1024);
+        if (route) {
+            const int owner = sc[S_OWNER_ROWS];
+            if (owner < rows || (long long)owner * g.topk > 1024) return -1;
+            for (int i = P_LOGITS; i <= P_LIVE; ++i) if (!p[i] && i != P_BIAS_ALT && i != P_TOKENS) return -1;
+            ca_moe_route_frontend<<<quant_blocks + 1, 1024, 0, s>>>(
+                x, ids, weights, (uint8_t*)p[P_PACKED], (uint8_t*)p[P_SCALES], (int32_t*)p[P_TOKEN_MAP], (float*)p[P_TOKEN_WEIGHTS],
+                (int32_t*)p[P_TASK_EXPERT], (int32_t*)p[P_TASK_VALID], (int32_t*)p[P_TILE_BASE], (const float*)p[P_LOGITS],
+                (const float*)p[P_BIAS], (const float*)p[P_BIAS_ALT], (const long long*)p[P_TOKENS], (const int32_t*)p[P_LIVE],
+                (const int32_t*)p[P_PADDING], rows, g.topk, g.experts, g.hidden, groups, tile_m, owner, g.act_block,
+                (uint8_t*)p[P_PACKED_MIN], (uint8_t*)p[P_SCALES_MIN], g.scoring, g.route_scale, (long long)g.alt_token);
+        } else {
+            ca_moe_frontend<<<quant_blocks, 1024, 0, s>>>(
+                x, ids, weights, (uint8_t*)p[P_PACKED], (uint8_t*)p[P_SCALES], (int32_t*)p[P_TOKEN_MAP], (float*)p[P_TOKEN_WEIGHTS],
+                (int32_t*)p[P_TASK_EXPERT], (int32_t*)p[P_TASK_VALID], (int32_t*)p[P_TILE_BASE], rows, g.topk, g.experts, g.hidden,
+                groups, tile_m, g.act_block, (uint8_t*)p[P_PACKED_MIN], (uint8_t*)p[P_SCALES_MIN]);
+        }
+    } else {
+        if (route || !p[P_PLAN_SCRATCH]) return -1;   // wide owners route with ca_route_topk first
+        const int waves = (int)((pairs + 63) / 64);
+        int32_t* wave_counts = (int32_t*)p[P_PLAN_SCRATCH];
+        int32_t* local_rank = wave_counts + (size_t)waves * g.experts;
+        ca_plan_wave_counts<<<(waves + 3) / 4, 256, 0, s>>>(ids, (int)pairs, g.experts, wave_counts, local_rank);
+        ca_plan_scan<<<1, 512, 0, s>>>(wave_counts, waves, g.experts, groups, tile_m, (int32_t*)p[P_TILE_BASE],
+                                       (int32_t*)p[P_TASK_EXPERT], (int32_t*)p[P_TASK_VALID]);
+        ca_plan_scatter<<<(int)((pairs + 255) / 256), 256, 0, s>>>(ids, weights, wave_counts, local_rank, (int32_t*)p[P_TILE_BASE],
+                                                                    (int)pairs, g.experts, tile_m, (int32_t*)p[P_TOKEN_MAP],
+                                                                    (float*)p[P_TOKEN_WEIGHTS]);
+        const long long items = (long long)rows * (g.hidden >> 3);
+        int blocks = (int)((items + 255) / 256);
+        if (blocks > c.cus * 16) blocks = c.cus * 16;
+        ca_quantize_rows<<<blocks, 256, 0, s>>>(x, (uint8_t*)p[P_PACKED], (uint8_t*)p[P_SCALES], (uint8_t*)p[P_PACKED_MIN],
+                                                (uint8_t*)p[P_SCALES_MIN], rows, g.hidden, g.act_block);
+    }
+    int status = launch_status();
+    if (status) return status;
+
+    const long long w13_stride = (long long)g.intermediate * g.hidden, s13_stride = w13_stride / 16;   // 2 I x H / 2, / 32
+    const long long w2_stride = (long long)g.hidden * g.intermediate / 2, s2_stride = w2_stride / 16;
+    if (few) {
+        StreamArgs a{};
+        a.a_codes = (const uint8_t*)p[P_PACKED]; a.a_scales = (const uint8_t*)p[P_SCALES];
+        a.w = (const uint8_t*)p[P_W13]; a.ws = (const uint8_t*)p[P_S13];
+        a.w_expert_stride = w13_stride; a.ws_expert_stride = s13_stride;
+        a.expert_tile_base = (const int32_t*)p[P_TILE_BASE]; a.task_expert = (const int32_t*)p[P_TASK_EXPERT];
+        a.task_valid_rows = (const int32_t*)p[P_TASK_VALID]; a.token_map = (const int32_t*)p[P_TOKEN_MAP];
+        a.token_weights = (const float*)p[P_TOKEN_WEIGHTS];
+        a.experts = g.experts; a.groups = groups; a.topk = g.topk;
+        a.k = g.hidden; a.inter = g.intermediate; a.hidden = g.hidden; a.act_block = g.act_block; a.limit = g.swiglu_limit;
+        a.out = (uint16_t*)p[P_INTER];
+        status = launch_fc1_stream<false>(a, c.stream_wgs, s);
+        if (status) return status;
+        StreamArgs b = a;
+        b.a_codes = nullptr; b.a_scales = nullptr; b.a_bf16 = (const uint16_t*)p[P_INTER];
+        b.q_codes = (uint8_t*)p[P_INTER_CODES]; b.q_scales = (uint8_t*)p[P_INTER_SCALES]; b.min_amax = 0.f;
+        b.w = (const uint8_t*)p[P_W2]; b.ws = (const uint8_t*)p[P_S2];
+        b.w_expert_stride = w2_stride; b.ws_expert_stride = s2_stride;
+        b.k = g.intermediate; b.out = (uint16_t*)p[P_SCATTER];
+        return launch_fc2_stream<false>(b, c.stream_wgs, s);
+    }
+    if (!p[P_INTER_CODES] || !p[P_INTER_SCALES]) return -1;
+    GemmArgs a{};
+    a.a_codes = (const uint8_t*)p[P_PACKED]; a.a_scales = (const uint8_t*)p[P_SCALES];
+    a.w = (const uint8_t*)p[P_W13]; a.ws = (const uint8_t*)p[P_S13];
+    a.w_expert_stride = w13_stride; a.ws_expert_stride = s13_stride;
+    a.expert_tile_base = (const int32_t*)p[P_TILE_BASE]; a.task_expert = (const int32_t*)p[P_TASK_EXPERT];
+    a.task_valid_rows = (const int32_t*)p[P_TASK_VALID]; a.token_map = (const int32_t*)p[P_TOKEN_MAP];
+    a.token_weights = (const float*)p[P_TOKEN_WEIGHTS];
+    a.experts = g.experts; a.groups = groups; a.topk = g.topk; a.max_tiles = max_tiles;
+    a.k = g.hidden; a.inter = g.intermediate; a.hidden = g.hidden; a.act_block = g.act_block; a.limit = g.swiglu_limit;
+    a.h_bf16 = (uint16_t*)p[P_INTER]; a.h_codes = (uint8_t*)p[P_INTER_CODES]; a.h_scales = (uint8_t*)p[P_INTER_SCALES];
+    a.out = (uint16_t*)p[P_SCATTER];
+    status = tf_launch_fc1_gemm(a, c.cus, s);
+    if (status) return status;
+    GemmArgs b = a;
+    b.a_codes = (const uint8_t*)p[P_INTER_CODES]; b.a_scales = (const uint8_t*)p[P_INTER_SCALES];
+    b.w = (const uint8_t*)p[P_W2]; b.ws = (const uint8_t*)p[P_S2];
+    b.w_expert_stride = w2_stride; b.ws_expert_stride = s2_stride;
+    b.k = g.intermediate;
+    return tf_launch_fc2_gemm(b, c.cus, s);
+}
+
+// ---- entry 2: moe.w4a16.topk_sum -----------------------------------------------------------------------------------
+int launch_topk_sum(const Context& c, const uint64_t* p, const int32_t* sc, hipStream_t s) {
+    if (!p[0] || !p[1] || sc[0] < 0 || sc[1] != 0 || sc[2] != 0) return -1;
+    if (sc[0] == 0) return 0;
+    const long long n8 = (long long)sc[0] * (c.g.hidden >> 3);
+    ca_moe_topk_sum<<<(int)((n8 + 255) / 256), 256, 0, s>>>((const uint16_t*)p[0], (uint16_t*)p[1], sc[0], c.g.topk, c.g.hidden,
+                                                           (const int32_t*)p[2], sc[0]);
+    return launch_status();
+}
+// ---- entry 3: gemm.mxfp8_quant_cute --------------------------------------------------------------------------------
+// pointers: input, values, scales (zero block -> scale 0), values_min, scales_min (amax floored at 1e-4); either pair may be null.
+int launch_quant(const Context& c, const uint64_t* p, const int32_t* sc, hipStream_t s) {
+    const int m = sc[0], k = sc[1];
+    if (!p[0] || (!p[1] != !p[2]) || (!p[3] != !p[4]) || (!p[1] && !p[3]) || m < 1 || k < c.g.act_block || k % c.g.act_block || sc[2] != 0)
+        return -1;
+    const long long items = (long long)m * (k >> 3);
+    int blocks = (int)((items + 255) / 256);
+    if (blocks > c.cus * 16) blocks = c.cus * 16;
+    ca_quantize_rows<<<blocks, 256, 0, s>>>((const uint16_t*)p[0], (uint8_t*)p[1], (uint8_t*)p[2], (uint8_t*)p[3], (uint8_t*)p[4], m, k,
+                                            c.g.act_block);
+    return launch_status();
+}
+// ---- entry 4: gemm.dense (FP8 x FP8 block-scaled -> BF16) -----------------------------------------------------------
+int launch_dense(const Context& c, const uint64_t* p, const int32_t* sc, hipStream_t s) {
+    const int m = sc[0], n = sc[1], k = sc[2];
+    for (int i = 0; i < 5; ++i) if (!p[i]) return -1;
+    if (m < 1 || n < 64 || n % 64 || !supported_k(k)) return -1;
+    if (m <= TF_STREAM_MAX_ROWS) {
+        StreamArgs a{};
+        a.a_codes = (const uint8_t*)p[0]; a.a_scales = (const uint8_t*)p[1];
+        a.w = (const uint8_t*)p[2]; a.ws = (const uint8_t*)p[3]; a.bn = c.g.shared_bn; a.bk = c.g.shared_bk;
+        a.dense_rows = m; a.k = k; a.hidden = n; a.act_block = c.g.act_block; a.out = (uint16_t*)p[4];
+        return launch_fc2_stream<true>(a, c.stream_wgs, s);
+    }
+    GemmArgs a{};
+    a.a_codes = (const uint8_t*)p[0]; a.a_scales = (const uint8_t*)p[1];
+    a.w = (const uint8_t*)p[2]; a.ws = (const uint8_t*)p[3]; a.bn = c.g.shared_bn; a.bk = c.g.shared_bk;
+    a.dense_rows = m; a.k = k; a.hidden = n; a.act_block = c.g.act_block; a.out = (uint16_t*)p[4];
+    return tf_launch_dense_gemm(a, c.cus, s);
+}
+// ---- entry 5: ffn.shared_expert (up + clipped SwiGLU + requant + down, from the quantized input) ---------------------
+enum SharedPtr { H_A, H_AS, H_W13, H_S13, H_W2, H_S2, H_ACT, H_ACT_CODES, H_ACT_SCALES, H_UP_TAP, H_OUT, H_COUNT };
+int launch_shared(const Context& c, const uint64_t* p, const int32_t* sc, hipStream_t s) {
+    const ca_geometry& g = c.g;
+    const int m = sc[0];
+    for (int i = 0; i < H_COUNT; ++i) if (!p[i] && i != H_UP_TAP && i != H_ACT_CODES && i != H_ACT_SCALES) return -1;
+    if (m < 1 || !supported_k(g.hidden) || !supported_k(g.shared_intermediate)) return -4;
+    if (m <= TF_STREAM_MAX_ROWS) {
+        StreamArgs a{};
+        a.a_codes = (const uint8_t*)p[H_A]; a.a_scales = (const uint8_t*)p[H_AS];
+        a.w = (const uint8_t*)p[H_W13]; a.ws = (const uint8_t*)p[H_S13]; a.bn = g.shared_bn; a.bk = g.shared_bk;
+        a.dense_rows = m; a.k = g.hidden; a.inter = g.shared_intermediate; a.hidden = g.hidden; a.act_block = g.act_block;
+        a.limit = g.swiglu_limit; a.out = (uint16_t*)p[H_ACT]; a.tap = (uint16_t*)p[H_UP_TAP];
+        int status = launch_fc1_stream<true>(a, c.stream_wgs, s);
+        if (status) return status;
+        StreamArgs b = a;
+        b.a_codes = nullptr; b.a_scales = nullptr; b.a_bf16 = (const uint16_t*)p[H_ACT];
+        b.q_codes = (uint8_t*)p[H_ACT_CODES]; b.q_scales = (uint8_t*)p[H_ACT_SCALES]; b.min_amax = 1e-4f;
+        b.w = (const uint8_t*)p[H_W2]; b.ws = (const uint8_t*)p[H_S2]; b.k = g.shared_intermediate; b.out = (uint16_t*)p[H_OUT];
+        b.tap = nullptr;
+        return launch_fc2_stream<true>(b, c.stream_wgs, s);
+    }
+    if (!p[H_ACT_CODES] || !p[H_ACT_SCALES]) return -1;
+    GemmArgs a{};
+    a.a_codes = (const uint8_t*)p[H_A]; a.a_scales = (const uint8_t*)p[H_AS];
+    a.w = (const uint8_t*)p[H_W13]; a.ws = (const uint8_t*)p[H_S13]; a.bn = g.shared_bn; a.bk = g.shared_bk;
+    a.dense_rows = m; a.k = g.hidden; a.inter = g.shared_intermediate; a.hidden = g.hidden; a.act_block = g.act_block;
+    a.limit = g.swiglu_limit; a.h_bf16 = (uint16_t*)p[H_ACT]; a.h_codes = (uint8_t*)p[H_ACT_CODES]; a.h_scales = (uint8_t*)p[H_ACT_SCALES];
+    a.tap = (uint16_t*)p[H_UP_TAP];
+    int status = tf_launch_shared_fc1_gemm(a, c.cus, s);
+    if (status) return status;
+    GemmArgs b{};
+    b.a_codes = (const uint8_t*)p[H_ACT_CODES]; b.a_scales = (const uint8_t*)p[H_ACT_SCALES];
+    b.w = (const uint8_t*)p[H_W2]; b.ws = (const uint8_t*)p[H_S2]; b.bn = g.shared_bn; b.bk = g.shared_bk;
+    b.dense_rows = m; b.k = g.shared_intermediate; b.hidden = g.hidden; b.act_block = g.act_block; b.out = (uint16_t*)p[H_OUT];
+    return tf_launch_dense_gemm(b, c.cus, s);
+}
+
+struct EntryShape { const char* kernel_id; size_t pointers, scalars; };
+const EntryShape kEntries[] = {
+    {"integration.tp_moe.dynamic", P_DYN_COUNT, S_DYN_COUNT},
+    {"integration.tp_moe.dynamic", P_ROUTE_COUNT, S_ROUTE_COUNT},
+    {"moe.w4a16.topk_sum", 3, 3},
+    {"gemm.mxfp8_quant_cute", 5, 3},
+    {"gemm.dense", 5, 3},
+    {"ffn.shared_expert", H_COUNT, 1},
+};
+constexpr int kEntryCount = sizeof(kEntries) / sizeof(kEntries[0]);
+
+struct KernelName { const char* name; const void* function; };
+#define TF_KERNEL(k) {#k, (const void*)k}
+const KernelName kKernels[] = {
+    TF_KERNEL(ca_router_logits_rows), TF_KERNEL(ca_route_topk), TF_KERNEL(ca_route_padding_rows), TF_KERNEL(ca_route_census),
+    TF_KERNEL(ca_moe_frontend), TF_KERNEL(ca_moe_route_frontend), TF_KERNEL(ca_quantize_rows), TF_KERNEL(ca_plan_wave_counts),
+    TF_KERNEL(ca_plan_scan), TF_KERNEL(ca_plan_scatter), TF_KERNEL(ca_shared_swiglu_rows), TF_KERNEL(ca_shared_swiglu_quant),
+    TF_KERNEL(ca_ffn_add_rows), TF_KERNEL(ca_moe_topk_sum), TF_KERNEL(ca_ffn_sum_shared), TF_KERNEL(ca_moe_group_sum_rows),
+    TF_KERNEL(ca_expert_compact_words), TF_KERNEL(ca_expert_expand_words), TF_KERNEL(ca_expert_compact_scales),
+    TF_KERNEL(ca_expert_expand_scales), TF_KERNEL(ca_dense_compact_fp8), TF_KERNEL(ca_moe_nibble_permute_words),
+    TF_KERNEL(ca_expert_scale_code1), TF_KERNEL(ca_expert_scale_code1_check), TF_KERNEL(ca_expert_scale_code1_census),
+    TF_KERNEL(ca_expert_scale_codes4), TF_KERNEL(ca_router_logits_mfma),
+};
+constexpr int kKernelCount = sizeof(kKernels) / sizeof(kKernels[0]);
+
+}  // namespace
+
+extern "C" {
+
+int ca_ffn_abi(void) { return 1; }
+int ca_ffn_configure(const ca_geometry* geometry) {
+    if (!geometry) return -1;
+    const int status = check_geometry(*geometry);
+    if (status) return status;
+    g_geometry = *geometry;
+    return 0;
+}
+int ca_ffn_geometry(ca_geometry* out) {
+    if (!out) return -1;
+    *out = g_geometry;
+    return 0;
+}
+int ca_router_logits(int rows, const void* x, const void* w, void* out, void* stream) {
+    if (rows < 1 || rows > 16 || !x || !w || !out) return -1;
+    ca_router_logits_rows<<<g_geometry.experts, 64, 0, (hipStream_t)stream>>>((const uint16_t*)x, (const uint16_t*)w, (float*)out, rows,
+                                                                              g_geometry.hidden, g_geometry.experts);
+    return launch_status();
+}
+int ca_router_logits_wide(int rows, const void* x, const void* w, void* out, void* stream) {
+    if (rows < 1 || !x || !w || !out) return -1;
+    if (rows <= 16) return ca_router_logits(rows, x, w, out, stream);
+    if (g_geometry.experts % 32 || g_geometry.hidden % 64) return -4;
+    const dim3 grid((rows + 63) / 64, g_geometry.experts / 32);
+    ca_router_logits_mfma<<<grid, 128, 0, (hipStream_t)stream>>>((const uint16_t*)x, (const uint16_t*)w, (float*)out, rows,
+                                                                 g_geometry.hidden, g_geometry.experts);
+    return launch_status();
+}
+int ca_shared_swiglu(int rows, const void* input, void* output, void* stream) {
+    if (rows < 1 || rows > 65536 || !input || !output) return -1;
+    const long long items = (long long)rows * (g_geometry.shared_intermediate >> 3);
+    ca_shared_swiglu_rows<<<(int)((items + 255) / 256), 256, 0, (hipStream_t)stream>>>(
+        (const uint16_t*)input, (uint16_t*)output, rows, g_geometry.shared_intermediate, g_geometry.swiglu_limit);
+    return launch_status();
+}
+int ca_ffn_add(int rows, const void* routed, const void* shared, void* out, void* stream) {
+    if (rows < 1 || rows > 65536 || !routed || !shared || !out) return -1;
+    const long long n8 = (long long)rows * (g_geometry.hidden >> 3);
+    ca_ffn_add_rows<<<(int)((n8 + 255) / 256), 256, 0, (hipStream_t)stream>>>((const uint16_t*)routed, (const uint16_t*)shared,
+                                                                              (uint16_t*)out, n8);
+    return launch_status();
+}
+int ca_moe_nibble_permute(void* data, uint64_t bytes, int inverse, void* stream) {
+    if (!data || bytes % 4 || (inverse != 0 && inverse != 1)) return -1;
+    ca_moe_nibble_permute_words<<<256, 256, 0, (hipStream_t)stream>>>((uint32_t*)data, bytes / 4, inverse);
+    return launch_status();
+}
+
+int ca_kernel_count(void) { return kKernelCount; }
+const char* ca_kernel_name(int index) { return index >= 0 && index < kKernelCount ? kKernels[index].name : nullptr; }
+int ca_kernel_launch(const char* name, const uint32_t grid[3], const uint32_t block[3], uint32_t shared_bytes, void** args, void* stream) {
+    if (!name || !grid || !block || !args) return -1;
+    if (!grid[0] || !grid[1] || !grid[2] || !block[0] || !block[1] || !block[2] || (uint64_t)block[0] * block[1] * block[2] > 1024) return -1;
+    for (int i = 0; i < kKernelCount; ++i)
+        if (!std::strcmp(name, kKernels[i].name))
+            return (int)hipLaunchKernel(kKernels[i].function, dim3(grid[0], grid[1], grid[2]), dim3(block[0], block[1], block[2]), args,
+                                        shared_bytes, (hipStream_t)stream);
+    return -3;
+}
+
+int32_t ca_primitives_abi(void) { return 1; }
+int32_t ca_primitives_entries(void) { return kEntryCount; }
+void* ca_primitives_open(int32_t* status) {
+    if (!status) return nullptr;
+    *status = check_geometry(g_geometry);
+    if (*status) return nullptr;
+    int device = 0, cus = 0;
+    hipError_t e = hipGetDevice(&device);
+    if (e == hipSuccess) e = hipDeviceGetAttribute(&cus, hipDeviceAttributeMultiprocessorCount, device);
+    if (e != hipSuccess) { *status = (int32_t)e; return nullptr; }
+    Context* c = new Context{g_geometry, cus, cus * 2};
+    if (const char* v = std::getenv("TITANIC_MOE_STREAM_WGS_PER_CU")) {
+        const int n = std::atoi(v);
+        if (n >= 1 && n <= 8) c->stream_wgs = cus * n;
+    }
+    return c;
+}
+void ca_primitives_close(void* context) { delete (Context*)context; }
+int32_t ca_primitives_launch(void* context, int32_t index, const uint64_t* pointers, size_t np, const int32_t* scalars, size_t ns,
+                             void* stream) {
+    if (!context || !pointers || !scalars) return -1;
+    if (index < 0 || index >= kEntryCount) return -3;
+    if (np != kEntries[index].pointers || ns != kEntries[index].scalars) return -2;
+    const Context& c = *(const Context*)context;
+    hipStream_t s = (hipStream_t)stream;
+    switch (index) {
+        case 0: return launch_dynamic(c, false, pointers, scalars, s);
+        case 1: return launch_dynamic(c, true, pointers, scalars, s);
+        case 2: return launch_topk_sum(c, pointers, scalars, s);
+        case 3: return launch_quant(c, pointers, scalars, s);
+        case 4: return launch_dense(c, pointers, scalars, s);
+        case 5: return launch_shared(c, pointers, scalars, s);
+        default: return -3;
+    }
+}
+int32_t ca_primitives_launch2(void* context, int32_t index, const uint64_t* words, size_t n, void* stream) {
+    if (!context || !words) return -1;
+    if (index < 0 || index >= kEntryCount) return -3;
+    const size_t np = kEntries[index].pointers, ns = kEntries[index].scalars;
+    if (n != np + ns) return -2;
+    int32_t scalars[16];
+    for (size_t i = 0; i < ns; ++i) scalars[i] = (int32_t)words[np + i];
+    return ca_primitives_launch(context, index, words, np, scalars, ns, stream);
+}
+int64_t ca_primitives_scratch_bytes(void* context, int32_t index, int32_t rows) {
+    if (!context || rows < 1 || (index != 0 && index != 1)) return -1;
+    const ca_geometry& g = ((const Context*)context)->g;
+    const long long pairs = (long long)rows * g.topk;
+    const int tile_m = rows <= TF_STREAM_MAX_ROWS ? 16 : TF_GEMM_TILE_M;
+    const long long tiles = pairs / tile_m + (g.experts < pairs ? g.experts : pairs), padded = tiles * tile_m;
+    long long bytes = 0;
+    auto add = [&](long long n) { bytes += (n + 255) / 256 * 256; };
+    add(2ll * rows * g.hidden); add(2ll * rows * g.hidden / g.act_block);              // packed + scales, both flavours
+    add(2ll * rows * g.hidden / g.act_block);
+    add(padded * g.intermediate * 2); add(padded * g.intermediate); add(padded * g.intermediate / g.act_block);
+    add(tiles * 4 * 8); add(tiles * 4 * 8); add((g.experts + 1) * 4ll); add(padded * 4); add(padded * 4);
+    add(pairs * g.hidden * 2);
+    add(((pairs + 63) / 64) * g.experts * 4 + pairs * 4);
+    return bytes;
+}
+
+}  // extern "C"

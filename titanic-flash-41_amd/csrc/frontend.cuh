@@ -1,0 +1,231 @@
+// Routed-expert front-end: route plan (counts, tiles, task tables, physical-row permutation) and the MXFP8
+// quantization of the token rows, with the router's top-k optionally inside.
+// Reference semantics: kernels/moe_frontend.cuh:158-265 (ca_moe_frontend / ca_moe_route_frontend).
+#pragma once
+#include "router.cuh"
+
+// Quantizes 8 consecutive BF16 values held by each lane of a group of `block / 8` adjacent lanes (one quantization
+// block per group).  Returns the routed-flavour codes (zero block -> scale byte 0) and, when asked, the shared-flavour
+// ones (amax floored at 1e-4).
+struct Quant8 { uint32_t lo, hi, exponent; };
+__device__ __forceinline__ Quant8 tf_quant8(const float (&v)[8], float amax, float min_amax) {
+    if (min_amax > 0.f) amax = fmaxf(amax, min_amax);
+    Quant8 q;
+    q.exponent = tf_block_exponent(amax);
+    const float inv = tf_block_inverse(q.exponent);
+    q.lo = tf_pack_e4m3(__fmul_rn(v[0], inv), __fmul_rn(v[1], inv), __fmul_rn(v[2], inv), __fmul_rn(v[3], inv));
+    q.hi = tf_pack_e4m3(__fmul_rn(v[4], inv), __fmul_rn(v[5], inv), __fmul_rn(v[6], inv), __fmul_rn(v[7], inv));
+    return q;
+}
+__device__ __forceinline__ float tf_group_amax(const float (&v)[8], int group_lanes) {
+    float amax = 0.f;
+#pragma unroll
+    for (int i = 0; i < 8; ++i) amax = fmaxf(amax, fabsf(v[i]));
+    for (int o = 1; o < group_lanes; o <<= 1) amax = fmaxf(amax, __shfl_xor(amax, o));
+    return amax;
+}
+// Quantizes `rows` x `cols` BF16 values in blocks of `block` (32 or 128) columns.  Work item = 8 values; items are
+// dealt to threads [first, first + count) of a virtual 1-D thread space with stride `stride`.
+__device__ __forceinline__ void tf_quantize_span(const uint16_t* __restrict__ input, uint8_t* __restrict__ codes,
+                                                 uint8_t* __restrict__ scales, uint8_t* __restrict__ codes_min,
+                                                 uint8_t* __restrict__ scales_min, long long total_items,
+                                                 int block, long long thread, long long stride) {
+    const int group_lanes = block >> 3;
+    // Whole groups stay together: thread and stride are multiples of 64 apart across waves, group_lanes divides 64.
+    const long long padded = (total_items + 63) & ~63ll;
+    for (long long q = thread; q < padded; q += stride) {
+        const bool on = q < total_items;
+        float v[8];
+        if (on) {
+            const u4v w = reinterpret_cast<const u4v*>(input)[q];
+#pragma unroll
+            for (int i = 0; i < 4; ++i) { v[2 * i] = tf_bf16_lo(w[i]); v[2 * i + 1] = tf_bf16_hi(w[i]); }
+        } else {
+#pragma unroll
+            for (int i = 0; i < 8; ++i) v[i] = 0.f;
+        }
+        const float amax = tf_group_amax(v, group_lanes);
+        if (!on) continue;
+        if (codes != nullptr) {
+            const Quant8 a = tf_quant8(v, amax, 0.f);
+            reinterpret_cast<u2v*>(codes)[q] = u2v{a.lo, a.hi};
+            if ((q & (group_lanes - 1)) == 0) scales[q / group_lanes] = (uint8_t)a.exponent;
+        }
+        if (codes_min != nullptr) {
+            const Quant8 b = tf_quant8(v, amax, 1e-4f);
+            reinterpret_cast<u2v*>(codes_min)[q] = u2v{b.lo, b.hi};
+            if ((q & (group_lanes - 1)) == 0) scales_min[q / group_lanes] = (uint8_t)b.exponent;
+        }
+    }
+}
+
+// Route plan of at most 1,024 routes by one block (the block's first `experts` threads own one expert each).
+__device__ __forceinline__ void tf_plan_block(const int32_t* ids, const float* weights, int32_t* token_map,
+                                              float* token_weights, int32_t* task_expert, int32_t* task_valid_rows,
+                                              int32_t* expert_tile_base, int pairs, int experts, int groups, int tile_m) {
+    __shared__ int32_t s_ids[1024];
+    __shared__ int32_t s_base[513];
+    __shared__ int32_t s_wave[16];
+    const int t = threadIdx.x, lane = t & 63, wave = t >> 6;
+    for (int p = t; p < pairs; p += blockDim.x) s_ids[p] = ids[p];
+    __syncthreads();
+    int count = 0;
+    if (t < experts) for (int p = 0; p < pairs; ++p) count += s_ids[p] == t;
+    const int tiles = (count + tile_m - 1) / tile_m;
+    int prefix = tiles;
+#pragma unroll
+    for (int o = 1; o < 64; o <<= 1) {
+        const int below = __shfl_up(prefix, o);
+        if (lane >= o) prefix += below;
+    }
+    if (lane == 63) s_wave[wave] = prefix;
+    __syncthreads();
+    int base = prefix - tiles;
+    for (int w = 0; w < wave; ++w) base += s_wave[w];
+    if (t <= experts) expert_tile_base[t] = base;
+    if (t < experts) {
+        s_base[t] = base;
+        for (int k = 0; k < tiles; ++k) {
+            const int valid = min(tile_m, count - k * tile_m);
+            for (int g = 0; g < groups; ++g) {
+                task_expert[(base + k) * groups + g] = t;
+                task_valid_rows[(base + k) * groups + g] = valid;
+            }
+        }
+    }
+    __syncthreads();
+    for (int p = t; p < pairs; p += blockDim.x) {
+        const int expert = s_ids[p];
+        if (expert >= 0 && expert < experts) {
+            int rank = 0;
+            for (int q = 0; q < p; ++q) rank += s_ids[q] == expert;
+            const int row = (s_base[expert] + rank / tile_m) * tile_m + rank % tile_m;
+            token_map[row] = p;
+            token_weights[row] = weights[p];
+        }
+    }
+}
+
+// Front-end of a few-row launch (rows * topk <= 1,024, experts < blockDim.x <= 1,024): block 0 plans the routes, the
+// blocks from `first` on quantize (first = 1: block 0 only routes and plans).
+__device__ __forceinline__ void tf_frontend_run(const uint16_t* input, const int32_t* ids, const float* weights,
+                                                uint8_t* packed, uint8_t* scales, uint8_t* packed_min, uint8_t* scales_min,
+                                                int32_t* token_map, float* token_weights, int32_t* task_expert,
+                                                int32_t* task_valid_rows, int32_t* expert_tile_base, int rows, int topk,
+                                                int experts, int cols, int groups, int tile_m, int act_block, int first) {
+    if (blockIdx.x == 0)
+        tf_plan_block(ids, weights, token_map, token_weights, task_expert, task_valid_rows, expert_tile_base,
+                      rows * topk, experts, groups, tile_m);
+    if ((int)blockIdx.x < first) return;
+    const long long total = (long long)rows * (cols >> 3);
+    tf_quantize_span(input, packed, scales, packed_min, scales_min, total, act_block,
+                     (long long)(blockIdx.x - first) * blockDim.x + threadIdx.x,
+                     (long long)(gridDim.x - first) * blockDim.x);
+}
+extern "C" __global__ void __launch_bounds__(1024) ca_moe_frontend(
+    const uint16_t* input, const int32_t* ids, const float* weights, uint8_t* packed, uint8_t* scales,
+    int32_t* token_map, float* token_weights, int32_t* task_expert, int32_t* task_valid_rows,
+    int32_t* expert_tile_base, int32_t rows, int32_t topk, int32_t experts, int32_t cols, int32_t groups,
+    int32_t tile_m, int32_t act_block, uint8_t* packed_min, uint8_t* scales_min) {
+    tf_frontend_run(input, ids, weights, packed, scales, packed_min, scales_min, token_map, token_weights, task_expert,
+                    task_valid_rows, expert_tile_base, rows, topk, experts, cols, groups, tile_m, act_block, 0);
+}
+// The front-end with the router's top-k inside: block 0 first routes every owner row from the gate's logits (and
+// applies padding routes), then plans; the other blocks quantize meanwhile (launch one block more).
+extern "C" __global__ void __launch_bounds__(1024) ca_moe_route_frontend(
+    const uint16_t* input, int32_t* ids, float* weights, uint8_t* packed, uint8_t* scales, int32_t* token_map,
+    float* token_weights, int32_t* task_expert, int32_t* task_valid_rows, int32_t* expert_tile_base,
+    const float* logits, const float* bias, const float* bias_alt, const long long* tokens, const int32_t* live,
+    const int32_t* padding, int32_t rows, int32_t topk, int32_t experts, int32_t cols, int32_t groups, int32_t tile_m,
+    int32_t owner_rows, int32_t act_block, uint8_t* packed_min, uint8_t* scales_min, int32_t scoring,
+    float route_scale, long long alt_token) {
+    if (blockIdx.x == 0) {
+        const RouteParams p{experts, topk, scoring, route_scale, alt_token};
+        tf_route_block(logits, bias, bias_alt, tokens, live, padding, ids, weights, owner_rows, p, 0,
+                       blockDim.x >> 6, true);
+    }
+    tf_frontend_run(input, ids, weights, packed, scales, packed_min, scales_min, token_map, token_weights, task_expert,
+                    task_valid_rows, expert_tile_base, rows, topk, experts, cols, groups, tile_m, act_block, 1);
+}
+// Row quantizer alone (any number of rows).
+extern "C" __global__ void __launch_bounds__(256) ca_quantize_rows(
+    const uint16_t* input, uint8_t* packed, uint8_t* scales, uint8_t* packed_min, uint8_t* scales_min, long long rows,
+    int32_t cols, int32_t act_block) {
+    tf_quantize_span(input, packed, scales, packed_min, scales_min, rows * (cols >> 3), act_block,
+                     (long long)blockIdx.x * blockDim.x + threadIdx.x, (long long)gridDim.x * blockDim.x);
+}
+
+// ---- Wide plan (any number of routes): three kernels, no atomics, same tables as the one-block plan. ----------------
+// 1. One wave per 64 consecutive routes: each route's rank among the wave's earlier routes of its expert, and the wave's
+//    per-expert counts.
+extern "C" __global__ void __launch_bounds__(256) ca_plan_wave_counts(
+    const int32_t* ids, int32_t pairs, int32_t experts, int32_t* wave_counts, int32_t* local_rank) {
+    __shared__ int32_t s_count[4][512];
+    const int lane = threadIdx.x & 63, w = threadIdx.x >> 6;
+    const int wave = blockIdx.x * 4 + w, p = wave * 64 + lane;
+    if (wave * 64 >= pairs) return;
+    for (int e = lane; e < experts; e += 64) s_count[w][e] = 0;
+    int id = p < pairs ? ids[p] : -1;
+    if (id >= experts) id = -1;
+    unsigned long long todo = __ballot(id >= 0);
+    int rank = 0;
+    while (todo) {
+        const int leader = __ffsll((long long)todo) - 1;
+        const int which = __shfl(id, leader);
+        const unsigned long long same = __ballot(id == which);
+        if (id == which) rank = __popcll(same & ((1ull << lane) - 1ull));
+        if (lane == leader) s_count[w][which] = __popcll(same);
+        todo &= ~same;
+    }
+    if (p < pairs) local_rank[p] = rank;
+    __builtin_amdgcn_wave_barrier();
+    for (int e = lane; e < experts; e += 64) wave_counts[(size_t)wave * experts + e] = s_count[w][e];
+}
+// 2. One block, one thread per expert: exclusive prefix of the wave counts (in place), tiles, tile bases, task tables.
+extern "C" __global__ void __launch_bounds__(512) ca_plan_scan(
+    int32_t* wave_counts, int32_t waves, int32_t experts, int32_t groups, int32_t tile_m, int32_t* expert_tile_base,
+    int32_t* task_expert, int32_t* task_valid_rows) {
+    __shared__ int32_t s_wave[8];
+    const int t = threadIdx.x, lane = t & 63, wave = t >> 6;
+    int count = 0;
+    if (t < experts)
+        for (int w = 0; w < waves; ++w) {
+            const int c = wave_counts[(size_t)w * experts + t];
+            wave_counts[(size_t)w * experts + t] = count;
+            count += c;
+        }
+    const int tiles = (count + tile_m - 1) / tile_m;
+    int prefix = tiles;
+#pragma unroll
+    for (int o = 1; o < 64; o <<= 1) {
+        const int below = __shfl_up(prefix, o);
+        if (lane >= o) prefix += below;
+    }
+    if (lane == 63) s_wave[wave] = prefix;
+    __syncthreads();
+    int base = prefix - tiles;
+    for (int w = 0; w < wave; ++w) base += s_wave[w];
+    if (t <= experts) expert_tile_base[t] = base;
+    if (t < experts)
+        for (int k = 0; k < tiles; ++k) {
+            const int valid = min(tile_m, count - k * tile_m);
+            for (int g = 0; g < groups; ++g) {
+                task_expert[(base + k) * groups + g] = t;
+                task_valid_rows[(base + k) * groups + g] = valid;
+            }
+        }
+}
+// 3. Every route: physical row from the expert's tile base and the route's rank.
+extern "C" __global__ void __launch_bounds__(256) ca_plan_scatter(
+    const int32_t* ids, const float* weights, const int32_t* wave_counts, const int32_t* local_rank,
+    const int32_t* expert_tile_base, int32_t pairs, int32_t experts, int32_t tile_m, int32_t* token_map,
+    float* token_weights) {
+    const int p = blockIdx.x * blockDim.x + threadIdx.x;
+    if (p >= pairs) return;
+    const int e = ids[p];
+    if (e < 0 || e >= experts) return;
+    const int rank = wave_counts[(size_t)(p >> 6) * experts + e] + local_rank[p];
+    const int row = (expert_tile_base[e] + rank / tile_m) * tile_m + rank % tile_m;
+    token_map[row] = p;
+    token_weights[row] = weights[p];
+}

@@ -1,0 +1,170 @@
+// Router: gate product for few rows, top-k with renormalised weights, padding routes, census.
+// Reference semantics: src/ffn.rs:330-413 (Router::run_routed), kernels/moe_frontend.cuh:85-157 (top-k),
+// kernels/core.cu:1093-1097 (padding rows), kernels/core.cu:161-166 (census).
+#pragma once
+#include "common.cuh"
+
+// logits[m][e] = sum_k x[m][k] * w[e][k], BF16 inputs, FP32 accumulate.  One wave per expert, up to 16 rows.
+// Fixed summation order: lane l accumulates the 8-element vectors at k = 512 j + 8 l (j ascending) with fma in k order,
+// then the 64 partials are combined by the xor butterfly 32, 16, 8, 4, 2, 1.  hidden % 512 == 0.
+extern "C" __global__ void __launch_bounds__(64) ca_router_logits_rows(
+    const uint16_t* __restrict__ x, const uint16_t* __restrict__ w, float* __restrict__ out, int rows, int hidden,
+    int experts) {
+    const int e = blockIdx.x, lane = threadIdx.x;
+    if (e >= experts) return;
+    float acc[16];
+#pragma unroll
+    for (int m = 0; m < 16; ++m) acc[m] = 0.f;
+    const u4v* wrow = reinterpret_cast<const u4v*>(w + (size_t)e * hidden);
+    for (int j = 0; j < hidden / 512; ++j) {
+        const u4v wv = wrow[j * 64 + lane];
+#pragma unroll
+        for (int m = 0; m < 16; ++m) {
+            if (m < rows) {
+                const u4v xv = reinterpret_cast<const u4v*>(x + (size_t)m * hidden)[j * 64 + lane];
+#pragma unroll
+                for (int i = 0; i < 4; ++i) {
+                    acc[m] = __fmaf_rn(tf_bf16_lo(xv[i]), tf_bf16_lo(wv[i]), acc[m]);
+                    acc[m] = __fmaf_rn(tf_bf16_hi(xv[i]), tf_bf16_hi(wv[i]), acc[m]);
+                }
+            }
+        }
+    }
+#pragma unroll
+    for (int m = 0; m < 16; ++m) {
+        if (m < rows) {
+            float v = acc[m];
+#pragma unroll
+            for (int o = 32; o > 0; o >>= 1) v = __fadd_rn(v, __shfl_xor(v, o));
+            if (lane == 0) out[(size_t)m * experts + e] = v;
+        }
+    }
+}
+
+struct RouteParams {
+    int experts, topk, scoring;   // scoring: 0 sigmoid, 1 sqrt(softplus)
+    float route_scale;
+    long long alt_token;          // token id that selects bias_alt, -1: none
+};
+
+// One wave routes one row.  Lane l holds experts l, l + 64, ... (at most 8 per lane: experts <= 512).  Every lane
+// returns the same ids / weights in registers [k]; topk <= 8.
+__device__ __forceinline__ void tf_route_row(const float* logits, const float* bias, int lane, const RouteParams& p,
+                                             int32_t* out_ids, float* out_weights) {
+    float score[8], biased[8];
+#pragma unroll
+    for (int i = 0; i < 8; ++i) {
+        const int e = i * 64 + lane;
+        score[i] = 0.f;
+        biased[i] = -INFINITY;
+        if (e < p.experts) {
+            const float x = logits[e];
+            float s;
+            if (p.scoring == 1) s = __builtin_sqrtf(x > 20.f ? x : tf_log1p_pos(tf_exp(x)));
+            else s = tf_logistic(x);
+            const float v = __fadd_rn(s, bias[e]);
+            score[i] = s;
+            biased[i] = (v == v) ? v : INFINITY;
+        }
+    }
+    float w[8];
+#pragma unroll
+    for (int k = 0; k < 8; ++k) {
+        w[k] = 0.f;
+        if (k < p.topk) {
+            float best = -INFINITY;
+#pragma unroll
+            for (int i = 0; i < 8; ++i) best = fmaxf(best, biased[i]);
+            best = tf_wave_max(best);
+            int32_t winner = 0x7fffffff;
+#pragma unroll
+            for (int i = 0; i < 8; ++i)
+                if (i * 64 + lane < p.experts && biased[i] == best) winner = min(winner, i * 64 + lane);
+#pragma unroll
+            for (int o = 32; o > 0; o >>= 1) winner = min(winner, __shfl_xor(winner, o));
+            float mine = 0.f;
+#pragma unroll
+            for (int i = 0; i < 8; ++i)
+                if (i * 64 + lane == winner) { mine = score[i]; biased[i] = -INFINITY; }
+            w[k] = __shfl(mine, winner & 63);
+            out_ids[k] = winner;
+        }
+    }
+    float total;
+    if (p.topk == 6) {
+        total = __fadd_rn(__fadd_rn(__fadd_rn(w[3], __fadd_rn(w[2], __fadd_rn(w[0], w[1]))), __fadd_rn(w[4], w[5])), 1e-20f);
+    } else {
+        total = w[0];
+#pragma unroll
+        for (int k = 1; k < 8; ++k) if (k < p.topk) total = __fadd_rn(total, w[k]);
+        total = __fadd_rn(total, 1e-20f);
+    }
+#pragma unroll
+    for (int k = 0; k < 8; ++k) if (k < p.topk) out_weights[k] = __fmul_rn(w[k] / total, p.route_scale);
+}
+
+// Routes rows [first_row, first_row + waves of this block) of `rows`; rows at or past min(rows, live[0]) get ids -1 and
+// weights 0.  `padding` (may be null) is applied only by a single-block launch, after a block barrier.
+__device__ __forceinline__ void tf_route_block(const float* logits, const float* bias, const float* bias_alt,
+                                               const long long* tokens, const int32_t* live, const int32_t* padding,
+                                               int32_t* ids, float* weights, int rows, const RouteParams& p,
+                                               int first_row, int row_stride, bool apply_padding) {
+    const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+    const int n_live = min(rows, live[0]);
+    for (int row = first_row + wave; row < rows; row += row_stride) {
+        const bool is_live = row < n_live;
+        int32_t chosen[8];
+        float share[8];
+        if (is_live) {
+            const bool alt = bias_alt != nullptr && tokens != nullptr && p.alt_token >= 0 && tokens[row] == p.alt_token;
+            tf_route_row(logits + (size_t)row * p.experts, alt ? bias_alt : bias, lane, p, chosen, share);
+        }
+#pragma unroll
+        for (int k = 0; k < 8; ++k)
+            if (k < p.topk && lane == k) {
+                ids[row * p.topk + k] = is_live ? chosen[k] : -1;
+                weights[row * p.topk + k] = is_live ? share[k] : 0.f;
+            }
+    }
+    if (apply_padding) {
+        __threadfence_block();
+        __syncthreads();
+        if (padding != nullptr)
+            for (int i = threadIdx.x; i < rows * p.topk; i += blockDim.x) {
+                const int r = i / p.topk, s = padding[r];
+                if (s >= 0) { ids[i] = ids[s * p.topk + (i - r * p.topk)]; weights[i] = 0.f; }
+            }
+        __syncthreads();
+    }
+}
+
+// The router's top-k alone.  One block: routes every row and applies `padding`.  Several blocks: each block routes its
+// waves' rows; the caller passes padding = null and launches ca_route_padding_rows afterwards.
+extern "C" __global__ void ca_route_topk(const float* logits, const float* bias, const float* bias_alt,
+                                         const long long* tokens, const int32_t* live, const int32_t* padding,
+                                         int32_t* ids, float* weights, int32_t rows, int32_t experts, int32_t topk,
+                                         int32_t scoring, float route_scale, long long alt_token) {
+    const RouteParams p{experts, topk, scoring, route_scale, alt_token};
+    const int waves = blockDim.x >> 6;
+    tf_route_block(logits, bias, bias_alt, tokens, live, padding, ids, weights, rows, p, blockIdx.x * waves,
+                   gridDim.x * waves, gridDim.x == 1);
+}
+
+// Padding rows of a batched step take their source row's experts with zero weights.
+extern "C" __global__ void ca_route_padding_rows(int32_t* ids, float* weights, const int32_t* source, int rows, int topk) {
+    const int i = blockIdx.x * blockDim.x + threadIdx.x;
+    if (i >= rows * topk) return;
+    const int r = i / topk, s = source[r];
+    if (s < 0) return;
+    ids[i] = ids[s * topk + (i - r * topk)];
+    weights[i] = 0.f;
+}
+
+// Diagnostic histogram of the routed slots of live rows.
+extern "C" __global__ void ca_route_census(const int32_t* ids, const int32_t* live, int rows, int topk,
+                                           uint32_t* counters, int experts) {
+    const int i = blockIdx.x * blockDim.x + threadIdx.x;
+    if (i >= rows * topk || i / topk >= live[0]) return;
+    const int e = ids[i];
+    if (e >= 0 && e < experts) atomicAdd(counters + e, 1u);
+}

@@ -1,0 +1,111 @@
+"""ctypes binding of the C ABI in include/titanic_moe.h (libtitanic_moe_hip.so).
+
+The product path has no fallback: if the library is missing the import fails with the build command to run.
+"""
+import ctypes
+import os
+
+HERE = os.path.dirname(os.path.abspath(__file__))
+KERNEL_LIB = os.path.join(HERE, "libtitanic_moe_hip.so")
+CODE_OBJECT = os.path.join(HERE, "titanic_moe_gfx950.hsaco")
+
+EXPORTS = ["ca_ffn_abi", "ca_ffn_configure", "ca_ffn_geometry", "ca_router_logits", "ca_shared_swiglu", "ca_ffn_add",
+           "ca_router_logits_wide", "ca_kernel_launch", "ca_kernel_count", "ca_kernel_name", "ca_moe_nibble_permute",
+           "ca_primitives_abi", "ca_primitives_open", "ca_primitives_close", "ca_primitives_launch", "ca_primitives_launch2",
+           "ca_primitives_entries", "ca_primitives_scratch_bytes"]
+
+
+class Geometry(ctypes.Structure):
+    _fields_ = [("hidden", ctypes.c_int32), ("experts", ctypes.c_int32), ("topk", ctypes.c_int32),
+                ("intermediate", ctypes.c_int32), ("shared_intermediate", ctypes.c_int32), ("scoring", ctypes.c_int32),
+                ("route_scale", ctypes.c_float), ("act_block", ctypes.c_int32), ("shared_bn", ctypes.c_int32),
+                ("shared_bk", ctypes.c_int32), ("alt_token", ctypes.c_int64), ("swiglu_limit", ctypes.c_float)]
+
+
+_lib = None
+
+
+def load():
+    global _lib
+    if _lib is not None:
+        return _lib
+    if not os.path.exists(KERNEL_LIB):
+        raise ImportError("%s is not built: run `python -c \"import __graft_entry__ as g; g.build()\"` at the repository root"
+                          % KERNEL_LIB)
+    lib = ctypes.CDLL(KERNEL_LIB)
+    vp, i32, u64p, i32p = ctypes.c_void_p, ctypes.c_int32, ctypes.POINTER(ctypes.c_uint64), ctypes.POINTER(ctypes.c_int32)
+    lib.ca_ffn_abi.restype = ctypes.c_int
+    lib.ca_ffn_configure.argtypes = [ctypes.POINTER(Geometry)]
+    lib.ca_ffn_geometry.argtypes = [ctypes.POINTER(Geometry)]
+    lib.ca_router_logits.argtypes = [ctypes.c_int, vp, vp, vp, vp]
+    lib.ca_router_logits_wide.argtypes = [ctypes.c_int, vp, vp, vp, vp]
+    lib.ca_shared_swiglu.argtypes = [ctypes.c_int, vp, vp, vp]
+    lib.ca_ffn_add.argtypes = [ctypes.c_int, vp, vp, vp, vp]
+    lib.ca_kernel_launch.argtypes = [ctypes.c_char_p, ctypes.POINTER(ctypes.c_uint32), ctypes.POINTER(ctypes.c_uint32),
+                                     ctypes.c_uint32, ctypes.POINTER(ctypes.c_void_p), vp]
+    lib.ca_kernel_name.restype = ctypes.c_char_p
+    lib.ca_kernel_name.argtypes = [ctypes.c_int]
+    lib.ca_moe_nibble_permute.argtypes = [vp, ctypes.c_uint64, ctypes.c_int, vp]
+    lib.ca_primitives_abi.restype = i32
+    lib.ca_primitives_open.restype = vp
+    lib.ca_primitives_open.argtypes = [i32p]
+    lib.ca_primitives_close.argtypes = [vp]
+    lib.ca_primitives_close.restype = None
+    lib.ca_primitives_launch.restype = i32
+    lib.ca_primitives_launch.argtypes = [vp, i32, u64p, ctypes.c_size_t, i32p, ctypes.c_size_t, vp]
+    lib.ca_primitives_launch2.restype = i32
+    lib.ca_primitives_launch2.argtypes = [vp, i32, u64p, ctypes.c_size_t, vp]
+    lib.ca_primitives_entries.restype = i32
+    lib.ca_primitives_scratch_bytes.restype = ctypes.c_int64
+    lib.ca_primitives_scratch_bytes.argtypes = [vp, i32, i32]
+    _lib = lib
+    return lib
+
+
+def kernel_names():
+    lib = load()
+    return [lib.ca_kernel_name(i).decode() for i in range(lib.ca_kernel_count())]
+
+
+class _Arg:
+    """One kernel argument kept alive for the duration of a launch."""
+
+    def __init__(self, value):
+        if isinstance(value, ctypes._SimpleCData):
+            self.c = value
+        elif isinstance(value, float):
+            self.c = ctypes.c_float(value)
+        elif isinstance(value, int):
+            self.c = ctypes.c_int32(value)
+        elif value is None:
+            self.c = ctypes.c_void_p(0)
+        else:  # torch tensor
+            self.c = ctypes.c_void_p(value.data_ptr())
+
+
+def ptr(t):
+    """Device pointer argument (None -> null)."""
+    return ctypes.c_void_p(0 if t is None else t.data_ptr())
+
+
+def launch(name, grid, block, args, stream=0, shared=0):
+    """ca_kernel_launch with python values: tensors and ptr() are pointers, ints are int32, floats float32; use ctypes
+    values (c_int64 ...) for anything else."""
+    lib = load()
+    if isinstance(grid, int):
+        grid = (grid, 1, 1)
+    if isinstance(block, int):
+        block = (block, 1, 1)
+    keep = [_Arg(a) for a in args]
+    argv = (ctypes.c_void_p * len(keep))(*[ctypes.cast(ctypes.pointer(k.c), ctypes.c_void_p) for k in keep])
+    status = lib.ca_kernel_launch(name.encode(), (ctypes.c_uint32 * 3)(*grid), (ctypes.c_uint32 * 3)(*block), shared, argv,
+                                  ctypes.c_void_p(stream))
+    if status != 0:
+        raise RuntimeError("ca_kernel_launch(%s) failed: %d" % (name, status))
+
+
+def primitives_launch(ctx, index, pointers, scalars, stream=0):
+    lib = load()
+    p = (ctypes.c_uint64 * len(pointers))(*[0 if t is None else (t if isinstance(t, int) else t.data_ptr()) for t in pointers])
+    s = (ctypes.c_int32 * len(scalars))(*scalars)
+    return lib.ca_primitives_launch(ctypes.c_void_p(ctx), index, p, len(pointers), s, len(scalars), ctypes.c_void_p(stream))
