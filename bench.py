@@ -1,0 +1,182 @@
+#!/usr/bin/env python3
+"""Benchmark of the MoE FFN layer on one MI355X.
+
+    python bench.py [--gpus 1] [--steps K] [--warmup W] [--config c2|c3]
+
+A step is one pass of the whole layer (gate product, top-k + plan + token quantization, routed FC1 + SwiGLU, FC2, shared
+expert, ordered sum + shared addition) over one batch of synthetic token rows that is already resident in HBM, replayed
+as a captured HIP graph as the reference replays its layer (src/probe.rs:1527-1542).  Sixteen distinct input batches
+are cycled so every step routes to other experts and streams their weights from HBM, not from the last step's cache.
+
+Prints one JSON line: whole-layer tokens/s, the roofline of the dominant kernel (routed FC1 + SwiGLU; algorithmic bytes
+over its average duration, measured with HIP events on its launch stream), and the CPU baseline (the C oracle, a port
+of the reference semantics: the reference has no CPU path) timed on a bounded sample of the same workload.
+"""
+import argparse
+import importlib
+import json
+import os
+import sys
+import time
+
+ROOT = os.path.dirname(os.path.abspath(__file__))
+sys.path.insert(0, ROOT)
+
+HBM_PEAK_GBS = 8000.0
+BATCHES = 16
+
+CONFIGS = {
+    "c2": dict(rows=4, hidden=4096, experts=256, topk=6, inter=2048, shared=2048,
+               workload="decode step, 4 requests x 1 token; H 4096, E 256, top-6, I 2048, 1 shared expert (I 2048)"),
+    "c3": dict(rows=32, hidden=4096, experts=256, topk=6, inter=2048, shared=2048,
+               workload="speculative verify, 4 requests x 8 draft tokens = 32 rows; H 4096, E 256, top-6, I 2048, 1 shared expert"),
+}
+
+
+def make_inputs(synth, name, cfg, device):
+    import torch
+    xs = []
+    for step in range(BATCHES):
+        if name == "c3":   # tokens of a request share a base vector: correlated router logits
+            base = synth.normal("c3/base.%d" % step, (4, 1, cfg["hidden"]), device=device)
+            noise = synth.normal("c3/noise.%d" % step, (4, 8, cfg["hidden"]), std=0.3, device=device)
+            xs.append(synth.to_bf16_bits((base + noise).reshape(32, cfg["hidden"])).contiguous())
+        else:
+            xs.append(synth.activations(name, cfg["rows"], cfg["hidden"], device=device, step=step).contiguous())
+    torch.cuda.synchronize()
+    return xs
+
+
+def cpu_baseline(pkg, g, ops, xs, taps_ids, budget_s=20.0):
+    """Times the C oracle (staged, active experts only) on host cores for a bounded number of steps."""
+    sys.path.insert(0, os.path.join(ROOT, "tests"))
+    import oracle
+    import helpers
+    threads = len(os.sched_getaffinity(0)) if hasattr(os, "sched_getaffinity") else (os.cpu_count() or 1)
+    threads = max(1, min(threads, 16))
+    oracle.set_threads(threads)
+    rows = xs[0].shape[0]
+    done, spent = 0, 0.0
+    while done < len(xs) and (done == 0 or spent + spent / done < budget_s):
+        x = xs[done]
+        # gather the operands the step touches outside the timed region (the oracle reads host memory)
+        small_ops = _HostSubset(ops, taps_ids[done], g)
+        t0 = time.perf_counter()
+        helpers.oracle_layer(g, small_ops, x.cpu())
+        spent += time.perf_counter() - t0
+        done += 1
+    return {"value": rows * done / spent, "unit": "tokens/s", "cores": threads, "kind": "port",
+            "sample": "%d steps of this workload (%d rows each), C oracle with %d OpenMP threads, %.1f s" % (done, rows, threads, spent)}
+
+
+class _HostSubset:
+    """Host copies of the operands one step reads: the step's active experts (others stay zero) and the dense parts."""
+
+    def __init__(self, ops, ids, g):
+        import torch
+        active = sorted(set(int(e) for e in ids.ravel() if e >= 0))
+        pick = torch.as_tensor(active, dtype=torch.long, device=ops.w13.device)
+        self.active = active
+        for name in ["gate_w", "bias", "bias_alt", "sh_w13", "sh_s13", "sh_w2", "sh_s2"]:
+            setattr(self, name, getattr(ops, name).cpu())
+        for name in ["w13", "s13", "w2", "s2"]:
+            full = getattr(ops, name)
+            setattr(self, name, _Sparse(full, pick, active))
+
+
+class _Sparse:
+    """Expert-major tensor of which only some experts are held on the host; indexing with a tensor of expert ids returns them."""
+
+    def __init__(self, full, pick, active):
+        self.data = full[pick].cpu()
+        self.index = {e: i for i, e in enumerate(active)}
+        self.device = self.data.device
+
+    def __getitem__(self, ids):
+        import torch
+        return self.data[torch.as_tensor([self.index[int(e)] for e in ids], dtype=torch.long)]
+
+
+def main():
+    ap = argparse.ArgumentParser()
+    ap.add_argument("--gpus", type=int, default=1)
+    ap.add_argument("--steps", type=int, default=2000)
+    ap.add_argument("--warmup", type=int, default=200)
+    ap.add_argument("--config", default="c2", choices=sorted(CONFIGS))
+    ap.add_argument("--no-cpu-baseline", action="store_true")
+    ap.add_argument("--profile-steps", type=int, default=64, help="eager passes with per-kernel HIP events for the roofline")
+    args = ap.parse_args()
+    if args.gpus != 1:
+        print("bench.py measures one GPU: the layer runs on a single MI355X (no sharding, no collectives); --gpus %d is not supported" % args.gpus,
+              file=sys.stderr)
+        sys.exit(2)
+    import numpy as np
+    import torch
+    pkg = importlib.import_module("titanic-flash-41_amd")
+    native, synth, host = pkg.native, pkg.synth, pkg.host
+    cfg = CONFIGS[args.config]
+    g = native.Geometry(cfg["hidden"], cfg["experts"], cfg["topk"], cfg["inter"], cfg["shared"], 0, 1.0, 128, 128, 128, -1, 10.0)
+    torch.cuda.set_device(0)
+    t0 = time.time()
+    ops = synth.LayerOperands(g, args.config, device="cuda")
+    xs = make_inputs(synth, args.config, cfg, "cuda")
+    layer = host.Layer(g, ops, cfg["rows"])
+    layer.set_tokens()
+    setup_s = time.time() - t0
+
+    # per-kernel durations (HIP events on the launch stream) and the routing of every batch
+    ids_per_batch, parts = [], np.zeros(7)
+    tiles_per_batch = []
+    for x in xs:                      # warm every batch once
+        layer.profile_step(x)
+    passes = 0
+    for i in range(args.profile_steps):
+        x = xs[i % BATCHES]
+        parts += np.array(layer.profile_step(x))
+        passes += 1
+        if i < BATCHES:
+            ids_per_batch.append(layer.tap("ids").reshape(cfg["rows"], cfg["topk"]).copy())
+            tiles_per_batch.append(int(layer.tap("tile_base")[-1]))
+    parts /= passes
+    H, I, S, E, K, rows = cfg["hidden"], cfg["inter"], cfg["shared"], cfg["experts"], cfg["topk"], cfg["rows"]
+    distinct = float(np.mean([len(set(ids.ravel().tolist())) for ids in ids_per_batch]))
+    tiles = float(np.mean(tiles_per_batch))
+    # algorithmic bytes: every streamed tile of FC1 reads one expert's up + gate weights and scales once
+    fc1_bytes = tiles * (2 * I * H // 2 + 2 * I * H // 32) + rows * (H + H // 128) + rows * K * I * 2
+    fc2_bytes = tiles * (H * I // 2 + H * I // 32) + rows * K * I * 2 + rows * K * H * 2
+    shared_bytes = 3 * H * S + rows * (H + 2 * S * 2 + S * 2 + H * 2)
+    router_bytes = 2 * E * H + rows * H * 2
+    step_bytes = fc1_bytes + fc2_bytes + shared_bytes + router_bytes + rows * (K + 2) * H * 2
+    fc1_ms = float(parts[2])
+    achieved = fc1_bytes / (fc1_ms * 1e-3) / 1e9
+
+    # whole-layer throughput: graph replays cycling the batches
+    graphs = [layer.capture(x) for x in xs]
+    torch.cuda.synchronize()
+    ms = layer.time(graphs, args.warmup, args.steps)
+    torch.cuda.synchronize()
+    ms_per_step = ms / args.steps
+    value = rows / (ms_per_step * 1e-3)
+
+    line = {
+        "metric": "MoE-layer tokens/s", "value": value, "unit": "tokens/s", "n_gpus": 1, "steps": args.steps, "warmup": args.warmup,
+        "ms_per_step": ms_per_step, "higher_is_better": True, "scaling": "weak", "vs_baseline": None,
+        "dtype": "fp4 (e2m1 weights, ue8m0 scales) x fp8 (e4m3 activations), f32 accumulate",
+        "data": "synthetic", "config": {"workload": args.config + ": " + cfg["workload"], "numerics": "sigmoid top-k renormalised, 128-wide activation blocks",
+                                        "input_batches": BATCHES, "distinct_experts_per_step": distinct, "schedule": "HIP graph replay, shared expert on a second stream"},
+        "roofline": {"bound": "hbm", "kernel": "tf_fc1_stream<fp4> (routed FC1 + SwiGLU)", "achieved": achieved, "peak": HBM_PEAK_GBS, "unit": "GB/s",
+                     "frac": achieved / HBM_PEAK_GBS, "traffic": None, "bytes_per_launch": fc1_bytes, "avg_launch_ms": fc1_ms},
+        "step_bytes": step_bytes, "step_gbs": step_bytes / (ms_per_step * 1e-3) / 1e9, "step_hbm_frac": step_bytes / (ms_per_step * 1e-3) / 1e9 / HBM_PEAK_GBS,
+        "kernel_ms": {"router": float(parts[0]), "front_end": float(parts[1]), "fc1_swiglu": fc1_ms, "fc2": float(parts[3]),
+                      "shared_expert": float(parts[4]), "sum_shared": float(parts[5]), "eager_pass": float(parts[6])},
+        "kernel_gbs": {"fc2": fc2_bytes / (float(parts[3]) * 1e-3) / 1e9, "shared_expert": shared_bytes / (float(parts[4]) * 1e-3) / 1e9},
+        "setup_s": setup_s,
+    }
+    if not args.no_cpu_baseline:
+        line["cpu_baseline"] = cpu_baseline(pkg, g, ops, xs, ids_per_batch)
+    layer.close()
+    print(json.dumps(line))
+
+
+if __name__ == "__main__":
+    main()

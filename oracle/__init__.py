@@ -56,6 +56,10 @@ def lib():
     return _lib
 
 
+def set_threads(n):
+    lib().orc_set_threads(_i32(n))
+
+
 def config(hidden, experts, topk, inter, shared_inter, scoring=0, route_scale=1.0, act_block=128, shared_bn=128,
            shared_bk=128, alt_token=-1, swiglu_limit=10.0):
     return Config(hidden, experts, topk, inter, shared_inter, scoring, route_scale, act_block, shared_bn, shared_bk,

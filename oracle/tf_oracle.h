@@ -35,6 +35,8 @@ typedef struct {
     float swiglu_limit;    /* 10 */
 } orc_config;
 
+void orc_set_threads(int32_t n);
+
 /* ---- number formats ------------------------------------------------------------------------- */
 float orc_bf16_to_f32(uint16_t v);
 uint16_t orc_f32_to_bf16(float v);

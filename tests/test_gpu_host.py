@@ -1,0 +1,69 @@
+"""GPU parity of the C++ host mirror (LayerFfn / Router / Workspace / prepare_layer over the C ABI) against the CPU oracle,
+in every schedule the reference has (dual-stream shared branch, fused or separate sum, top-k inside or before the
+front-end), eager and as a replayed graph."""
+import numpy as np
+import pytest
+import torch
+
+import oracle
+from helpers import pkg, synth
+from test_gpu_layer import check_layer, make
+
+pytestmark = pytest.mark.gpu
+host = pkg.host
+
+
+@pytest.mark.parametrize("overlap,sum_shared,route_front", [(True, True, True), (False, False, False), (False, True, True), (True, False, False)])
+def test_c1_schedules(overlap, sum_shared, route_front):
+    g, ops, x, rows = make("c1", "benchmark", "cpu")
+    layer = host.Layer(g, ops, rows, overlap=overlap, sum_shared=sum_shared, route_front=route_front)
+    layer.set_tokens()
+    layer.run(x.cuda())
+    taps = layer.taps()
+    if overlap:   # the branch quantized the input itself; the routed front-end emitted no shared-flavour codes
+        taps["xq_min"], taps["xs_min"] = oracle.quantize_rows(x.numpy().view(np.uint16), g.act_block, 1e-4)
+    check_layer(g, ops, x, taps)
+    layer.close()
+
+
+def test_reference_mode_tokens_live_padding_and_errors():
+    g, ops, x, rows = make("c1", "reference", "cpu")
+    layer = host.Layer(g, ops, rows, overlap=False)
+    tokens = [5, 129264, 7, 129264, 1, 2, 3, 4]
+    padding = [-1, -1, -1, -1, 0, 2, -1, -1]
+    layer.set_tokens(tokens, live=4, padding=padding)
+    layer.run(x.cuda())
+    check_layer(g, ops, x, layer.taps(), tokens=tokens, live=4, padding=np.array(padding, np.int32), max_rel=2e-2)
+    assert layer.census().sum() == 4 * g.topk
+    with pytest.raises(host.HostError, match="padding route sources must name live rows"):
+        layer.set_tokens(tokens, live=4, padding=[-1, -1, -1, -1, 6, -1, -1, -1])
+    with pytest.raises(host.HostError, match="router token metadata domain"):
+        layer.set_tokens([129280] * 8)
+    layer.close()
+
+
+def test_scale_code_and_prepared_layout_report():
+    g, ops, x, rows = make("c1", "benchmark", "cpu")
+    layer = host.Layer(g, ops, rows, code_scales=True)
+    info = layer.info()
+    E, H, I = g.experts, g.hidden, g.intermediate
+    assert info["expert_bytes"] == E * (3 * H * I // 2 + 3 * H * I // 32)
+    assert info["scale_code_bytes"] == oracle.scale_code1_layout(E, H, I)[5] * 4
+    assert info["coded_rows"] == E * (2 * (I // 128) * (H // 128) + (H // 128) * (I // 128)) * 128 and info["raw_rows"] < info["coded_rows"]
+    layer.close()
+
+
+@pytest.mark.parametrize("config", ["c2", "c3"])
+def test_graph_replay_matches_eager_and_oracle(config):
+    g, ops, x, rows = make(config, "benchmark", "cuda")
+    layer = host.Layer(g, ops, rows)
+    layer.set_tokens()
+    xs = [x, synth.activations(config + "/second", rows, g.hidden, device="cuda")]
+    graphs = [layer.capture(t) for t in xs]
+    for which in (0, 1, 0):       # replays with other work between them must not see stale scratch
+        layer.time([graphs[which]], 0, 1)
+        taps = layer.taps()
+        taps["xq_min"], taps["xs_min"] = oracle.quantize_rows(xs[which].cpu().numpy().view(np.uint16), g.act_block, 1e-4)
+        check_layer(g, ops, xs[which], taps)
+        layer.run(xs[1 - which])
+    layer.close()

@@ -65,7 +65,8 @@ enum DynPtr {
 };
 enum DynScalar { S_TOKENS, S_MAX_ROWS, S_ROWS_PADDED, S_MAX_TILES, S_TILE_M, S_GROUPS, S_DYN_COUNT, S_OWNER_ROWS = S_DYN_COUNT, S_ROUTE_COUNT };
 
-int launch_dynamic(const Context& c, bool route, const uint64_t* p, const int32_t* sc, hipStream_t s) {
+// phases: 1 front-end (plan + quantize), 2 FC1 + SwiGLU, 4 FC2
+int launch_dynamic(const Context& c, bool route, const uint64_t* p, const int32_t* sc, hipStream_t s, int phases = 7) {
     const ca_geometry& g = c.g;
     const int rows = sc[S_TOKENS], tile_m = sc[S_TILE_M], groups = sc[S_GROUPS], max_tiles = sc[S_MAX_TILES];
     if (rows < 1 || rows > sc[S_MAX_ROWS] || groups < 1 || max_tiles < 1 || sc[S_ROWS_PADDED] != max_tiles * tile_m) return -1;
@@ -82,7 +83,8 @@ int launch_dynamic(const Context& c, bool route, const uint64_t* p, const int32_
     const uint16_t* x = (const uint16_t*)p[P_A];
     int32_t* ids = (int32_t*)p[P_IDS];
     float* weights = (float*)p[P_WEIGHTS];
-    if (pairs <= 1024 && g.experts < 1024) {
+    if (!(phases & 1)) {
+    } else if (pairs <= 1024 && g.experts < 1024) {
         const int quant_blocks = (int)((((long long)rows * (g.hidden >> 3)) + 1023) / 1024);
         if (route) {
             const int owner = sc[S_OWNER_ROWS];
@@ -133,8 +135,11 @@ int launch_dynamic(const Context& c, bool route, const uint64_t* p, const int32_
         a.experts = g.experts; a.groups = groups; a.topk = g.topk;
         a.k = g.hidden; a.inter = g.intermediate; a.hidden = g.hidden; a.act_block = g.act_block; a.limit = g.swiglu_limit;
         a.out = (uint16_t*)p[P_INTER];
-        status = launch_fc1_stream<false>(a, c.stream_wgs, s);
-        if (status) return status;
+        if (phases & 2) {
+            status = launch_fc1_stream<false>(a, c.stream_wgs, s);
+            if (status) return status;
+        }
+        if (!(phases & 4)) return 0;
         StreamArgs b = a;
         b.a_codes = nullptr; b.a_scales = nullptr; b.a_bf16 = (const uint16_t*)p[P_INTER];
         b.q_codes = (uint8_t*)p[P_INTER_CODES]; b.q_scales = (uint8_t*)p[P_INTER_SCALES]; b.min_amax = 0.f;
@@ -155,8 +160,11 @@ int launch_dynamic(const Context& c, bool route, const uint64_t* p, const int32_
     a.k = g.hidden; a.inter = g.intermediate; a.hidden = g.hidden; a.act_block = g.act_block; a.limit = g.swiglu_limit;
     a.h_bf16 = (uint16_t*)p[P_INTER]; a.h_codes = (uint8_t*)p[P_INTER_CODES]; a.h_scales = (uint8_t*)p[P_INTER_SCALES];
     a.out = (uint16_t*)p[P_SCATTER];
-    status = tf_launch_fc1_gemm(a, c.cus, s);
-    if (status) return status;
+    if (phases & 2) {
+        status = tf_launch_fc1_gemm(a, c.cus, s);
+        if (status) return status;
+    }
+    if (!(phases & 4)) return 0;
     GemmArgs b = a;
     b.a_codes = (const uint8_t*)p[P_INTER_CODES]; b.a_scales = (const uint8_t*)p[P_INTER_SCALES];
     b.w = (const uint8_t*)p[P_W2]; b.ws = (const uint8_t*)p[P_S2];
@@ -251,6 +259,9 @@ const EntryShape kEntries[] = {
     {"gemm.mxfp8_quant_cute", 5, 3},
     {"gemm.dense", 5, 3},
     {"ffn.shared_expert", H_COUNT, 1},
+    {"moe.w4a8.phase1", P_DYN_COUNT, S_DYN_COUNT},
+    {"moe.w4a8.phase2", P_DYN_COUNT, S_DYN_COUNT},
+    {"moe.front_end", P_DYN_COUNT, S_DYN_COUNT},
 };
 constexpr int kEntryCount = sizeof(kEntries) / sizeof(kEntries[0]);
 
@@ -364,6 +375,9 @@ int32_t ca_primitives_launch(void* context, int32_t index, const uint64_t* point
         case 3: return launch_quant(c, pointers, scalars, s);
         case 4: return launch_dense(c, pointers, scalars, s);
         case 5: return launch_shared(c, pointers, scalars, s);
+        case 6: return launch_dynamic(c, false, pointers, scalars, s, 2);
+        case 7: return launch_dynamic(c, false, pointers, scalars, s, 4);
+        case 8: return launch_dynamic(c, false, pointers, scalars, s, 1);
         default: return -3;
     }
 }

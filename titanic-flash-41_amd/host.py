@@ -1,0 +1,141 @@
+"""ctypes binding of libtitanic_ffn_host.so, the C++ host mirror of the reference's Rust FFN operators
+(LayerFfn / Router / Workspace / prepare_layer).  Inputs are torch tensors (device memory only); results are numpy."""
+import ctypes
+import os
+
+import numpy as np
+
+from . import native
+
+HERE = os.path.dirname(os.path.abspath(__file__))
+HOST_LIB = os.path.join(HERE, "libtitanic_ffn_host.so")
+_lib = None
+
+TAPS = {"logits": np.float32, "ids": np.int32, "weights": np.float32, "xq": np.uint8, "xs": np.uint8, "xq_min": np.uint8,
+        "xs_min": np.uint8, "h": np.uint16, "hq": np.uint8, "hs": np.uint8, "task_expert": np.int32, "task_valid": np.int32,
+        "tile_base": np.int32, "token_map": np.int32, "token_weights": np.float32, "route_out": np.uint16, "routed": np.uint16,
+        "shared_up": np.uint16, "shared_act": np.uint16, "shared_aq": np.uint8, "shared_as": np.uint8, "shared_down": np.uint16,
+        "out": np.uint16}
+
+
+def load():
+    global _lib
+    if _lib is None:
+        if not os.path.exists(HOST_LIB):
+            raise ImportError("%s is not built: run __graft_entry__.build()" % HOST_LIB)
+        lib = ctypes.CDLL(HOST_LIB)
+        vp, cp, sz = ctypes.c_void_p, ctypes.c_char_p, ctypes.c_size_t
+        lib.tfh_layer_create.restype = vp
+        lib.tfh_layer_create.argtypes = [cp, ctypes.POINTER(native.Geometry), ctypes.c_int, ctypes.POINTER(vp), ctypes.c_int, ctypes.c_int,
+                                         ctypes.c_int, ctypes.c_int, ctypes.c_int, cp, sz]
+        lib.tfh_layer_destroy.argtypes = [vp]
+        lib.tfh_layer_destroy.restype = None
+        lib.tfh_layer_set_tokens.argtypes = [vp, vp, ctypes.c_int, vp, cp, sz]
+        lib.tfh_layer_run.argtypes = [vp, ctypes.c_uint64, cp, sz]
+        lib.tfh_layer_capture.argtypes = [vp, ctypes.c_uint64, cp, sz]
+        lib.tfh_layer_time.argtypes = [vp, ctypes.POINTER(ctypes.c_int), ctypes.c_int, ctypes.c_int, ctypes.c_int, ctypes.POINTER(ctypes.c_float), cp, sz]
+        lib.tfh_layer_time_phase.argtypes = [vp, ctypes.c_int, ctypes.c_uint64, ctypes.c_int, ctypes.POINTER(ctypes.c_float), cp, sz]
+        lib.tfh_layer_profile_step.argtypes = [vp, ctypes.c_uint64, ctypes.POINTER(ctypes.c_float), cp, sz]
+        lib.tfh_layer_tap.restype = ctypes.c_longlong
+        lib.tfh_layer_tap.argtypes = [vp, cp, vp, sz, cp, sz]
+        lib.tfh_layer_census.argtypes = [vp, vp, cp, sz]
+        lib.tfh_layer_info.argtypes = [vp, ctypes.POINTER(ctypes.c_longlong)]
+        lib.tfh_layer_info.restype = None
+        _lib = lib
+    return _lib
+
+
+class HostError(RuntimeError):
+    pass
+
+
+class Layer:
+    """One LayerFfn + Workspace + TokenRows on cuda:0 for `rows` token rows."""
+
+    def __init__(self, geometry, operands, rows, overlap=True, sum_shared=True, route_front=True, code_scales=False):
+        self.lib = load()
+        native.load()
+        self.g, self.rows = geometry, rows
+        self._err = ctypes.create_string_buffer(512)
+        names = ["gate_w", "bias", "bias_alt", "w13", "s13", "w2", "s2", "sh_w13", "sh_s13", "sh_w2", "sh_s2"]
+        tensors = [getattr(operands, n).contiguous() for n in names]
+        on_device = tensors[0].is_cuda
+        assert all(t.is_cuda == on_device for t in tensors)
+        ptrs = (ctypes.c_void_p * 11)(*[t.data_ptr() for t in tensors])
+        if on_device:
+            import torch
+            torch.cuda.synchronize()
+        self.h = self.lib.tfh_layer_create(native.KERNEL_LIB.encode(), ctypes.byref(geometry), rows, ptrs, int(on_device), int(overlap),
+                                           int(sum_shared), int(route_front), int(code_scales), self._err, 512)
+        if not self.h:
+            raise HostError(self._err.value.decode())
+        self.h = ctypes.c_void_p(self.h)
+
+    def _check(self, status):
+        if status < 0:
+            raise HostError(self._err.value.decode())
+        return status
+
+    def close(self):
+        if self.h:
+            self.lib.tfh_layer_destroy(self.h)
+            self.h = None
+
+    def set_tokens(self, ids=None, live=None, padding=None):
+        ids = np.zeros(self.rows, np.int64) if ids is None else np.ascontiguousarray(ids, np.int64)
+        pad = None if padding is None else np.ascontiguousarray(padding, np.int32)
+        self._check(self.lib.tfh_layer_set_tokens(self.h, ids.ctypes.data, self.rows if live is None else live,
+                                                  None if pad is None else pad.ctypes.data, self._err, 512))
+
+    def run(self, x):
+        assert x.is_cuda and x.is_contiguous() and x.numel() == self.rows * self.g.hidden
+        self._check(self.lib.tfh_layer_run(self.h, x.data_ptr(), self._err, 512))
+
+    def capture(self, x):
+        assert x.is_cuda and x.is_contiguous()
+        return self._check(self.lib.tfh_layer_capture(self.h, x.data_ptr(), self._err, 512))
+
+    def time(self, order, warmup, steps):
+        ms = ctypes.c_float(0)
+        arr = (ctypes.c_int * len(order))(*order)
+        self._check(self.lib.tfh_layer_time(self.h, arr, len(order), warmup, steps, ctypes.byref(ms), self._err, 512))
+        return ms.value
+
+    def time_phase(self, entry, x, iterations):
+        ms = ctypes.c_float(0)
+        self._check(self.lib.tfh_layer_time_phase(self.h, entry, x.data_ptr(), iterations, ctypes.byref(ms), self._err, 512))
+        return ms.value
+
+    def profile_step(self, x):
+        """Milliseconds of (router, front-end, FC1, FC2, shared expert, sum, whole pass) of one eager pass."""
+        ms = (ctypes.c_float * 7)()
+        self._check(self.lib.tfh_layer_profile_step(self.h, x.data_ptr(), ms, self._err, 512))
+        return list(ms)
+
+    def tap(self, name):
+        size = self._check(self.lib.tfh_layer_tap(self.h, name.encode(), None, 0, self._err, 512))
+        out = np.empty(size // np.dtype(TAPS[name]).itemsize, TAPS[name])
+        self._check(self.lib.tfh_layer_tap(self.h, name.encode(), out.ctypes.data, size, self._err, 512))
+        return out
+
+    def taps(self):
+        g, rows = self.g, self.rows
+        K, H, I, S, B = g.topk, g.hidden, g.intermediate, g.shared_intermediate, g.act_block
+        t = {n: self.tap(n) for n in TAPS}
+        shape = {"logits": (rows, g.experts), "ids": (rows, K), "weights": (rows, K), "xq": (rows, H), "xs": (rows, H // B),
+                 "xq_min": (rows, H), "xs_min": (rows, H // B), "h": (-1, I), "hq": (-1, I), "hs": (-1, I // B),
+                 "route_out": (rows, K, H), "routed": (rows, H), "shared_up": (rows, 2 * S), "shared_act": (rows, S),
+                 "shared_aq": (rows, S), "shared_as": (rows, S // B), "shared_down": (rows, H), "out": (rows, H)}
+        for n, s in shape.items():
+            t[n] = t[n].reshape(s)
+        return t
+
+    def census(self):
+        counts = np.zeros(self.g.experts, np.uint32)
+        self._check(self.lib.tfh_layer_census(self.h, counts.ctypes.data, self._err, 512))
+        return counts
+
+    def info(self):
+        v = (ctypes.c_longlong * 8)()
+        self.lib.tfh_layer_info(self.h, v)
+        return dict(zip(["tile_m", "max_tiles", "scratch_bytes", "atlas_bytes", "expert_bytes", "scale_code_bytes", "raw_rows", "coded_rows"], v))

@@ -1,0 +1,199 @@
+// Flat C interface of the host mirror for the python tests and the benchmark (ctypes): one handle per layer instance.
+// Every function returns 0 on success and -1 on failure with the message in the caller's buffer.
+#include "ffn_host.hpp"
+#include <cstdio>
+#include <cstring>
+
+namespace {
+struct Handle {
+    std::shared_ptr<tf::Native> native;
+    std::shared_ptr<tf::Weights> weights;
+    tf::Prepared prepared;
+    std::unique_ptr<tf::LayerFfn> layer;
+    std::unique_ptr<tf::Workspace> workspace;
+    std::unique_ptr<tf::TokenRows> tokens;
+    std::unique_ptr<tf::Stream> stream;
+    std::vector<std::unique_ptr<tf::Graph>> graphs;
+    tf::ScaleCodeReport scale_code;
+    size_t rows = 0;
+};
+template <class F>
+int guarded(char* error, size_t error_len, F&& body) {
+    try { body(); return 0; }
+    catch (const std::exception& e) { if (error && error_len) std::snprintf(error, error_len, "%s", e.what()); return -1; }
+}
+}  // namespace
+
+extern "C" {
+
+// operands: gate_w, bias, bias_alt, w13, s13, w2, s2, sh_w13, sh_s13, sh_w2, sh_s2 (canonical checkpoint layout).
+void* tfh_layer_create(const char* kernel_library, const ca_geometry* geometry, int rows, const void* const* operands, int operands_on_device,
+                       int overlap, int sum_shared, int route_front, int code_scales, char* error, size_t error_len) {
+    Handle* h = new Handle;
+    const int status = guarded(error, error_len, [&] {
+        h->native = std::make_shared<tf::Native>(kernel_library, *geometry);
+        tf::Weights::Host src{(const uint16_t*)operands[0], (const float*)operands[1], (const float*)operands[2], (const uint8_t*)operands[3],
+                              (const uint8_t*)operands[4], (const uint8_t*)operands[5], (const uint8_t*)operands[6], (const uint8_t*)operands[7],
+                              (const uint8_t*)operands[8], (const uint8_t*)operands[9], (const uint8_t*)operands[10]};
+        h->weights = operands_on_device ? std::make_shared<tf::Weights>(*geometry, src, true) : std::make_shared<tf::Weights>(*geometry, src);
+        h->prepared = tf::prepare_layer(*h->native, *h->weights, 0);
+        if (code_scales) h->scale_code = tf::code_layer_scales(*h->native, *h->weights, h->prepared);
+        tf::LayerFfn::Options options;
+        options.overlap = overlap != 0; options.sum_shared = sum_shared != 0; options.route_front = route_front != 0;
+        h->layer = std::make_unique<tf::LayerFfn>(h->native, h->weights, h->prepared, (size_t)rows, options);
+        h->workspace = std::make_unique<tf::Workspace>(h->native, (size_t)rows);
+        std::vector<int64_t> ids((size_t)rows, 0);
+        h->tokens = std::make_unique<tf::TokenRows>(ids.data(), (size_t)rows, (size_t)rows);
+        h->stream = std::make_unique<tf::Stream>();
+        h->rows = (size_t)rows;
+    });
+    if (status != 0) { delete h; return nullptr; }
+    return h;
+}
+void tfh_layer_destroy(void* handle) { delete (Handle*)handle; }
+
+int tfh_layer_set_tokens(void* handle, const int64_t* ids, int live, const int32_t* padding, char* error, size_t error_len) {
+    Handle* h = (Handle*)handle;
+    return guarded(error, error_len, [&] {
+        h->tokens->update(ids, h->rows, (size_t)live);
+        if (padding) h->tokens->set_padding_sources(padding, h->rows);
+    });
+}
+// One eager pass over the device-resident BF16 input [rows][hidden]; returns after the stream has drained.
+int tfh_layer_run(void* handle, uint64_t input, char* error, size_t error_len) {
+    Handle* h = (Handle*)handle;
+    return guarded(error, error_len, [&] {
+        h->layer->run(*h->workspace, input, h->rows * (size_t)h->native->geometry().hidden, *h->tokens, *h->stream);
+        h->stream->synchronize();
+    });
+}
+// Captures one pass into a graph (src/probe.rs:1527-1542 replays the layer the same way); returns the graph's index.
+int tfh_layer_capture(void* handle, uint64_t input, char* error, size_t error_len) {
+    Handle* h = (Handle*)handle;
+    int index = -1;
+    const int status = guarded(error, error_len, [&] {
+        auto graph = std::make_unique<tf::Graph>();
+        graph->capture(*h->stream, [&] { h->layer->run(*h->workspace, input, h->rows * (size_t)h->native->geometry().hidden, *h->tokens, *h->stream); });
+        h->graphs.push_back(std::move(graph));
+        index = (int)h->graphs.size() - 1;
+    });
+    return status == 0 ? index : -1;
+}
+// Replays graphs[order[i % n]] for `warmup` untimed and `steps` timed launches; milliseconds of the timed launches.
+int tfh_layer_time(void* handle, const int* order, int n, int warmup, int steps, float* milliseconds, char* error, size_t error_len) {
+    Handle* h = (Handle*)handle;
+    return guarded(error, error_len, [&] {
+        tf::ensure(n > 0 && steps > 0, "timing arguments");
+        for (int i = 0; i < n; ++i) tf::ensure(order[i] >= 0 && (size_t)order[i] < h->graphs.size(), "graph index");
+        tf::Event begin(true), end(true);
+        for (int i = 0; i < warmup; ++i) h->graphs[order[i % n]]->launch(*h->stream);
+        h->stream->synchronize();
+        begin.record(h->stream->raw());
+        for (int i = 0; i < steps; ++i) h->graphs[order[(warmup + i) % n]]->launch(*h->stream);
+        end.record(h->stream->raw());
+        end.synchronize();
+        *milliseconds = end.elapsed_since(begin);
+    });
+}
+// Times `iterations` back-to-back launches of one expert phase (6: FC1 + SwiGLU, 7: FC2, 5: shared expert) with events on
+// the launch stream, using the routing the last pass left in the workspace.
+int tfh_layer_time_phase(void* handle, int entry, uint64_t input, int iterations, float* milliseconds, char* error, size_t error_len) {
+    Handle* h = (Handle*)handle;
+    return guarded(error, error_len, [&] {
+        tf::Event begin(true), end(true);
+        auto once = [&] {
+            if (entry == 5) h->layer->run_shared(*h->workspace, input, *h->stream);
+            else h->workspace->run_phase(entry, h->layer->expert(), input, h->layer->router().ids(), h->layer->router().routing(), *h->stream);
+        };
+        once();
+        h->stream->synchronize();
+        begin.record(h->stream->raw());
+        for (int i = 0; i < iterations; ++i) once();
+        end.record(h->stream->raw());
+        end.synchronize();
+        *milliseconds = end.elapsed_since(begin);
+    });
+}
+// One eager pass with HIP events on the launch stream around each part (no overlap, separate top-k): milliseconds of
+// [0] gate product + top-k, [1] front-end, [2] FC1 + SwiGLU, [3] FC2, [4] shared expert, [5] sum + addition, [6] whole pass.
+int tfh_layer_profile_step(void* handle, uint64_t input, float* milliseconds, char* error, size_t error_len) {
+    Handle* h = (Handle*)handle;
+    return guarded(error, error_len, [&] {
+        std::vector<std::unique_ptr<tf::Event>> e;
+        for (int i = 0; i < 7; ++i) e.push_back(std::make_unique<tf::Event>(true));
+        tf::LayerFfn& l = *h->layer;
+        tf::Workspace& w = *h->workspace;
+        const tf::Stream& s = *h->stream;
+        const ca_geometry& g = h->native->geometry();
+        w.emit_shared_input(true);
+        e[0]->record(s.raw());
+        l.router().run(input, h->rows * (size_t)g.hidden, *h->tokens, s);
+        e[1]->record(s.raw());
+        w.run_phase(8, l.expert(), input, l.router().ids(), l.router().routing(), s);
+        e[2]->record(s.raw());
+        w.run_phase(6, l.expert(), input, l.router().ids(), l.router().routing(), s);
+        e[3]->record(s.raw());
+        w.run_phase(7, l.expert(), input, l.router().ids(), l.router().routing(), s);
+        e[4]->record(s.raw());
+        l.run_shared(w, 0, s);
+        e[5]->record(s.raw());
+        l.sum_shared(w, h->tokens->active_rows(), s);
+        e[6]->record(s.raw());
+        e[6]->synchronize();
+        for (int i = 0; i < 6; ++i) milliseconds[i] = e[i + 1]->elapsed_since(*e[i]);
+        milliseconds[6] = e[6]->elapsed_since(*e[0]);
+    });
+}
+// Copies a named tap to the host.  Returns the tap's size in bytes (or -1); copies min(bytes, size).
+long long tfh_layer_tap(void* handle, const char* name, void* out, size_t bytes, char* error, size_t error_len) {
+    Handle* h = (Handle*)handle;
+    long long size = -1;
+    guarded(error, error_len, [&] {
+        const std::string n(name);
+        uint64_t p = 0;
+        auto buf = [&](uint64_t ptr, size_t b) { p = ptr; size = (long long)b; };
+        tf::LayerFfn& l = *h->layer;
+        tf::Workspace& w = *h->workspace;
+        if (n == "logits") buf(l.router().logits().ptr(), l.router().logits().bytes());
+        else if (n == "ids") buf(l.router().ids().ptr(), l.router().ids().bytes());
+        else if (n == "weights") buf(l.router().routing().ptr(), l.router().routing().bytes());
+        else if (n == "shared_up") buf(l.shared_up().ptr(), l.shared_up().bytes());
+        else if (n == "shared_act") buf(l.activation().ptr(), l.activation().bytes());
+        else if (n == "shared_aq") buf(l.activation_codes().ptr(), l.activation_codes().bytes());
+        else if (n == "shared_as") buf(l.activation_scales().ptr(), l.activation_scales().bytes());
+        else if (n == "shared_down") buf(l.shared_down().ptr(), l.shared_down().bytes());
+        else if (n == "out") buf(l.output().ptr(), l.output().bytes());
+        else if (n == "routed") buf(w.output().ptr(), w.output().bytes());
+        else {
+            static const std::map<std::string, std::string> alias = {
+                {"xq", "packed_a_storage_ptr"}, {"xs", "scale_storage_ptr"}, {"xq_min", "shared_a_storage_ptr"}, {"xs_min", "shared_scale_storage_ptr"},
+                {"h", "intermediate_ptr"}, {"hq", "intermediate_codes_ptr"}, {"hs", "intermediate_scales_ptr"}, {"task_expert", "task_expert_ptr"},
+                {"task_valid", "task_valid_rows_ptr"}, {"tile_base", "expert_tile_base"}, {"token_map", "token_map_ptr"},
+                {"token_weights", "token_weights_ptr"}, {"route_out", "scatter_ptr"}};
+            auto it = alias.find(n);
+            tf::ensure(it != alias.end(), "unknown tap");
+            buf(w.at(it->second), w.bytes_of(it->second));
+        }
+        h->stream->synchronize();
+        if (out && bytes) tf::check(hipMemcpy(out, (const void*)p, std::min<size_t>(bytes, (size_t)size), hipMemcpyDeviceToHost), "tap download");
+    });
+    return size;
+}
+int tfh_layer_census(void* handle, uint32_t* counts, char* error, size_t error_len) {
+    Handle* h = (Handle*)handle;
+    return guarded(error, error_len, [&] {
+        h->layer->router().census(*h->tokens, *h->stream);
+        h->stream->synchronize();
+        const std::vector<uint32_t> c = h->layer->router().census_counts();
+        std::memcpy(counts, c.data(), c.size() * 4);
+    });
+}
+// info[0] tile_m, [1] max_tiles, [2] scratch bytes, [3] atlas bytes, [4] resident expert bytes, [5] scale-code bytes, [6] raw rows, [7] coded rows
+void tfh_layer_info(void* handle, long long* info) {
+    Handle* h = (Handle*)handle;
+    info[0] = (long long)h->workspace->tile_m(); info[1] = (long long)h->workspace->max_tiles(); info[2] = (long long)h->workspace->scratch_bytes();
+    info[3] = (long long)h->weights->bytes(); info[4] = (long long)h->prepared.resident_bytes; info[5] = (long long)h->scale_code.bytes;
+    info[6] = (long long)h->scale_code.raw_rows; info[7] = (long long)h->scale_code.rows;
+}
+
+}  // extern "C"

@@ -1,0 +1,437 @@
+// Host mirror of the reference's Rust FFN operators: see ffn_host.hpp for the map of names.
+#include "ffn_host.hpp"
+#include <dlfcn.h>
+#include <algorithm>
+
+namespace tf {
+
+namespace {
+template <class F>
+F symbol(void* lib, const char* name) {
+    void* p = dlsym(lib, name);
+    if (!p) throw Error(std::string("missing symbol ") + name);
+    return reinterpret_cast<F>(p);
+}
+size_t align256(size_t n) { return (n + 255) / 256 * 256; }
+}  // namespace
+
+// ---- Native ---------------------------------------------------------------------------------------------------------
+Native::Native(const std::string& library, const ca_geometry& geometry) : g_(geometry) {
+    lib_ = dlopen(library.c_str(), RTLD_NOW | RTLD_LOCAL);
+    if (!lib_) throw Error(std::string("load kernel library: ") + dlerror());
+    ensure(symbol<int (*)()>(lib_, "ca_ffn_abi")() == 1, "FFN native ABI mismatch");                    // src/ffn.rs:76-77
+    ensure(symbol<int32_t (*)()>(lib_, "ca_primitives_abi")() == 1, "primitive entrypoint ABI mismatch"); // src/primitives.rs:104-108
+    const int configured = symbol<int (*)(const ca_geometry*)>(lib_, "ca_ffn_configure")(&g_);
+    if (configured != 0) throw Error("FFN native contract changed: geometry rejected (" + std::to_string(configured) + ")");
+    router_logits_ = symbol<decltype(router_logits_)>(lib_, "ca_router_logits");
+    router_logits_wide_ = symbol<decltype(router_logits_wide_)>(lib_, "ca_router_logits_wide");
+    shared_swiglu_ = symbol<decltype(shared_swiglu_)>(lib_, "ca_shared_swiglu");
+    ffn_add_ = symbol<decltype(ffn_add_)>(lib_, "ca_ffn_add");
+    kernel_launch_ = symbol<decltype(kernel_launch_)>(lib_, "ca_kernel_launch");
+    close_ = symbol<decltype(close_)>(lib_, "ca_primitives_close");
+    launch_ = symbol<decltype(launch_)>(lib_, "ca_primitives_launch");
+    scratch_bytes_ = symbol<decltype(scratch_bytes_)>(lib_, "ca_primitives_scratch_bytes");
+    int32_t status = 0;
+    ctx_ = symbol<void* (*)(int32_t*)>(lib_, "ca_primitives_open")(&status);
+    if (status != 0 || !ctx_) throw Error("initialize primitive library: " + std::to_string(status));   // src/primitives.rs:116-119
+}
+Native::~Native() {
+    if (ctx_ && close_) close_(ctx_);
+    if (lib_) dlclose(lib_);
+}
+void Native::router_logits(int rows, uint64_t x, uint64_t w, uint64_t out, hipStream_t s) const {
+    ensure(router_logits_(rows, (const void*)x, (const void*)w, (void*)out, s) == 0, "tiny router GPU launch failed");   // src/ffn.rs:352-363
+}
+void Native::router_logits_wide(int rows, uint64_t x, uint64_t w, uint64_t out, hipStream_t s) const {
+    ensure(router_logits_wide_(rows, (const void*)x, (const void*)w, (void*)out, s) == 0, "wide router GPU launch failed");
+}
+void Native::shared_swiglu(int rows, uint64_t in, uint64_t out, hipStream_t s) const {
+    ensure(shared_swiglu_(rows, (const void*)in, (void*)out, s) == 0, "shared SwiGLU launch failed");                    // src/ffn.rs:1108-1118
+}
+void Native::ffn_add(int rows, uint64_t routed, uint64_t shared, uint64_t out, hipStream_t s) const {
+    ensure(ffn_add_(rows, (const void*)routed, (const void*)shared, (void*)out, s) == 0, "FFN shared addition launch failed");   // src/ffn.rs:1071-1082
+}
+void Native::launch(const char* name, uint32_t grid_x, uint32_t grid_y, uint32_t block, uint32_t shared, void** args, hipStream_t s) const {
+    const uint32_t grid[3] = {grid_x, grid_y, 1}, blk[3] = {block, 1, 1};
+    const int status = kernel_launch_(name, grid, blk, shared, args, s);
+    if (status != 0) throw Error(std::string("kernel launch failed: ") + name + " (" + std::to_string(status) + ")");
+}
+void Native::primitive(int index, const uint64_t* pointers, size_t np, const int32_t* scalars, size_t ns, hipStream_t s, const char* what) const {
+    const int32_t status = launch_(ctx_, index, pointers, np, scalars, ns, s);
+    if (status != 0) throw Error(std::string(what) + ": primitive launch status " + std::to_string(status));            // src/primitives.rs:150
+}
+int64_t Native::scratch_bytes(int index, int rows) const { return scratch_bytes_(ctx_, index, rows); }
+
+// ---- Weights --------------------------------------------------------------------------------------------------------
+void Weights::layout(const ca_geometry& g) {
+    const size_t H = g.hidden, E = g.experts, I = g.intermediate, S = g.shared_intermediate;
+    const size_t wb = I * H / 2, sb = I * H / 32;
+    size_t at = 0;
+    auto add = [&](const std::string& name, size_t bytes) { views_[name] = View{at, bytes}; at += align256(bytes); };
+    add("ffn.gate.weight", E * H * 2);
+    add("ffn.gate.bias", E * 4);
+    add("ffn.gate.bias_vl", E * 4);
+    // expert groups, contiguous and in the kernels' order (src/weights.rs:330-353): [e][w3 | w1], [e][w2], scales likewise
+    add("ffn.experts.w13", E * 2 * wb);
+    add("ffn.experts.w2", E * wb);
+    add("ffn.experts.s13", E * 2 * sb);
+    add("ffn.experts.s2", E * sb);
+    add("ffn.shared_experts.w13.weight", 2 * S * H);
+    add("ffn.shared_experts.w13.scale", (2 * S / g.shared_bn) * (H / g.shared_bk));
+    add("ffn.shared_experts.w2.weight", H * S);
+    add("ffn.shared_experts.w2.scale", (H / g.shared_bn) * (S / g.shared_bk));
+    add("ffn.shared_experts.w13.prepared", 2 * S * H);
+    add("ffn.shared_experts.w2.prepared", H * S);
+    atlas_ = Buffer<uint8_t>(at);
+}
+void Weights::fill(const Host& src, hipMemcpyKind kind) {
+    auto put = [&](const char* name, const void* from) {
+        const View& v = view(name);
+        check(hipMemcpy((void*)(atlas_.ptr() + v.offset), from, v.bytes, kind), "weight upload");
+    };
+    put("ffn.gate.weight", src.gate_w); put("ffn.gate.bias", src.bias); put("ffn.gate.bias_vl", src.bias_alt);
+    put("ffn.experts.w13", src.w13); put("ffn.experts.w2", src.w2); put("ffn.experts.s13", src.s13); put("ffn.experts.s2", src.s2);
+    put("ffn.shared_experts.w13.weight", src.sh_w13); put("ffn.shared_experts.w13.scale", src.sh_s13);
+    put("ffn.shared_experts.w2.weight", src.sh_w2); put("ffn.shared_experts.w2.scale", src.sh_s2);
+}
+Weights::Weights(const ca_geometry& g, const Host& host) { layout(g); fill(host, hipMemcpyHostToDevice); }
+Weights::Weights(const ca_geometry& g, const Host& device, bool) { layout(g); fill(device, hipMemcpyDeviceToDevice); }
+const View& Weights::view(const std::string& name) const {
+    auto it = views_.find(name);
+    if (it == views_.end()) throw Error("unknown weight view " + name);
+    return it->second;
+}
+uint64_t Weights::pointer_at(size_t offset, size_t bytes) const {
+    ensure(offset + bytes <= atlas_.bytes(), "weight range outside the atlas");
+    return atlas_.ptr() + offset;
+}
+
+// ---- expert preparation ---------------------------------------------------------------------------------------------------
+// src/expert_packing.rs:46-207: validate the contiguous atlas, re-lay every matrix through a scratch buffer and copy it
+// back in place (here: one launch per group, since the layouts tile by 16 rows and expert matrices are whole tiles).
+Prepared prepare_layer(const Native& native, Weights& weights, size_t layer) {
+    const ca_geometry& g = native.geometry();
+    const size_t E = g.experts, n = g.intermediate, k = g.hidden;
+    ensure(n > 0 && n <= 65536 && k > 0 && k <= 65536 && n % 64 == 0 && k % 64 == 0 && n % 512 == 0 && k % 512 == 0,
+           "compact expert layout requires whole N64/K64 row groups");                                // :260-274 (+ the 512 scale words here)
+    const size_t wb = n * k / 2, sb = n * k / 32;
+    const View w13 = weights.view("ffn.experts.w13"), w2 = weights.view("ffn.experts.w2"), s13 = weights.view("ffn.experts.s13"),
+               s2 = weights.view("ffn.experts.s2");
+    ensure(w13.bytes == E * 2 * wb && w2.bytes == E * wb && s13.bytes == E * 2 * sb && s2.bytes == E * sb,
+           "expert atlas is not the exact contiguous kernel layout");                                // :124-128
+    ensure(!weights.expert_ready(), "expert layer already prepared");
+    Stream stream;
+    Buffer<uint8_t> scratch(E * 2 * wb);
+    struct Job { const char* symbol; View view; int rows, cols; size_t unit; };
+    const Job jobs[] = {
+        {"ca_expert_compact_words", w13, (int)(E * 2 * n), (int)k, 32}, {"ca_expert_compact_scales", s13, (int)(E * 2 * n), (int)k, 32},
+        {"ca_expert_compact_words", w2, (int)(E * k), (int)n, 32}, {"ca_expert_compact_scales", s2, (int)(E * k), (int)n, 32}};
+    for (const Job& j : jobs) {
+        uint64_t src = weights.pointer_at(j.view.offset, j.view.bytes), dst = scratch.ptr();
+        int nr = j.rows, kr = j.cols, group = j.rows;
+        void* args[] = {&src, &dst, &nr, &kr, &group};
+        const size_t total = (size_t)j.rows * (j.cols / j.unit);
+        native.launch(j.symbol, (uint32_t)((total + 255) / 256), 1, 256, 0, args, stream.raw());
+        check(hipMemcpyAsync((void*)src, (void*)dst, j.view.bytes, hipMemcpyDeviceToDevice, stream.raw()), "prepared copy back");   // :170
+    }
+    stream.synchronize();
+    weights.finish_expert_layer();
+    Prepared p;
+    p.layer = layer; p.experts = E; p.hidden = k; p.intermediate = n;
+    p.w13_offset = w13.offset; p.w2_offset = w2.offset; p.s13_offset = s13.offset; p.s2_offset = s2.offset;
+    p.resident_bytes = E * (3 * wb + 3 * sb); p.temporary_bytes = scratch.bytes();
+    return p;
+}
+// src/expert_packing.rs:212-259 + src/config.rs:1365-1375
+ScaleCodeReport code_layer_scales(const Native& native, Weights& weights, const Prepared& p) {
+    const size_t E = p.experts, n = p.intermediate, k = p.hidden;
+    const size_t t13 = (n + 127) / 128, s13 = (k + 127) / 128, t2 = (k + 127) / 128, s2 = (n / 32 + 3) / 4;
+    const size_t u13 = t13 * s13, u2 = t2 * s2;
+    const size_t f13 = E * 2 * u13 * 16, b13 = f13 + E * 2 * u13 * 4, c2 = b13 + (2 * E + 3) / 4 * 4, f2 = c2 + E * u2 * 16,
+                 b2 = f2 + E * u2 * 4, words = b2 + E;
+    Buffer<uint32_t> code(words), error(1);
+    Buffer<unsigned long long> counts(1);
+    code.zero(); error.zero(); counts.zero();
+    Stream stream;
+    struct Part { size_t offset, matrices, rows, columns, c, f, b; };
+    const Part parts[] = {{p.s13_offset, 2 * E, n, k / 32, 0, f13, b13}, {p.s2_offset, E, k, n / 32, c2, f2, b2}};
+    for (const Part& part : parts) {
+        const size_t units = (part.rows + 127) / 128 * ((part.columns + 3) / 4);
+        uint64_t src = weights.pointer_at(part.offset, part.matrices * part.rows * part.columns);
+        uint64_t cp = code.ptr() + part.c * 4, fp = code.ptr() + part.f * 4, bp = code.ptr() + part.b * 4, status = error.ptr(), tally = counts.ptr();
+        int nr = (int)part.rows, cols = (int)part.columns;
+        void* a1[] = {&src, &cp, &fp, &bp, &nr, &cols};
+        native.launch("ca_expert_scale_code1", (uint32_t)part.matrices, 1, 256, 0, a1, stream.raw());
+        void* a2[] = {&src, &cp, &fp, &bp, &status, &nr, &cols};
+        native.launch("ca_expert_scale_code1_check", (uint32_t)((units * 128 + 255) / 256), (uint32_t)part.matrices, 256, 0, a2, stream.raw());
+        size_t flag_words = part.matrices * units * 4;
+        void* a3[] = {&fp, &tally, &flag_words};
+        native.launch("ca_expert_scale_code1_census", (uint32_t)((flag_words + 255) / 256), 1, 256, 0, a3, stream.raw());
+    }
+    stream.synchronize();
+    const uint32_t status = error.download()[0];
+    if (status != 0) throw Error("expert scale code failed its decode check (layer " + std::to_string(p.layer) + ", error " + std::to_string(status) + ")");
+    ScaleCodeReport report;
+    report.bytes = words * 4;
+    report.raw_rows = (size_t)counts.download()[0];
+    report.rows = E * (2 * u13 + u2) * 128;
+    weights.install_expert_scale_code1(std::move(code));
+    return report;
+}
+
+Expert::Expert(std::shared_ptr<Weights> weights, Prepared layout) : weights_(std::move(weights)), layout_(layout) {
+    ensure(weights_->expert_ready(), "expert layer is not ready");                                        // src/moe.rs:128-131
+}
+std::pair<uint64_t, size_t> Expert::region(const std::string& role) const {                                // src/moe.rs:143-155
+    const Prepared& l = layout_;
+    const size_t wb = l.hidden * l.intermediate / 2, sb = l.hidden * l.intermediate / 32;
+    size_t offset, bytes;
+    if (role == "w13") { offset = l.w13_offset; bytes = 2 * l.experts * wb; }
+    else if (role == "w2") { offset = l.w2_offset; bytes = l.experts * wb; }
+    else if (role == "s13") { offset = l.s13_offset; bytes = 2 * l.experts * sb; }
+    else if (role == "s2") { offset = l.s2_offset; bytes = l.experts * sb; }
+    else throw Error("unknown expert operand");
+    return {weights_->pointer_at(offset, bytes), bytes};
+}
+
+SharedMatrix prepare_shared(const Native& native, Weights& weights, const std::string& name, size_t n, size_t k) {
+    const View src = weights.view(name + ".weight"), dst = weights.view(name + ".prepared");
+    ensure(src.bytes == n * k && dst.bytes == n * k && n % 16 == 0 && k % 128 == 0, "shared matrix geometry mismatch");
+    Stream stream;
+    uint64_t from = weights.pointer_at(src.offset, src.bytes), to = weights.pointer_at(dst.offset, dst.bytes);
+    int nr = (int)n, kr = (int)k, inverse = 0;
+    void* args[] = {&from, &to, &nr, &kr, &inverse};
+    native.launch("ca_dense_compact_fp8", (uint32_t)((n * (k / 16) + 255) / 256), 1, 256, 0, args, stream.raw());
+    stream.synchronize();
+    return SharedMatrix{to, weights.ptr(name + ".scale"), n, k};
+}
+
+// ---- TokenRows --------------------------------------------------------------------------------------------------------------
+TokenRows::TokenRows(const int64_t* ids, size_t rows, size_t live) : ids_(rows), live_(1), padding_sources_(rows), rows_(rows) {
+    ensure(rows > 0 && rows <= 65536, "token row capacity");                                                // src/ffn.rs:103
+    std::vector<int32_t> none(rows, -1);
+    padding_sources_.upload(none);
+    update(ids, rows, live);
+}
+void TokenRows::update(const int64_t* ids, size_t rows, size_t live) {
+    bool domain = rows == rows_ && live <= rows_;
+    for (size_t i = 0; domain && i < rows; ++i) domain = ids[i] >= 0 && ids[i] < 129280;
+    ensure(domain, "router token metadata domain");                                                          // src/ffn.rs:121-126
+    ids_.upload(ids, rows);
+    const int32_t n = (int32_t)live;
+    live_.upload(&n, 1);
+    active_rows_ = live;
+    padding_active_ = false;                                                                                 // :132-133
+}
+void TokenRows::set_padding_sources(const int32_t* sources, size_t rows) {
+    bool ok = rows == rows_;
+    for (size_t r = 0; ok && r < rows; ++r) {
+        const int32_t s = sources[r];
+        ok = s < 0 || ((size_t)s < active_rows_ && (size_t)s != r && sources[s] < 0);
+    }
+    ensure(ok, "padding route sources must name live rows");                                                 // src/ffn.rs:139-141
+    padding_sources_.upload(sources, rows);
+    padding_active_ = true;
+}
+
+// ---- Router -----------------------------------------------------------------------------------------------------------------
+Router::Router(std::shared_ptr<const Native> native, std::shared_ptr<Weights> weights, size_t rows)
+    : native_(std::move(native)), weights_(std::move(weights)), rows_(rows), logits_(rows * native_->geometry().experts),
+      routing_(rows * native_->geometry().topk), ids_(rows * native_->geometry().topk), census_(native_->geometry().experts) {
+    const ca_geometry& g = native_->geometry();
+    ensure(rows >= 1, "router row capacity");
+    ensure(weights_->view("ffn.gate.weight").bytes == (size_t)g.experts * g.hidden * 2 && weights_->view("ffn.gate.bias").bytes == (size_t)g.experts * 4,
+           "router checkpoint shape/dtype mismatch");                                                        // src/ffn.rs:225-228
+    census_.zero();
+}
+std::optional<RouteOperands> Router::run_routed(uint64_t input, size_t input_len, const TokenRows& tokens, bool fused, const Stream& stream) {
+    const ca_geometry& g = native_->geometry();
+    ensure(input_len == rows_ * (size_t)g.hidden && tokens.rows() == rows_, "router shape/context mismatch");   // src/ffn.rs:331-339
+    ensure(!stream_set_ || stream_ == stream.raw(), "router needs one ordered stream");                        // :340-345
+    stream_ = stream.raw(); stream_set_ = true;
+    const uint64_t gate = weights_->ptr("ffn.gate.weight");
+    if (rows_ <= 64) {
+        for (size_t offset = 0; offset < rows_; offset += 16)                                                  // :351-364
+            native_->router_logits((int)std::min<size_t>(16, rows_ - offset), input + offset * g.hidden * 2, gate,
+                                   logits_.ptr() + offset * g.experts * 4, stream.raw());
+    } else {
+        native_->router_logits_wide((int)rows_, input, gate, logits_.ptr(), stream.raw());                     // Scores::Vendor, :366
+    }
+    const uint64_t bias = weights_->ptr("ffn.gate.bias"), bias_alt = weights_->ptr("ffn.gate.bias_vl");
+    if (fused) {
+        ensure(rows_ * g.topk <= 1024, "fused routing owner");                                                 // :370-371
+        return RouteOperands{logits_.ptr(), bias, bias_alt, tokens.ids().ptr(), tokens.live().ptr(),
+                             tokens.padding_active() ? tokens.padding_sources().ptr() : 0, ids_.ptr(), routing_.ptr(), rows_};
+    }
+    uint64_t lp = logits_.ptr(), tp = tokens.ids().ptr(), vp = tokens.live().ptr(), ip = ids_.ptr(), wp = routing_.ptr();
+    uint64_t b = bias, ba = bias_alt;
+    const uint32_t blocks = (uint32_t)((rows_ + 15) / 16);
+    uint64_t pad = (tokens.padding_active() && blocks == 1) ? tokens.padding_sources().ptr() : 0;
+    int rows = (int)rows_, experts = g.experts, topk = g.topk, scoring = g.scoring;
+    float scale = g.route_scale;
+    long long alt = g.alt_token;
+    void* args[] = {&lp, &b, &ba, &tp, &vp, &pad, &ip, &wp, &rows, &experts, &topk, &scoring, &scale, &alt};
+    native_->launch("ca_route_topk", blocks, 1, 1024, 0, args, stream.raw());                                  // :380-395
+    if (tokens.padding_active() && blocks > 1) {                                                               // :396-409
+        uint64_t source = tokens.padding_sources().ptr();
+        void* pargs[] = {&ip, &wp, &source, &rows, &topk};
+        native_->launch("ca_route_padding_rows", (uint32_t)((rows_ * g.topk + 127) / 128), 1, 128, 0, pargs, stream.raw());
+    }
+    return std::nullopt;
+}
+void Router::census(const TokenRows& tokens, const Stream& stream) {                                          // src/route_census.rs:63-76
+    const ca_geometry& g = native_->geometry();
+    uint64_t ip = ids_.ptr(), vp = tokens.live().ptr(), cp = census_.ptr();
+    int rows = (int)rows_, topk = g.topk, experts = g.experts;
+    void* args[] = {&ip, &vp, &rows, &topk, &cp, &experts};
+    native_->launch("ca_route_census", (uint32_t)((rows_ * g.topk + 255) / 256), 1, 256, 0, args, stream.raw());
+}
+
+// ---- Workspace ----------------------------------------------------------------------------------------------------------------
+// The runtime contract's scratch layout (src/moe.rs:34-68 Contract / Node pointer offsets), computed instead of read from
+// JSON: the same table tools/contracts writes into contracts/runtime-contract-m<rows>.json.
+Workspace::Workspace(std::shared_ptr<const Native> native, size_t rows) : native_(std::move(native)), rows_(rows) {
+    const ca_geometry& g = native_->geometry();
+    ensure(rows >= 1, "MoE workspace rows");
+    tile_m_ = rows <= 64 ? 16 : 128;
+    const size_t pairs = rows * g.topk;
+    max_tiles_ = pairs / tile_m_ + std::min<size_t>(g.experts, pairs);
+    const size_t padded = max_tiles_ * tile_m_, H = g.hidden, I = g.intermediate, B = g.act_block;
+    size_t at = 0;
+    auto add = [&](const char* name, size_t bytes) { regions_[name] = View{at, bytes}; at += align256(bytes); };
+    add("packed_a_storage_ptr", rows * H); add("scale_storage_ptr", rows * H / B);
+    add("shared_a_storage_ptr", rows * H); add("shared_scale_storage_ptr", rows * H / B);
+    add("intermediate_ptr", padded * I * 2); add("intermediate_codes_ptr", padded * I); add("intermediate_scales_ptr", padded * I / B);
+    add("task_expert_ptr", max_tiles_ * 4); add("task_valid_rows_ptr", max_tiles_ * 4); add("expert_tile_base", (g.experts + 1) * 4);
+    add("token_map_ptr", padded * 4); add("token_weights_ptr", padded * 4);
+    add("scatter_ptr", pairs * H * 2);
+    add("plan_scratch_ptr", ((pairs + 63) / 64 * g.experts + pairs) * 4);
+    scratch_ = Buffer<uint8_t>(at);
+    scratch_.zero();                                                                                          // scratch_initializer "zero", src/moe.rs:440
+    output_ = Buffer<uint16_t>(rows * H);
+    output_.zero();
+}
+uint64_t Workspace::at(const std::string& name) const {
+    auto it = regions_.find(name);
+    if (it == regions_.end()) throw Error("unknown MoE runtime pointer role");                                 // src/moe.rs:1214-1216
+    return scratch_.ptr() + it->second.offset;
+}
+size_t Workspace::bytes_of(const std::string& name) const {
+    auto it = regions_.find(name);
+    if (it == regions_.end()) throw Error("unknown MoE runtime pointer role");
+    return it->second.bytes;
+}
+void Workspace::guard_stream(const Stream& stream) {                                                           // src/moe.rs:584-595
+    ensure(!stream_set_ || stream_ == stream.raw(), "MoE workspace needs one ordered stream");
+    stream_ = stream.raw(); stream_set_ = true;
+}
+void Workspace::pointers(const Expert& expert, uint64_t input, const Buffer<int32_t>& ids, const Buffer<float>& routing_weights, uint64_t* p) const {
+    const char* scratch_names[] = {"packed_a_storage_ptr", "scale_storage_ptr", "shared_a_storage_ptr", "shared_scale_storage_ptr",
+                                   "intermediate_ptr", "intermediate_codes_ptr", "intermediate_scales_ptr", "task_expert_ptr",
+                                   "task_valid_rows_ptr", "expert_tile_base", "token_map_ptr", "token_weights_ptr"};
+    p[0] = input; p[1] = ids.ptr(); p[2] = routing_weights.ptr();
+    for (int i = 0; i < 12; ++i) p[3 + i] = at(scratch_names[i]);
+    if (!emit_shared_input_) p[5] = p[6] = 0;
+    p[15] = expert.region("w13").first; p[16] = expert.region("s13").first; p[17] = expert.region("w2").first; p[18] = expert.region("s2").first;
+    p[19] = at("scatter_ptr"); p[20] = at("plan_scratch_ptr");
+}
+std::optional<std::pair<uint64_t, size_t>> Workspace::run_live_for_ffn(const Expert& expert, uint64_t input, size_t input_len, const Buffer<int32_t>& ids,
+                                                                       const Buffer<float>& routing_weights, size_t live, bool fuse_sum,
+                                                                       const std::optional<RouteOperands>& route, const Stream& stream) {
+    const ca_geometry& g = native_->geometry();
+    ensure(live <= rows_, "MoE live row domain");                                                             // src/moe.rs:1045
+    guard_stream(stream);
+    ensure(input_len == rows_ * (size_t)g.hidden, "BF16 MoE operand");                                         // :1057-1058
+    ensure(expert.layout().experts == (size_t)g.experts && expert.layout().hidden == (size_t)g.hidden &&
+               expert.layout().intermediate == (size_t)g.intermediate && ids.len() == rows_ * g.topk && routing_weights.len() == rows_ * g.topk,
+           "MoE input shape mismatch");                                                                       // :1103-1114
+    uint64_t p[27];
+    pointers(expert, input, ids, routing_weights, p);
+    int32_t scalars[7] = {(int32_t)rows_, (int32_t)rows_, (int32_t)(max_tiles_ * tile_m_), (int32_t)max_tiles_, (int32_t)tile_m_, 1, 0};
+    if (route) {
+        ensure(route->ids == p[1] && route->weights == p[2] && route->owner_rows == rows_ && route->logits && route->bias && route->live,
+               "fused routing domain");                                                                       // :1266-1269
+        p[21] = route->logits; p[22] = route->bias; p[23] = route->bias_alt; p[24] = route->tokens; p[25] = route->live; p[26] = route->padding;
+        scalars[6] = (int32_t)route->owner_rows;
+        native_->primitive(1, p, 27, scalars, 7, stream.raw(), "integration.tp_moe.dynamic (route front)");
+    } else {
+        native_->primitive(0, p, 21, scalars, 6, stream.raw(), "integration.tp_moe.dynamic");
+    }
+    if (fuse_sum) return std::make_pair(at("scatter_ptr"), live);                                              // :1005-1008
+    const uint64_t sp[3] = {at("scatter_ptr"), output_.ptr(), 0};
+    const int32_t ss[3] = {(int32_t)live, 0, 0};                                                              // active_m patched to the live rows, :1229
+    native_->primitive(2, sp, 3, ss, 3, stream.raw(), "moe.w4a16.topk_sum");
+    return std::nullopt;
+}
+void Workspace::run_phase(int entry, const Expert& expert, uint64_t input, const Buffer<int32_t>& ids, const Buffer<float>& routing_weights,
+                          const Stream& stream) {
+    ensure(entry == 6 || entry == 7 || entry == 8, "phase entry");
+    uint64_t p[21];
+    pointers(expert, input, ids, routing_weights, p);
+    const int32_t scalars[6] = {(int32_t)rows_, (int32_t)rows_, (int32_t)(max_tiles_ * tile_m_), (int32_t)max_tiles_, (int32_t)tile_m_, 1};
+    native_->primitive(entry, p, 21, scalars, 6, stream.raw(), "expert phase");
+}
+
+// ---- LayerFfn -----------------------------------------------------------------------------------------------------------------
+LayerFfn::LayerFfn(std::shared_ptr<const Native> native, std::shared_ptr<Weights> weights, Prepared layout, size_t rows, Options options)
+    : native_(native), router_(native, weights, rows), expert_(weights, layout),
+      shared_up_(rows * 2 * native->geometry().shared_intermediate), activation_(rows * native->geometry().shared_intermediate),
+      shared_down_(rows * native->geometry().hidden), output_(rows * native->geometry().hidden),
+      activation_codes_(rows * native->geometry().shared_intermediate),
+      activation_scales_(rows * native->geometry().shared_intermediate / native->geometry().act_block), rows_(rows), options_(options) {
+    const ca_geometry& g = native->geometry();
+    ensure(layout.experts == (size_t)g.experts, "FFN namespace/expert geometry");                              // src/ffn.rs:617-620
+    shared_w13_ = prepare_shared(*native, *weights, "ffn.shared_experts.w13", 2 * g.shared_intermediate, g.hidden);
+    shared_w2_ = prepare_shared(*native, *weights, "ffn.shared_experts.w2", g.hidden, g.shared_intermediate);
+    output_.zero();
+    if (options_.overlap) {                                                                                    // :700-706 SharedBranch
+        branch_stream_ = std::make_unique<Stream>();
+        input_ready_ = std::make_unique<Event>();
+        output_ready_ = std::make_unique<Event>();
+    }
+}
+void LayerFfn::run_shared(const Workspace& workspace, uint64_t input, const Stream& stream) {                  // :1053-1124 run_shared / run_shared_quantized_input + finish_shared
+    if (input) {   // Linear::run: this branch quantizes the BF16 input itself (src/fp8_linear.rs:782-806)
+        const uint64_t q[5] = {input, 0, 0, workspace.at("shared_a_storage_ptr"), workspace.at("shared_scale_storage_ptr")};
+        const int32_t qs[3] = {(int32_t)rows_, native_->geometry().hidden, 0};
+        native_->primitive(3, q, 5, qs, 3, stream.raw(), "gemm.mxfp8_quant_cute");
+    }
+    const uint64_t p[11] = {workspace.at("shared_a_storage_ptr"), workspace.at("shared_scale_storage_ptr"), shared_w13_.values, shared_w13_.scales,
+                            shared_w2_.values, shared_w2_.scales, activation_.ptr(), activation_codes_.ptr(), activation_scales_.ptr(),
+                            shared_up_.ptr(), shared_down_.ptr()};
+    const int32_t s[1] = {(int32_t)rows_};
+    native_->primitive(5, p, 11, s, 1, stream.raw(), "ffn.shared_expert");
+}
+void LayerFfn::add_shared(const Workspace& workspace, const Stream& stream) {                                  // :1066-1084
+    native_->ffn_add((int)rows_, workspace.output().ptr(), shared_down_.ptr(), output_.ptr(), stream.raw());
+}
+void LayerFfn::run(Workspace& workspace, uint64_t input, size_t input_len, const TokenRows& tokens, const Stream& stream) {   // :974-1047
+    const ca_geometry& g = native_->geometry();
+    ensure(workspace.rows() == rows_, "MoE workspace context mismatch");
+    const bool fused = options_.route_front && rows_ * g.topk <= 1024;                                          // :988-990
+    // Dual-stream schedule (:1007-1010, :1028-1036): the shared branch forks before routing, quantizes the input itself
+    // and joins before the sum.  Without the branch the front-end emits the shared-flavour codes beside the routed ones.
+    workspace.emit_shared_input(!branch_stream_);
+    if (branch_stream_) {
+        input_ready_->record(stream.raw());
+        input_ready_->wait(branch_stream_->raw());
+        run_shared(workspace, input, *branch_stream_);
+        output_ready_->record(branch_stream_->raw());
+    }
+    const std::optional<RouteOperands> route = router_.run_routed(input, input_len, tokens, fused, stream);
+    const auto deferred = workspace.run_live_for_ffn(expert_, input, input_len, router_.ids(), router_.routing(), tokens.active_rows(),
+                                                     options_.sum_shared, route, stream);
+    if (branch_stream_) output_ready_->wait(stream.raw());
+    else run_shared(workspace, 0, stream);
+    if (deferred) sum_shared(workspace, deferred->second, stream);
+    else add_shared(workspace, stream);
+}
+void LayerFfn::sum_shared(const Workspace& workspace, size_t live_rows, const Stream& stream) {               // :1037-1046 ca_ffn_sum_shared
+    const ca_geometry& g = native_->geometry();
+    uint64_t routes = workspace.at("scatter_ptr"), shared = shared_down_.ptr(), routed = workspace.output().ptr(), output = output_.ptr();
+    int n = (int)(rows_ * g.hidden), live = (int)live_rows, topk = g.topk, hidden = g.hidden;
+    void* args[] = {&routes, &shared, &routed, &output, &n, &live, &topk, &hidden};
+    native_->launch("ca_ffn_sum_shared", (uint32_t)((n / 8 + 255) / 256), 1, 256, 0, args, stream.raw());
+}
+
+}  // namespace tf
