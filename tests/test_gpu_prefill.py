@@ -1,0 +1,100 @@
+"""GPU parity of the many-row (prefill) path: wide plan, grouped GEMM on the scaled matrix instruction with the fused
+SwiGLU -> FP8 epilogue, scatter with routing weights, ordered sum.  The gate product of many rows runs on the matrix cores
+(its summation order is not the oracle's), so routing is checked bit-exactly against the oracle's routing of the GPU's own
+logits, and the logits themselves by tolerance."""
+import numpy as np
+import pytest
+import torch
+
+import oracle
+from helpers import CONFIGS, GpuLayer, geometry, np_of, synth, u16
+from test_gpu_layer import check_layer
+
+pytestmark = pytest.mark.gpu
+
+
+def small_wide(mode, rows, experts=16, topk=2):
+    g = geometry(1024, experts, topk, 512, 512, mode)
+    ops = synth.LayerOperands(g, "wide-small", device="cpu")
+    x = synth.activations("wide-small", rows, g.hidden)
+    return g, ops, x
+
+
+@pytest.mark.parametrize("mode,rows", [("benchmark", 300), ("reference", 129), ("benchmark", 1000)])
+def test_small_wide_layer(mode, rows):
+    g, ops, x = small_wide(mode, rows)
+    layer = GpuLayer(g, ops, rows)
+    taps = layer.run(x)
+    want = oracle.router_logits(u16(x), u16(ops.gate_w))
+    assert np.abs(taps["logits"] - want).max() <= 1e-5 * np.abs(want).max() + 1e-6
+    print(mode, rows, check_layer(g, ops, x, taps, exact_logits=False, max_rel=2e-2 if mode == "reference" else 1e-2))
+    layer.close()
+
+
+def test_wide_live_rows_and_skewed_routing():
+    g, ops, x = small_wide("benchmark", 700)
+    ops.bias = synth.zipf_bias(g.experts, 1.1, 0.5)        # popularity ~ rank^-1.1: a few experts take most rows
+    layer = GpuLayer(g, ops, 700)
+    taps = layer.run(x, live=650)
+    counts = np.bincount(taps["ids"][taps["ids"] >= 0], minlength=g.experts)
+    assert counts.max() > 3 * counts.mean()
+    check_layer(g, ops, x, taps, live=650, exact_logits=False)
+    layer.close()
+
+
+@pytest.mark.parametrize("config", ["c4"])
+def test_full_size_prefill(config):
+    c = CONFIGS[config]
+    g = geometry(c["hidden"], c["experts"], c["topk"], c["inter"], c["shared"], "benchmark")
+    ops = synth.LayerOperands(g, config, device="cuda")
+    rows = c["rows"]
+    x = synth.activations(config, rows, g.hidden, device="cuda")
+    layer = GpuLayer(g, ops, rows)
+    taps = layer.run(x)
+    # the oracle is evaluated on a sample of rows (all their routes), against the GPU's own routing
+    sample = np.arange(0, rows, rows // 16)[:16]
+    sub_taps = subset(taps, sample, g, rows)
+    print(config, check_rows(g, ops, x[torch.as_tensor(sample, device=x.device)], sub_taps, taps, sample))
+    layer.close()
+
+
+def subset(taps, sample, g, rows):
+    return {k: taps[k][sample] for k in ["logits", "ids", "weights", "xq", "xs", "xq_min", "xs_min", "route_out", "routed", "shared_up",
+                                         "shared_act", "shared_aq", "shared_as", "shared_down", "out"]}
+
+
+def check_rows(g, ops, x, sub, taps, sample):
+    """Row-sampled check of a large layer: every per-row tap of the sampled rows against the oracle's evaluation of those
+    rows (routing from the GPU's own logits), plus the global invariants of the plan."""
+    from helpers import bf16_ulp_distance, error_stats, oracle_layer
+    rows_all = taps["ids"].shape[0]
+    K, I, B = g.topk, g.intermediate, g.act_block
+    want = oracle_layer(g, ops, x, logits=sub["logits"])
+    ref_logits = oracle.router_logits(u16(x), u16(ops.gate_w))
+    assert np.abs(sub["logits"] - ref_logits).max() <= 1e-5 * np.abs(ref_logits).max() + 1e-6
+    assert np.array_equal(sub["ids"], want["ids"]) and np.array_equal(sub["weights"].view(np.uint32), want["weights"].view(np.uint32))
+    for name in ["xq", "xs", "xq_min", "xs_min"]:
+        assert np.array_equal(sub[name], want[name]), name
+    # plan invariants over the whole batch
+    base, te, tv, tmap, tw = oracle.plan(taps["ids"], taps["weights"], g.experts, 1, 128, capacity_tiles=len(taps["task_expert"]))
+    tiles = int(base[-1])
+    assert np.array_equal(taps["tile_base"], base) and np.array_equal(taps["task_expert"][:tiles], te[:tiles])
+    occupied = tmap >= 0
+    assert np.array_equal(taps["token_map"][occupied], tmap[occupied])
+    # intermediate rows of the sampled tokens
+    inverse = np.full(rows_all * K, -1, np.int64)
+    inverse[tmap[occupied]] = np.nonzero(occupied)[0]
+    routes = (sample[:, None] * K + np.arange(K)[None, :]).ravel()
+    phys = inverse[routes]
+    h_gpu = taps["h"][phys]
+    assert bf16_ulp_distance(h_gpu, want["h"].reshape(-1, I)) <= 2.0
+    hq, hs = oracle.quantize_rows(h_gpu, B, 0.0)
+    assert np.array_equal(taps["hq"][phys], hq) and np.array_equal(taps["hs"][phys], hs)
+    assert bf16_ulp_distance(sub["shared_up"], want["shared_up"]) <= 2.0
+    act, aq, asc = oracle.shared_swiglu_quant(sub["shared_up"], B, g.swiglu_limit)
+    assert np.array_equal(sub["shared_act"], act) and np.array_equal(sub["shared_aq"], aq) and np.array_equal(sub["shared_as"], asc)
+    routed, out = oracle.ffn_sum_shared(sub["route_out"], sub["shared_down"])
+    assert np.array_equal(sub["routed"], routed) and np.array_equal(sub["out"], out)
+    rel, mean = error_stats(sub["out"], want["out"])
+    assert rel <= 1e-2 and mean <= 1e-3, (rel, mean)
+    return rel, mean

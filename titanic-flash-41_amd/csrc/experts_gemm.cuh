@@ -1,4 +1,20 @@
-// Many-row (prefill) expert projections: grouped GEMM on the scaled FP8 x FP4 matrix instruction.
+// Many-row (prefill) expert projections: grouped GEMM on v_mfma_scale_f32_16x16x128_f8f6f4.
+//
+// One task = one M tile of 128 physical rows (one expert's rows, gathered through the permutation map) x one column
+// group.  A workgroup of four waves keeps a 128 x 256 accumulator (each wave 128 rows x 64 weight rows, in AGPRs/VGPRs):
+//   FC1: 128 intermediate columns = 128 "up" + 128 "gate" weight rows, so SwiGLU and the FP8 requantization of the
+//        result (one scale a row and `act_block` columns) run in the epilogue, from registers;
+//   FC2 / dense: 256 output columns; routed rows are scaled by their routing weight and scattered to route order.
+// The E4M3 token tile goes through LDS (double-buffered, stored in matrix-instruction fragment order so every wave reads
+// 1 KiB contiguous, conflict-free, per fragment); the prepared weights go from global memory straight into the B operand
+// (each wave owns its weight rows, 1 KiB contiguous per fragment and k-step) with the next k-step in flight.
+// Workgroups are persistent and XCD-aware: workgroup b runs on XCD b % 8 and only ever touches 1/8 of the column groups,
+// so every XCD's L2 holds its own slices of the expert's weights while the expert's tiles pass by; partially filled
+// tiles skip the 16-row fragments past their last valid row.
+//
+// Reference semantics (contract level): the two phase kernels of the reference's dynamic MoE node
+// (src/moe.rs:1098-1289; runtime/kernels/moe-runtime-*/manifest.json precision string) and its block-scaled dense GEMM
+// for the shared expert (src/fp8_linear.rs:782-806).
 #pragma once
 #include "experts_stream.cuh"
 
@@ -6,14 +22,14 @@
 #define TF_GEMM_TILE_M 128
 
 struct GemmArgs {
-    const uint8_t* a_codes;
-    const uint8_t* a_scales;
-    const uint8_t* w;
-    const uint8_t* ws;
+    const uint8_t* a_codes;          // E4M3 [rows][k]: token rows (FC1), physical rows (routed FC2), dense rows
+    const uint8_t* a_scales;         // UE8M0 [rows][k / act_block]
+    const uint8_t* w;                // prepared weights, expert-major
+    const uint8_t* ws;               // prepared scales (FP4) or row-major block scales (FP8)
     long long w_expert_stride, ws_expert_stride;
     int bn, bk;
-    const int32_t* expert_tile_base;
-    const int32_t* task_expert;
+    const int32_t* expert_tile_base; // routed: [experts + 1]
+    const int32_t* task_expert;      // routed: [tile * groups]; null: dense
     const int32_t* task_valid_rows;
     const int32_t* token_map;
     const float* token_weights;
@@ -21,26 +37,314 @@ struct GemmArgs {
     int dense_rows;
     int k, inter, hidden, act_block;
     float limit;
-    uint16_t* h_bf16;
-    uint8_t* h_codes;
-    uint8_t* h_scales;
-    uint16_t* out;
-    uint16_t* tap;
+    uint16_t* h_bf16;                // FC1: optional BF16 activation [phys_row][inter]
+    uint8_t* h_codes;                // FC1: E4M3 activation codes [phys_row][inter]
+    uint8_t* h_scales;               // FC1: UE8M0 [phys_row][inter / act_block]
+    uint16_t* out;                   // FC2 / dense: BF16 [route or row][hidden]
+    uint16_t* tap;                   // shared FC1: optional BF16 projections [row][2 inter]
 };
-inline int tf_launch_fc1_gemm(const GemmArgs&, int, hipStream_t) { return -4; }
-inline int tf_launch_fc2_gemm(const GemmArgs&, int, hipStream_t) { return -4; }
-inline int tf_launch_dense_gemm(const GemmArgs&, int, hipStream_t) { return -4; }
-inline int tf_launch_shared_fc1_gemm(const GemmArgs&, int, hipStream_t) { return -4; }
 
-// Gate product for many rows.  grid (ceil(rows / 64), experts / 32), block 128.
+enum { TF_GEMM_FC1_ROUTED = 0, TF_GEMM_FC1_SHARED = 1, TF_GEMM_FC2_ROUTED = 2, TF_GEMM_DENSE = 3 };
+
+template <bool FP8>
+struct BFrag { u4v lo; u4v hi; };
+
+template <bool FP8, int MODE>
+__global__ void __launch_bounds__(256) tf_gemm(const GemmArgs p) {
+    constexpr bool FC1 = MODE == TF_GEMM_FC1_ROUTED || MODE == TF_GEMM_FC1_SHARED;
+    constexpr bool ROUTED = MODE == TF_GEMM_FC1_ROUTED || MODE == TF_GEMM_FC2_ROUTED;
+    constexpr int GROUP_COLS = FC1 ? 128 : 256;          // output columns a task covers
+    __shared__ __attribute__((aligned(16))) uint8_t s_a[2][16384];     // [stage][m-frag 8][half 2][lane 64][16 B]
+    __shared__ uint32_t s_as[2][128];                                   // [stage][row]: scale bytes of the row's four K32 blocks
+    __shared__ float s_amax[4][128];
+    __shared__ long long s_row[128];                                    // source row of each tile row (-1: unused)
+    const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6, g = lane >> 4, r16 = lane & 15;
+    const int ksteps = p.k / 128;
+    const int n_cols = FC1 ? p.inter : p.hidden, groups = n_cols / GROUP_COLS;
+    const int tiles = ROUTED ? p.expert_tile_base[p.experts] : (p.dense_rows + 127) / 128;
+    const int xcd = blockIdx.x & 7, local = blockIdx.x >> 3, local_count = gridDim.x >> 3;
+    const bool split = groups % 8 == 0;
+    const int gpx = split ? groups / 8 : 0;
+    const long long my_tasks = split ? (long long)tiles * gpx : ((long long)tiles * groups - xcd + 7) / 8;
+
+    for (long long q = local; q < my_tasks; q += local_count) {
+        int tile, ng;
+        if (split) { tile = (int)(q / gpx); ng = xcd * gpx + (int)(q % gpx); }
+        else { const long long id = q * 8 + xcd; tile = (int)(id / groups); ng = (int)(id % groups); }
+        int expert = 0, valid;
+        if (ROUTED) { expert = p.task_expert[tile * p.groups]; valid = p.task_valid_rows[tile * p.groups]; }
+        else valid = min(128, p.dense_rows - tile * 128);
+        const uint8_t* w = p.w + (size_t)expert * p.w_expert_stride;
+        const uint8_t* ws = p.ws + (size_t)expert * p.ws_expert_stride;
+        __syncthreads();
+        if (tid < 128) {
+            long long src = -1;
+            if (tid < valid) {
+                if (MODE == TF_GEMM_FC1_ROUTED) src = p.token_map[tile * 128 + tid] / p.topk;
+                else src = (long long)tile * 128 + tid;
+            }
+            s_row[tid] = src;
+        }
+        __syncthreads();
+        // this thread's four 16-byte chunks of every k-step's A tile: chunk id c = tid + 256 i -> row c / 8, piece c % 8
+        const uint8_t* a_src[4];
+        int a_dst[4];
+#pragma unroll
+        for (int i = 0; i < 4; ++i) {
+            const int c = tid + 256 * i, row = c >> 3, piece = c & 7;
+            const long long src = s_row[row];
+            a_src[i] = src >= 0 ? p.a_codes + src * p.k + piece * 16 : nullptr;
+            a_dst[i] = (((row >> 4) * 2 + (piece >> 2)) * 64 + (piece & 3) * 16 + (row & 15)) * 16;
+        }
+        const long long my_row = tid < 128 ? s_row[tid] : -1;
+        const uint8_t* as_src = my_row >= 0 ? p.a_scales + my_row * (p.k / p.act_block) : nullptr;
+        // weight row tiles of this wave: FC1 routed: up tiles then gate tiles; FC1 shared: gate tiles then up tiles
+        int ntile[4];
+#pragma unroll
+        for (int j = 0; j < 4; ++j) {
+            if (FC1) ntile[j] = (j >> 1) * (p.inter / 16) + (ng * 128 + wave * 32) / 16 + (j & 1);
+            else ntile[j] = (ng * 256 + wave * 64) / 16 + j;
+        }
+        auto load_a = [&](int ks, u4v (&ra)[4], uint32_t& rs) {
+#pragma unroll
+            for (int i = 0; i < 4; ++i) ra[i] = a_src[i] ? *reinterpret_cast<const u4v*>(a_src[i] + (size_t)ks * 128) : u4v{0, 0, 0, 0};
+            rs = 0x7f7f7f7fu;
+            if (as_src) {
+                if (p.act_block == 32) rs = *reinterpret_cast<const uint32_t*>(as_src + ks * 4);
+                else rs = 0x01010101u * as_src[ks];
+            }
+        };
+        auto store_a = [&](int stage, const u4v (&ra)[4], uint32_t rs) {
+#pragma unroll
+            for (int i = 0; i < 4; ++i) *reinterpret_cast<u4v*>(&s_a[stage][a_dst[i]]) = ra[i];
+            if (tid < 128) s_as[stage][tid] = rs;
+        };
+        auto load_b = [&](int ks, BFrag<FP8> (&b)[4], uint32_t (&sb)[4]) {
+#pragma unroll
+            for (int j = 0; j < 4; ++j) {
+                if constexpr (FP8) {
+                    const u4v* src = reinterpret_cast<const u4v*>(w) + (((size_t)ntile[j] * ksteps + ks) * 2) * 64 + lane;
+                    b[j].lo = tf_stream_load(src);
+                    b[j].hi = tf_stream_load(src + 64);
+                    sb[j] = ws[(size_t)((ntile[j] * 16 + r16) / p.bn) * (p.k / p.bk) + (ks * 128 + 32 * g) / p.bk];
+                } else {
+                    b[j].lo = tf_stream_load(reinterpret_cast<const u4v*>(w) + ((size_t)ntile[j] * ksteps + ks) * 64 + lane);
+                    if ((ks & 3) == 0)
+                        sb[j] = __builtin_nontemporal_load(reinterpret_cast<const uint32_t*>(ws) + ((size_t)ntile[j] * (p.k / 512) + ks / 4) * 64 + lane);
+                }
+            }
+        };
+        v4f acc[8][4];
+#pragma unroll
+        for (int f = 0; f < 8; ++f)
+#pragma unroll
+            for (int j = 0; j < 4; ++j) acc[f][j] = v4f{0.f, 0.f, 0.f, 0.f};
+        const int frags = (valid + 15) >> 4;
+
+        u4v ra[4];
+        uint32_t rs;
+        BFrag<FP8> b[4], bn[4];
+        uint32_t sb[4] = {0, 0, 0, 0};
+        load_a(0, ra, rs);
+        load_b(0, b, sb);
+        store_a(0, ra, rs);
+        __syncthreads();
+        for (int ks = 0; ks < ksteps; ++ks) {
+            const int stage = ks & 1;
+            uint32_t sbn[4] = {sb[0], sb[1], sb[2], sb[3]};
+            if (ks + 1 < ksteps) { load_a(ks + 1, ra, rs); load_b(ks + 1, bn, sbn); }
+#pragma unroll
+            for (int f = 0; f < 8; ++f) {
+                if (f < frags) {
+                    const u4v lo = *reinterpret_cast<const u4v*>(&s_a[stage][((f * 2) * 64 + lane) * 16]);
+                    const u4v hi = *reinterpret_cast<const u4v*>(&s_a[stage][((f * 2 + 1) * 64 + lane) * 16]);
+                    const v8i av = v8i{(int)lo[0], (int)lo[1], (int)lo[2], (int)lo[3], (int)hi[0], (int)hi[1], (int)hi[2], (int)hi[3]};
+                    const int sa = (int)((s_as[stage][f * 16 + r16] >> (8 * g)) & 0xffu);
+#pragma unroll
+                    for (int j = 0; j < 4; ++j) {
+                        v8i bv;
+                        if constexpr (FP8) bv = v8i{(int)b[j].lo[0], (int)b[j].lo[1], (int)b[j].lo[2], (int)b[j].lo[3], (int)b[j].hi[0],
+                                                    (int)b[j].hi[1], (int)b[j].hi[2], (int)b[j].hi[3]};
+                        else bv = v8i{(int)b[j].lo[0], (int)b[j].lo[1], (int)b[j].lo[2], (int)b[j].lo[3], 0, 0, 0, 0};
+                        if constexpr (FP8) {
+                            acc[f][j] = __builtin_amdgcn_mfma_scale_f32_16x16x128_f8f6f4(av, bv, acc[f][j], 0, 0, 0, sa, 0, (int)sb[j]);
+                        } else {
+                            const int sbj = (int)(sb[j] >> (8 * (ks & 3)));
+                            acc[f][j] = __builtin_amdgcn_mfma_scale_f32_16x16x128_f8f6f4(av, bv, acc[f][j], 0, 4, 0, sa, 0, sbj);
+                        }
+                    }
+                }
+            }
+            if (ks + 1 < ksteps) {
+                store_a(stage ^ 1, ra, rs);
+#pragma unroll
+                for (int j = 0; j < 4; ++j) { b[j] = bn[j]; sb[j] = sbn[j]; }
+            }
+            __syncthreads();
+        }
+
+        // ---- epilogue --------------------------------------------------------------------------------------------------
+        if constexpr (FC1) {
+            const float hi_lim = tf_bf16(tf_to_bf16(p.limit)), lo_lim = tf_bf16(tf_to_bf16(-p.limit));
+            float hv[8][2][4];
+            float amax[8][4];
+#pragma unroll
+            for (int f = 0; f < 8; ++f)
+#pragma unroll
+                for (int i = 0; i < 4; ++i) {
+                    float m = 0.f;
+#pragma unroll
+                    for (int j = 0; j < 2; ++j) {
+                        float value;
+                        if (MODE == TF_GEMM_FC1_SHARED) {
+                            const uint16_t gb = tf_to_bf16(acc[f][j][i]), ub = tf_to_bf16(acc[f][2 + j][i]);
+                            if (p.tap != nullptr && f < frags) {
+                                const int row = 16 * f + 4 * g + i;
+                                if (row < valid) {
+                                    const size_t at = (size_t)(tile * 128 + row) * 2 * p.inter + ng * 128 + wave * 32 + j * 16 + r16;
+                                    p.tap[at] = gb;
+                                    p.tap[at + p.inter] = ub;
+                                }
+                            }
+                            const float gv = fminf(tf_bf16(gb), hi_lim), uv = fminf(fmaxf(tf_bf16(ub), lo_lim), hi_lim);
+                            value = __fmul_rn(gv / __fadd_rn(1.0f, tf_exp(-gv)), uv);
+                        } else {
+                            const float gv = fminf(acc[f][2 + j][i], p.limit), uv = fminf(p.limit, fmaxf(-p.limit, acc[f][j][i]));
+                            value = __fmul_rn(__fmul_rn(gv, tf_logistic(gv)), uv);
+                        }
+                        value = tf_bf16(tf_to_bf16(value));
+                        hv[f][j][i] = value;
+                        m = fmaxf(m, fabsf(value));
+                    }
+#pragma unroll
+                    for (int o = 1; o < 16; o <<= 1) m = fmaxf(m, __shfl_xor(m, o));
+                    amax[f][i] = m;
+                }
+            if (p.act_block == 128) {
+#pragma unroll
+                for (int f = 0; f < 8; ++f)
+#pragma unroll
+                    for (int i = 0; i < 4; ++i) if (r16 == 0) s_amax[wave][16 * f + 4 * g + i] = amax[f][i];
+                __syncthreads();
+#pragma unroll
+                for (int f = 0; f < 8; ++f)
+#pragma unroll
+                    for (int i = 0; i < 4; ++i) {
+                        const int row = 16 * f + 4 * g + i;
+                        amax[f][i] = fmaxf(fmaxf(s_amax[0][row], s_amax[1][row]), fmaxf(s_amax[2][row], s_amax[3][row]));
+                    }
+            }
+            const float min_amax = MODE == TF_GEMM_FC1_SHARED ? 1e-4f : 0.f;
+#pragma unroll
+            for (int f = 0; f < 8; ++f) {
+                if (f < frags) {
+#pragma unroll
+                    for (int i = 0; i < 4; ++i) {
+                        const int row = 16 * f + 4 * g + i;
+                        if (row < valid) {
+                            const uint32_t exponent = tf_block_exponent(min_amax > 0.f ? fmaxf(amax[f][i], min_amax) : amax[f][i]);
+                            const float inv = tf_block_inverse(exponent);
+                            const size_t phys = (size_t)tile * 128 + row;
+                            const int col = ng * 128 + wave * 32 + r16;
+#pragma unroll
+                            for (int j = 0; j < 2; ++j) {
+                                p.h_codes[phys * p.inter + col + 16 * j] = (uint8_t)tf_to_e4m3(__fmul_rn(hv[f][j][i], inv));
+                                if (p.h_bf16 != nullptr) p.h_bf16[phys * p.inter + col + 16 * j] = tf_to_bf16(hv[f][j][i]);
+                            }
+                            if (r16 == 0) {
+                                if (p.act_block == 32) p.h_scales[phys * (p.inter / 32) + ng * 4 + wave] = (uint8_t)exponent;
+                                else if (wave == 0) p.h_scales[phys * (p.inter / 128) + ng] = (uint8_t)exponent;
+                            }
+                        }
+                    }
+                }
+            }
+        } else {
+#pragma unroll
+            for (int f = 0; f < 8; ++f) {
+                if (f < frags) {
+#pragma unroll
+                    for (int i = 0; i < 4; ++i) {
+                        const int row = 16 * f + 4 * g + i;
+                        if (row < valid) {
+                            const int phys = tile * 128 + row;
+                            size_t out_row = (size_t)phys;
+                            float scale = 1.f;
+                            if (MODE == TF_GEMM_FC2_ROUTED) { out_row = (size_t)p.token_map[phys]; scale = p.token_weights[phys]; }
+#pragma unroll
+                            for (int j = 0; j < 4; ++j) {
+                                const float v = MODE == TF_GEMM_FC2_ROUTED ? __fmul_rn(acc[f][j][i], scale) : acc[f][j][i];
+                                p.out[out_row * p.hidden + ng * 256 + wave * 64 + 16 * j + r16] = tf_to_bf16(v);
+                            }
+                        }
+                    }
+                }
+            }
+        }
+    }
+}
+
+inline int tf_gemm_grid(int cus) { return cus >= 8 ? cus / 8 * 8 : 8; }
+inline bool tf_gemm_shape_ok(const GemmArgs& a, bool fc1) {
+    return a.k >= 512 && a.k % 512 == 0 && (a.act_block == 32 || a.act_block == 128) &&
+           (fc1 ? (a.inter >= 128 && a.inter % 128 == 0) : (a.hidden >= 256 && a.hidden % 256 == 0));
+}
+inline int tf_launch_fc1_gemm(const GemmArgs& a, int cus, hipStream_t s) {
+    if (!tf_gemm_shape_ok(a, true)) return -4;
+    tf_gemm<false, TF_GEMM_FC1_ROUTED><<<tf_gemm_grid(cus), 256, 0, s>>>(a);
+    return (int)hipGetLastError();
+}
+inline int tf_launch_fc2_gemm(const GemmArgs& a, int cus, hipStream_t s) {
+    if (!tf_gemm_shape_ok(a, false)) return -4;
+    tf_gemm<false, TF_GEMM_FC2_ROUTED><<<tf_gemm_grid(cus), 256, 0, s>>>(a);
+    return (int)hipGetLastError();
+}
+inline int tf_launch_dense_gemm(const GemmArgs& a, int cus, hipStream_t s) {
+    if (!tf_gemm_shape_ok(a, false)) return -4;
+    tf_gemm<true, TF_GEMM_DENSE><<<tf_gemm_grid(cus), 256, 0, s>>>(a);
+    return (int)hipGetLastError();
+}
+inline int tf_launch_shared_fc1_gemm(const GemmArgs& a, int cus, hipStream_t s) {
+    if (!tf_gemm_shape_ok(a, true)) return -4;
+    tf_gemm<true, TF_GEMM_FC1_SHARED><<<tf_gemm_grid(cus), 256, 0, s>>>(a);
+    return (int)hipGetLastError();
+}
+
+// Gate product for many rows: logits[rows][experts] = x . w^T, BF16 inputs, FP32 accumulate on the matrix cores
+// (v_mfma_f32_32x32x16_bf16).  One wave per 32 x 32 output tile; grid (ceil(rows / 64), experts / 32), block 128: waves
+// (0, 1) take the block's two row halves of expert tile 2 y, waves (2, 3) of tile 2 y + 1 ... here: wave w -> row half
+// w & 1, expert tile blockIdx.y * 2 + (w >> 1)?  No: blockIdx.y indexes 32-expert tiles; waves 0..1 = row halves, and the
+// block covers 64 rows x 32 experts with its first two waves (the other two split K and add through LDS).
+typedef __bf16 bf16x8 __attribute__((ext_vector_type(8)));
+typedef float v16f __attribute__((ext_vector_type(16)));
 extern "C" __global__ void __launch_bounds__(128) ca_router_logits_mfma(const uint16_t* x, const uint16_t* w, float* out, int rows,
                                                                         int hidden, int experts) {
-    // placeholder: scalar dot products, one thread per (row, expert) pair of the block's 64 x 32 tile
-    for (int i = threadIdx.x; i < 64 * 32; i += blockDim.x) {
-        const int row = blockIdx.x * 64 + i / 32, e = blockIdx.y * 32 + i % 32;
-        if (row >= rows || e >= experts) continue;
-        float acc = 0.f;
-        for (int k = 0; k < hidden; ++k) acc = __fmaf_rn(tf_bf16(x[(size_t)row * hidden + k]), tf_bf16(w[(size_t)e * hidden + k]), acc);
-        out[(size_t)row * experts + e] = acc;
+    __shared__ float s_part[2][32 * 32];
+    const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6, half = wave & 1, kpart = wave >> 1;
+    const int row = blockIdx.x * 64 + half * 32 + (lane & 31), e = blockIdx.y * 32 + (lane & 31);
+    const int kg = lane >> 5;                                 // lane group: k = 8 kg .. 8 kg + 7 of each 16-wide step
+    v16f acc;
+#pragma unroll
+    for (int i = 0; i < 16; ++i) acc[i] = 0.f;
+    const int k_begin = kpart * (hidden / 2), k_end = k_begin + hidden / 2;
+    const bool row_ok = row < rows;
+    for (int k = k_begin; k < k_end; k += 16) {
+        u4v av = {0, 0, 0, 0};
+        if (row_ok) av = *reinterpret_cast<const u4v*>(x + (size_t)row * hidden + k + 8 * kg);
+        const u4v bv = *reinterpret_cast<const u4v*>(w + (size_t)e * hidden + k + 8 * kg);
+        acc = __builtin_amdgcn_mfma_f32_32x32x16_bf16(__builtin_bit_cast(bf16x8, av), __builtin_bit_cast(bf16x8, bv), acc, 0, 0, 0);
+    }
+    if (kpart == 1) {
+#pragma unroll
+        for (int i = 0; i < 16; ++i) s_part[half][i * 64 + lane] = acc[i];
+    }
+    __syncthreads();
+    if (kpart == 0) {
+#pragma unroll
+        for (int i = 0; i < 16; ++i) {
+            const int m = 8 * (i >> 2) + 4 * (lane >> 5) + (i & 3);          // D[m][n = lane % 32]
+            const int out_row = blockIdx.x * 64 + half * 32 + m;
+            if (out_row < rows) out[(size_t)out_row * experts + blockIdx.y * 32 + (lane & 31)] = __fadd_rn(acc[i], s_part[half][i * 64 + lane]);
+        }
     }
 }
