@@ -106,6 +106,7 @@ class GpuLayer:
         self.live = z((1,), torch.int32)
         self.tokens = z((rows,), torch.int64)
         self.padding = torch.full((rows,), -1, dtype=torch.int32, device=d)
+        self.sync = z((64,), torch.int32)
 
     def _compact(self, src, kernel, n, k, unit_bytes, unit_elems, extra=None):
         src = src.contiguous()
@@ -119,7 +120,7 @@ class GpuLayer:
     def close(self):
         self.lib.ca_primitives_close(ctypes.c_void_p(self.ctx))
 
-    def run(self, x, tokens=None, live=None, padding=None, stream=0, fuse_route=None):
+    def run(self, x, tokens=None, live=None, padding=None, stream=0, fuse_route=None, fuse_gate=False):
         g, rows = self.g, self.rows
         K = g.topk
         self.x = x.to(self.dev).contiguous()
@@ -131,8 +132,10 @@ class GpuLayer:
             self.padding.copy_(torch.as_tensor(padding, dtype=torch.int32))
         torch.cuda.synchronize()
         sp = ctypes.c_void_p(stream)
+        fuse = rows * K <= 1024 if fuse_route is None else fuse_route
+        fuse_gate = fuse_gate and fuse and rows <= 16
         for off in range(0, rows, 16):
-            if rows > 16 and rows > STREAM_MAX_ROWS:
+            if fuse_gate or (rows > 16 and rows > STREAM_MAX_ROWS):
                 break
             n = min(16, rows - off)
             st = self.lib.ca_router_logits(n, ctypes.c_void_p(self.x.data_ptr() + off * g.hidden * 2), native.ptr(self.gate_w),
@@ -141,14 +144,13 @@ class GpuLayer:
         if rows > STREAM_MAX_ROWS:
             st = self.lib.ca_router_logits_wide(rows, native.ptr(self.x), native.ptr(self.gate_w), native.ptr(self.logits), sp)
             assert st == 0, st
-        fuse = rows * K <= 1024 if fuse_route is None else fuse_route
         dyn = [self.x, self.ids, self.weights, self.xq, self.xs, self.xq_min, self.xs_min, self.h, self.hq, self.hs,
                self.task_expert, self.task_valid, self.tile_base, self.token_map, self.token_weights, self.w13, self.s13,
                self.w2, self.s2, self.route_out, self.plan_scratch]
         scalars = [rows, rows, self.max_tiles * self.tile_m, self.max_tiles, self.tile_m, 1]
         if fuse:
             st = native.primitives_launch(self.ctx, 1, dyn + [self.logits, self.bias, self.bias_alt, self.tokens, self.live,
-                                                             self.padding if use_padding else None], scalars + [rows], stream)
+                                                             self.padding if use_padding else None, self.gate_w if fuse_gate else None, self.sync], scalars + [rows], stream)
         else:
             blocks = (rows + 15) // 16
             native.launch("ca_route_topk", blocks, 1024,

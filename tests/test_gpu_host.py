@@ -13,14 +13,15 @@ pytestmark = pytest.mark.gpu
 host = pkg.host
 
 
-@pytest.mark.parametrize("overlap,sum_shared,route_front", [(True, True, True), (False, False, False), (False, True, True), (True, False, False)])
-def test_c1_schedules(overlap, sum_shared, route_front):
+@pytest.mark.parametrize("overlap,sum_shared,route_front,fold", [(True, True, True, False), (False, False, False, False), (False, True, True, False),
+                                                                  (True, False, False, False), (False, True, True, True), (True, True, False, True)])
+def test_c1_schedules(overlap, sum_shared, route_front, fold):
     g, ops, x, rows = make("c1", "benchmark", "cpu")
-    layer = host.Layer(g, ops, rows, overlap=overlap, sum_shared=sum_shared, route_front=route_front)
+    layer = host.Layer(g, ops, rows, overlap=overlap, sum_shared=sum_shared, route_front=route_front, fold_shared=fold)
     layer.set_tokens()
     layer.run(x.cuda())
     taps = layer.taps()
-    if overlap:   # the branch quantized the input itself; the routed front-end emitted no shared-flavour codes
+    if overlap and not fold:   # the branch quantized the input itself; the routed front-end emitted no shared-flavour codes
         taps["xq_min"], taps["xs_min"] = oracle.quantize_rows(x.numpy().view(np.uint16), g.act_block, 1e-4)
     check_layer(g, ops, x, taps)
     layer.close()
@@ -63,7 +64,6 @@ def test_graph_replay_matches_eager_and_oracle(config):
     for which in (0, 1, 0):       # replays with other work between them must not see stale scratch
         layer.time([graphs[which]], 0, 1)
         taps = layer.taps()
-        taps["xq_min"], taps["xs_min"] = oracle.quantize_rows(xs[which].cpu().numpy().view(np.uint16), g.act_block, 1e-4)
         check_layer(g, ops, xs[which], taps)
         layer.run(xs[1 - which])
     layer.close()

@@ -106,6 +106,16 @@ def test_c1_reference_mode_live_padding_and_image_token():
     layer.close()
 
 
+def test_gate_product_inside_the_front_end():
+    g, ops, x, rows = make("c1", "benchmark", "cpu")
+    layer = GpuLayer(g, ops, rows)
+    taps = layer.run(x, fuse_gate=True)
+    check_layer(g, ops, x, taps)
+    taps = layer.run(synth.activations("c1-third", rows, g.hidden), fuse_gate=True)      # the sync word was left at zero
+    check_layer(g, ops, synth.activations("c1-third", rows, g.hidden), taps)
+    layer.close()
+
+
 def test_zero_input_gives_zero_output():
     # known answer recoverable from the reference (runtime/kernels/ffn-global-v1/index.json, case "zero": the output
     # digest is the digest of all-zero bytes)

@@ -13,7 +13,7 @@ namespace {
 
 ca_geometry g_geometry = {5120, 384, 6, 576, 576, 1, 1.5f, 32, 32, 32, 129264, 10.f};   // src/ffn.rs:65-66, 245-258
 
-bool supported_k(int k) { return k == 512 || k == 1024 || k == 2048 || k == 4096 || k == 8192; }
+bool supported_k(int k) { return k == 512 || k == 1024 || k == 2048 || k == 4096; }
 int check_geometry(const ca_geometry& g) {
     if (g.hidden <= 0 || g.hidden % 512 || g.experts <= 0 || g.experts > 512 || g.topk <= 0 || g.topk > 8 ||
         g.topk > g.experts || g.intermediate <= 0 || g.intermediate % 512 || g.shared_intermediate <= 0 ||
@@ -31,26 +31,32 @@ struct Context {
     int stream_wgs;    // persistent workgroups of the streaming kernels
 };
 
-template <bool FP8>
-int launch_fc1_stream(const StreamArgs& a, int wgs, hipStream_t s) {
-    switch (a.k) {
-        case 512: tf_fc1_stream<FP8, 1><<<wgs, 256, 0, s>>>(a); break;
-        case 1024: tf_fc1_stream<FP8, 2><<<wgs, 256, 0, s>>>(a); break;
-        case 2048: tf_fc1_stream<FP8, 4><<<wgs, 256, 0, s>>>(a); break;
-        case 4096: tf_fc1_stream<FP8, 8><<<wgs, 256, 0, s>>>(a); break;
-        case 8192: tf_fc1_stream<FP8, 16><<<wgs, 256, 0, s>>>(a); break;
+// Phase launches of the streaming kernels; either operand set may be absent (w == nullptr).
+int launch_phase1(const StreamArgs& routed, const StreamArgs& shared, int wgs, hipStream_t s) {
+    const int k = routed.w ? routed.k : shared.k;
+    if (routed.w && shared.w && routed.k != shared.k) return -4;
+    switch (k) {
+        case 512: tf_phase1_stream<1, 1><<<wgs, 256, 0, s>>>(routed, shared); break;
+        case 1024: tf_phase1_stream<2, 2><<<wgs, 256, 0, s>>>(routed, shared); break;
+        case 2048: tf_phase1_stream<4, 4><<<wgs, 256, 0, s>>>(routed, shared); break;
+        case 4096: tf_phase1_stream<8, 8><<<wgs, 256, 0, s>>>(routed, shared); break;
         default: return -4;
     }
     return launch_status();
 }
-template <bool FP8>
-int launch_fc2_stream(const StreamArgs& a, int wgs, hipStream_t s) {
-    const size_t lds = 16 * (size_t)a.k + 16 * (size_t)(a.k / a.act_block);
-    switch (a.k) {
-        case 512: tf_fc2_stream<FP8, 1><<<wgs, 256, lds, s>>>(a); break;
-        case 1024: tf_fc2_stream<FP8, 2><<<wgs, 256, lds, s>>>(a); break;
-        case 2048: tf_fc2_stream<FP8, 4><<<wgs, 256, lds, s>>>(a); break;
-        case 4096: tf_fc2_stream<FP8, 8><<<wgs, 256, lds, s>>>(a); break;
+int launch_phase2(const StreamArgs& routed, const StreamArgs& shared, int wgs, hipStream_t s) {
+    if (routed.w && shared.w && routed.k != shared.k) {       // different intermediate sizes: one launch each
+        StreamArgs none{};
+        const int status = launch_phase2(routed, none, wgs, s);
+        return status ? status : launch_phase2(none, shared, wgs, s);
+    }
+    const int k = routed.w ? routed.k : shared.k, block = routed.w ? routed.act_block : shared.act_block;
+    const size_t lds = 16 * (size_t)k + 16 * (size_t)(k / block);
+    switch (k) {
+        case 512: tf_phase2_stream<1, 1><<<wgs, 256, lds, s>>>(routed, shared); break;
+        case 1024: tf_phase2_stream<2, 2><<<wgs, 256, lds, s>>>(routed, shared); break;
+        case 2048: tf_phase2_stream<4, 4><<<wgs, 256, lds, s>>>(routed, shared); break;
+        case 4096: tf_phase2_stream<8, 8><<<wgs, 256, lds, s>>>(routed, shared); break;
         default: return -4;
     }
     return launch_status();
@@ -61,12 +67,28 @@ enum DynPtr {
     P_A, P_IDS, P_WEIGHTS, P_PACKED, P_SCALES, P_PACKED_MIN, P_SCALES_MIN, P_INTER, P_INTER_CODES, P_INTER_SCALES,
     P_TASK_EXPERT, P_TASK_VALID, P_TILE_BASE, P_TOKEN_MAP, P_TOKEN_WEIGHTS, P_W13, P_S13, P_W2, P_S2, P_SCATTER,
     P_PLAN_SCRATCH, P_DYN_COUNT,
-    P_LOGITS = P_DYN_COUNT, P_BIAS, P_BIAS_ALT, P_TOKENS, P_LIVE, P_PADDING, P_ROUTE_COUNT
+    P_LOGITS = P_DYN_COUNT, P_BIAS, P_BIAS_ALT, P_TOKENS, P_LIVE, P_PADDING, P_GATE_W, P_SYNC, P_ROUTE_COUNT
 };
 enum DynScalar { S_TOKENS, S_MAX_ROWS, S_ROWS_PADDED, S_MAX_TILES, S_TILE_M, S_GROUPS, S_DYN_COUNT, S_OWNER_ROWS = S_DYN_COUNT, S_ROUTE_COUNT };
 
-// phases: 1 front-end (plan + quantize), 2 FC1 + SwiGLU, 4 FC2
-int launch_dynamic(const Context& c, bool route, const uint64_t* p, const int32_t* sc, hipStream_t s, int phases = 7) {
+enum SharedPtr { H_A, H_AS, H_W13, H_S13, H_W2, H_S2, H_ACT, H_ACT_CODES, H_ACT_SCALES, H_UP_TAP, H_OUT, H_COUNT };
+// Streaming operands of the shared expert's two projections (few rows).
+void shared_stream_args(const Context& c, const uint64_t* p, int m, StreamArgs& a, StreamArgs& b) {
+    const ca_geometry& g = c.g;
+    a = StreamArgs{};
+    a.a_codes = (const uint8_t*)p[H_A]; a.a_scales = (const uint8_t*)p[H_AS];
+    a.w = (const uint8_t*)p[H_W13]; a.ws = (const uint8_t*)p[H_S13]; a.bn = g.shared_bn; a.bk = g.shared_bk;
+    a.dense_rows = m; a.k = g.hidden; a.inter = g.shared_intermediate; a.hidden = g.hidden; a.act_block = g.act_block;
+    a.limit = g.swiglu_limit; a.out = (uint16_t*)p[H_ACT]; a.tap = (uint16_t*)p[H_UP_TAP];
+    b = a;
+    b.a_codes = nullptr; b.a_scales = nullptr; b.a_bf16 = (const uint16_t*)p[H_ACT];
+    b.q_codes = (uint8_t*)p[H_ACT_CODES]; b.q_scales = (uint8_t*)p[H_ACT_SCALES]; b.min_amax = 1e-4f;
+    b.w = (const uint8_t*)p[H_W2]; b.ws = (const uint8_t*)p[H_S2]; b.k = g.shared_intermediate; b.out = (uint16_t*)p[H_OUT];
+    b.tap = nullptr;
+}
+// phases: 1 front-end (plan + quantize), 2 FC1 + SwiGLU, 4 FC2.  `sh` (may be null): the shared expert's operands (SharedPtr
+// order, its input codes taken from the front-end's shared-flavour output), folded into the same phase launches.
+int launch_dynamic(const Context& c, bool route, const uint64_t* p, const int32_t* sc, hipStream_t s, int phases = 7, const uint64_t* sh = nullptr) {
     const ca_geometry& g = c.g;
     const int rows = sc[S_TOKENS], tile_m = sc[S_TILE_M], groups = sc[S_GROUPS], max_tiles = sc[S_MAX_TILES];
     if (rows < 1 || rows > sc[S_MAX_ROWS] || groups < 1 || max_tiles < 1 || sc[S_ROWS_PADDED] != max_tiles * tile_m) return -1;
@@ -90,14 +112,19 @@ int launch_dynamic(const Context& c, bool route, const uint64_t* p, const int32_
             const int owner = sc[S_OWNER_ROWS];
             if (owner < rows || (long long)owner * g.topk > 1024) return -1;
             for (int i = P_LOGITS; i <= P_LIVE; ++i) if (!p[i] && i != P_BIAS_ALT && i != P_TOKENS) return -1;
-            ca_moe_route_frontend<<<quant_blocks + 1, 1024, 0, s>>>(
+            // with the gate weight (and a zeroed sync word) the gate product runs inside this launch too (owner rows <= 16)
+            const bool gate = p[P_GATE_W] != 0;
+            if (gate && (!p[P_SYNC] || owner > 16 || g.hidden > 8192)) return -1;
+            const int logit_blocks = gate ? (g.experts + 7) / 8 : 0;
+            ca_moe_route_frontend<<<quant_blocks + 1 + logit_blocks, 512, 0, s>>>(
                 x, ids, weights, (uint8_t*)p[P_PACKED], (uint8_t*)p[P_SCALES], (int32_t*)p[P_TOKEN_MAP], (float*)p[P_TOKEN_WEIGHTS],
-                (int32_t*)p[P_TASK_EXPERT], (int32_t*)p[P_TASK_VALID], (int32_t*)p[P_TILE_BASE], (const float*)p[P_LOGITS],
+                (int32_t*)p[P_TASK_EXPERT], (int32_t*)p[P_TASK_VALID], (int32_t*)p[P_TILE_BASE], (float*)p[P_LOGITS],
                 (const float*)p[P_BIAS], (const float*)p[P_BIAS_ALT], (const long long*)p[P_TOKENS], (const int32_t*)p[P_LIVE],
                 (const int32_t*)p[P_PADDING], rows, g.topk, g.experts, g.hidden, groups, tile_m, owner, g.act_block,
-                (uint8_t*)p[P_PACKED_MIN], (uint8_t*)p[P_SCALES_MIN], g.scoring, g.route_scale, (long long)g.alt_token);
+                (uint8_t*)p[P_PACKED_MIN], (uint8_t*)p[P_SCALES_MIN], g.scoring, g.route_scale, (long long)g.alt_token,
+                (const uint16_t*)p[P_GATE_W], (uint32_t*)p[P_SYNC], logit_blocks);
         } else {
-            ca_moe_frontend<<<quant_blocks, 1024, 0, s>>>(
+            ca_moe_frontend<<<quant_blocks, 512, 0, s>>>(
                 x, ids, weights, (uint8_t*)p[P_PACKED], (uint8_t*)p[P_SCALES], (int32_t*)p[P_TOKEN_MAP], (float*)p[P_TOKEN_WEIGHTS],
                 (int32_t*)p[P_TASK_EXPERT], (int32_t*)p[P_TASK_VALID], (int32_t*)p[P_TILE_BASE], rows, g.topk, g.experts, g.hidden,
                 groups, tile_m, g.act_block, (uint8_t*)p[P_PACKED_MIN], (uint8_t*)p[P_SCALES_MIN]);
@@ -135,8 +162,14 @@ int launch_dynamic(const Context& c, bool route, const uint64_t* p, const int32_
         a.experts = g.experts; a.groups = groups; a.topk = g.topk;
         a.k = g.hidden; a.inter = g.intermediate; a.hidden = g.hidden; a.act_block = g.act_block; a.limit = g.swiglu_limit;
         a.out = (uint16_t*)p[P_INTER];
+        StreamArgs sa{}, sb{};
+        if (sh) {
+            for (int i = 0; i < H_COUNT; ++i) if (!sh[i] && i != H_UP_TAP && i != H_ACT_CODES && i != H_ACT_SCALES) return -1;
+            if (!supported_k(g.shared_intermediate)) return -4;
+            shared_stream_args(c, sh, rows, sa, sb);
+        }
         if (phases & 2) {
-            status = launch_fc1_stream<false>(a, c.stream_wgs, s);
+            status = launch_phase1(a, sa, c.stream_wgs, s);
             if (status) return status;
         }
         if (!(phases & 4)) return 0;
@@ -146,8 +179,9 @@ int launch_dynamic(const Context& c, bool route, const uint64_t* p, const int32_
         b.w = (const uint8_t*)p[P_W2]; b.ws = (const uint8_t*)p[P_S2];
         b.w_expert_stride = w2_stride; b.ws_expert_stride = s2_stride;
         b.k = g.intermediate; b.out = (uint16_t*)p[P_SCATTER];
-        return launch_fc2_stream<false>(b, c.stream_wgs, s);
+        return launch_phase2(b, sb, c.stream_wgs, s);
     }
+    if (sh) return -4;   // many rows: the shared expert runs through its own entry
     if (!p[P_INTER_CODES] || !p[P_INTER_SCALES]) return -1;
     GemmArgs a{};
     a.a_codes = (const uint8_t*)p[P_PACKED]; a.a_scales = (const uint8_t*)p[P_SCALES];
@@ -205,7 +239,7 @@ int launch_dense(const Context& c, const uint64_t* p, const int32_t* sc, hipStre
         a.a_codes = (const uint8_t*)p[0]; a.a_scales = (const uint8_t*)p[1];
         a.w = (const uint8_t*)p[2]; a.ws = (const uint8_t*)p[3]; a.bn = c.g.shared_bn; a.bk = c.g.shared_bk;
         a.dense_rows = m; a.k = k; a.hidden = n; a.act_block = c.g.act_block; a.out = (uint16_t*)p[4];
-        return launch_fc2_stream<true>(a, c.stream_wgs, s);
+        return -4;   // few-row dense products run inside ffn.shared_expert
     }
     GemmArgs a{};
     a.a_codes = (const uint8_t*)p[0]; a.a_scales = (const uint8_t*)p[1];
@@ -214,26 +248,16 @@ int launch_dense(const Context& c, const uint64_t* p, const int32_t* sc, hipStre
     return tf_launch_dense_gemm(a, c.cus, s);
 }
 // ---- entry 5: ffn.shared_expert (up + clipped SwiGLU + requant + down, from the quantized input) ---------------------
-enum SharedPtr { H_A, H_AS, H_W13, H_S13, H_W2, H_S2, H_ACT, H_ACT_CODES, H_ACT_SCALES, H_UP_TAP, H_OUT, H_COUNT };
 int launch_shared(const Context& c, const uint64_t* p, const int32_t* sc, hipStream_t s) {
     const ca_geometry& g = c.g;
     const int m = sc[0];
     for (int i = 0; i < H_COUNT; ++i) if (!p[i] && i != H_UP_TAP && i != H_ACT_CODES && i != H_ACT_SCALES) return -1;
     if (m < 1 || !supported_k(g.hidden) || !supported_k(g.shared_intermediate)) return -4;
     if (m <= TF_STREAM_MAX_ROWS) {
-        StreamArgs a{};
-        a.a_codes = (const uint8_t*)p[H_A]; a.a_scales = (const uint8_t*)p[H_AS];
-        a.w = (const uint8_t*)p[H_W13]; a.ws = (const uint8_t*)p[H_S13]; a.bn = g.shared_bn; a.bk = g.shared_bk;
-        a.dense_rows = m; a.k = g.hidden; a.inter = g.shared_intermediate; a.hidden = g.hidden; a.act_block = g.act_block;
-        a.limit = g.swiglu_limit; a.out = (uint16_t*)p[H_ACT]; a.tap = (uint16_t*)p[H_UP_TAP];
-        int status = launch_fc1_stream<true>(a, c.stream_wgs, s);
-        if (status) return status;
-        StreamArgs b = a;
-        b.a_codes = nullptr; b.a_scales = nullptr; b.a_bf16 = (const uint16_t*)p[H_ACT];
-        b.q_codes = (uint8_t*)p[H_ACT_CODES]; b.q_scales = (uint8_t*)p[H_ACT_SCALES]; b.min_amax = 1e-4f;
-        b.w = (const uint8_t*)p[H_W2]; b.ws = (const uint8_t*)p[H_S2]; b.k = g.shared_intermediate; b.out = (uint16_t*)p[H_OUT];
-        b.tap = nullptr;
-        return launch_fc2_stream<true>(b, c.stream_wgs, s);
+        StreamArgs a, b, none{};
+        shared_stream_args(c, p, m, a, b);
+        const int status = launch_phase1(none, a, c.stream_wgs, s);
+        return status ? status : launch_phase2(none, b, c.stream_wgs, s);
     }
     if (!p[H_ACT_CODES] || !p[H_ACT_SCALES]) return -1;
     GemmArgs a{};
@@ -262,6 +286,7 @@ const EntryShape kEntries[] = {
     {"moe.w4a8.phase1", P_DYN_COUNT, S_DYN_COUNT},
     {"moe.w4a8.phase2", P_DYN_COUNT, S_DYN_COUNT},
     {"moe.front_end", P_DYN_COUNT, S_DYN_COUNT},
+    {"ffn.experts_with_shared", P_ROUTE_COUNT + H_COUNT - 2, S_ROUTE_COUNT},
 };
 constexpr int kEntryCount = sizeof(kEntries) / sizeof(kEntries[0]);
 
@@ -305,9 +330,8 @@ int ca_router_logits(int rows, const void* x, const void* w, void* out, void* st
 int ca_router_logits_wide(int rows, const void* x, const void* w, void* out, void* stream) {
     if (rows < 1 || !x || !w || !out) return -1;
     if (rows <= 16) return ca_router_logits(rows, x, w, out, stream);
-    if (g_geometry.experts % 32 || g_geometry.hidden % 64) return -4;
-    const dim3 grid((rows + 63) / 64, g_geometry.experts / 32);
-    ca_router_logits_mfma<<<grid, 128, 0, (hipStream_t)stream>>>((const uint16_t*)x, (const uint16_t*)w, (float*)out, rows,
+    const dim3 grid((rows + 63) / 64, (g_geometry.experts + 31) / 32);
+    ca_router_logits_mfma<<<grid, 256, 0, (hipStream_t)stream>>>((const uint16_t*)x, (const uint16_t*)w, (float*)out, rows,
                                                                  g_geometry.hidden, g_geometry.experts);
     return launch_status();
 }
@@ -378,6 +402,13 @@ int32_t ca_primitives_launch(void* context, int32_t index, const uint64_t* point
         case 6: return launch_dynamic(c, false, pointers, scalars, s, 2);
         case 7: return launch_dynamic(c, false, pointers, scalars, s, 4);
         case 8: return launch_dynamic(c, false, pointers, scalars, s, 1);
+        case 9: {   // routed experts (top-k inside the front-end when logits are given) + shared expert in the same launches
+            uint64_t sh[H_COUNT];
+            sh[H_A] = pointers[P_PACKED_MIN]; sh[H_AS] = pointers[P_SCALES_MIN];
+            for (int i = 2; i < H_COUNT; ++i) sh[i] = pointers[P_ROUTE_COUNT + i - 2];
+            if (!sh[H_A] || !sh[H_AS]) return -1;
+            return launch_dynamic(c, pointers[P_LOGITS] != 0, pointers, scalars, s, 7, sh);
+        }
         default: return -3;
     }
 }

@@ -311,13 +311,11 @@ inline int tf_launch_shared_fc1_gemm(const GemmArgs& a, int cus, hipStream_t s) 
 }
 
 // Gate product for many rows: logits[rows][experts] = x . w^T, BF16 inputs, FP32 accumulate on the matrix cores
-// (v_mfma_f32_32x32x16_bf16).  One wave per 32 x 32 output tile; grid (ceil(rows / 64), experts / 32), block 128: waves
-// (0, 1) take the block's two row halves of expert tile 2 y, waves (2, 3) of tile 2 y + 1 ... here: wave w -> row half
-// w & 1, expert tile blockIdx.y * 2 + (w >> 1)?  No: blockIdx.y indexes 32-expert tiles; waves 0..1 = row halves, and the
-// block covers 64 rows x 32 experts with its first two waves (the other two split K and add through LDS).
+// (v_mfma_f32_32x32x16_bf16).  grid (ceil(rows / 64), ceil(experts / 32)), block 256: wave w takes row half w & 1 of the
+// block's 64 rows and half w >> 1 of K; the two K halves of a tile are added through LDS (first half + second half).
 typedef __bf16 bf16x8 __attribute__((ext_vector_type(8)));
 typedef float v16f __attribute__((ext_vector_type(16)));
-extern "C" __global__ void __launch_bounds__(128) ca_router_logits_mfma(const uint16_t* x, const uint16_t* w, float* out, int rows,
+extern "C" __global__ void __launch_bounds__(256) ca_router_logits_mfma(const uint16_t* x, const uint16_t* w, float* out, int rows,
                                                                         int hidden, int experts) {
     __shared__ float s_part[2][32 * 32];
     const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6, half = wave & 1, kpart = wave >> 1;
@@ -331,7 +329,7 @@ extern "C" __global__ void __launch_bounds__(128) ca_router_logits_mfma(const ui
     for (int k = k_begin; k < k_end; k += 16) {
         u4v av = {0, 0, 0, 0};
         if (row_ok) av = *reinterpret_cast<const u4v*>(x + (size_t)row * hidden + k + 8 * kg);
-        const u4v bv = *reinterpret_cast<const u4v*>(w + (size_t)e * hidden + k + 8 * kg);
+        const u4v bv = *reinterpret_cast<const u4v*>(w + (size_t)min(e, experts - 1) * hidden + k + 8 * kg);
         acc = __builtin_amdgcn_mfma_f32_32x32x16_bf16(__builtin_bit_cast(bf16x8, av), __builtin_bit_cast(bf16x8, bv), acc, 0, 0, 0);
     }
     if (kpart == 1) {
@@ -344,7 +342,7 @@ extern "C" __global__ void __launch_bounds__(128) ca_router_logits_mfma(const ui
         for (int i = 0; i < 16; ++i) {
             const int m = 8 * (i >> 2) + 4 * (lane >> 5) + (i & 3);          // D[m][n = lane % 32]
             const int out_row = blockIdx.x * 64 + half * 32 + m;
-            if (out_row < rows) out[(size_t)out_row * experts + blockIdx.y * 32 + (lane & 31)] = __fadd_rn(acc[i], s_part[half][i * 64 + lane]);
+            if (out_row < rows && e < experts) out[(size_t)out_row * experts + e] = __fadd_rn(acc[i], s_part[half][i * 64 + lane]);
         }
     }
 }

@@ -55,90 +55,102 @@ __device__ __forceinline__ void tf_load_a(ATile<KS>& t, const uint8_t* codes, co
     }
 }
 
-// B operand of one 16-row weight tile for this wave's KS k-steps.
-template <int KS, bool FP8>
-struct BTile {
-    u4v lo[KS];
-    u4v hi[FP8 ? KS : 1];
-    uint32_t scale[(KS + 3) / 4];
+// One pipeline unit of streamed weights for this wave: N 16-byte loads a lane (N KiB a wave).
+//   FP4 (routed): TILES weight tiles of 16 rows, KS k-steps each: d[t * KS + s].
+//   FP8 (shared): TILES / 2 weight tiles, each k-step as two 16-byte planes: d[(t * KS + s) * 2 + half].
+// Scale bytes travel as one dword per tile and four k-steps (byte q = k-step 4 i + q of the wave's share).
+template <int TILES, int KS>
+struct Unit {
+    u4v d[TILES * KS];
+    uint32_t scale[TILES * ((KS + 3) / 4)];
 };
 // FP4: words [n/16][k/128][lane][16 B], scales [n/16][k/512][lane][4 B] (byte q of a word = k-step 4 kq + q).
-// FP8: bytes [n/16][k/128][half][lane][16 B]; scales row-major UE8M0 [n/bn][k/bk].
 // KS is 1, 2 or a multiple of 4, so a wave's k-steps never straddle a scale word.
-template <int KS, bool FP8>
-__device__ __forceinline__ void tf_load_b(BTile<KS, FP8>& b, const uint8_t* w, const uint8_t* scales, int ntile, int k,
-                                          int ks_first, int lane, int bn, int bk) {
-    if constexpr (FP8) {
-        const u4v* src = reinterpret_cast<const u4v*>(w) + (((size_t)ntile * (k / 128) + ks_first) * 2) * 64 + lane;
+template <int TILES, int KS>
+__device__ __forceinline__ void tf_load_fp4(Unit<TILES, KS>& u, const uint8_t* w, const uint8_t* scales, const int (&ntile)[TILES], int k,
+                                            int ks_first, int lane) {
+    constexpr int SW = (KS + 3) / 4;
 #pragma unroll
-        for (int s = 0; s < KS; ++s) {
-            b.lo[s] = tf_stream_load(src + (s * 2) * 64);
-            b.hi[s] = tf_stream_load(src + (s * 2 + 1) * 64);
-        }
-        const int row = ntile * 16 + (lane & 15), g = lane >> 4;
+    for (int t = 0; t < TILES; ++t) {
+        const u4v* src = reinterpret_cast<const u4v*>(w) + ((size_t)ntile[t] * (k / 128) + ks_first) * 64 + lane;
 #pragma unroll
-        for (int q = 0; q < (KS + 3) / 4; ++q) b.scale[q] = 0x7f7f7f7fu;
+        for (int s = 0; s < KS; ++s) u.d[t * KS + s] = tf_stream_load(src + s * 64);
+        const uint32_t* sc = reinterpret_cast<const uint32_t*>(scales) + ((size_t)ntile[t] * (k / 512) + ks_first / 4) * 64 + lane;
 #pragma unroll
-        for (int s = 0; s < KS; ++s) {
-            const uint32_t byte = scales[(size_t)(row / bn) * (k / bk) + ((ks_first + s) * 128 + 32 * g) / bk];
-            b.scale[s >> 2] = (b.scale[s >> 2] & ~(0xffu << (8 * (s & 3)))) | (byte << (8 * (s & 3)));
-        }
-    } else {
-        const u4v* src = reinterpret_cast<const u4v*>(w) + ((size_t)ntile * (k / 128) + ks_first) * 64 + lane;
-#pragma unroll
-        for (int s = 0; s < KS; ++s) b.lo[s] = tf_stream_load(src + s * 64);
-        const uint32_t* sc = reinterpret_cast<const uint32_t*>(scales) + ((size_t)ntile * (k / 512) + ks_first / 4) * 64 + lane;
-#pragma unroll
-        for (int q = 0; q < (KS + 3) / 4; ++q) b.scale[q] = __builtin_nontemporal_load(sc + q * 64) >> (8 * (ks_first & 3));
+        for (int q = 0; q < SW; ++q) u.scale[t * SW + q] = __builtin_nontemporal_load(sc + q * 64) >> (8 * (ks_first & 3));
     }
 }
-template <int KS, bool FP8>
-__device__ __forceinline__ v4f tf_dot_tile(const ATile<KS>& a, const BTile<KS, FP8>& b) {
+// FP8: bytes [n/16][k/128][half][lane][16 B]; scales row-major UE8M0 [n/bn][k/bk].  TILES counts 16-byte planes: tile = t / 2.
+template <int TILES, int KS>
+__device__ __forceinline__ void tf_load_fp8(Unit<TILES, KS>& u, const uint8_t* w, const uint8_t* scales, const int (&ntile)[TILES], int k,
+                                            int ks_first, int lane, int bn, int bk) {
+    constexpr int SW = (KS + 3) / 4;
+    const int g = lane >> 4;
+#pragma unroll
+    for (int t = 0; t < TILES / 2; ++t) {
+        const u4v* src = reinterpret_cast<const u4v*>(w) + (((size_t)ntile[t] * (k / 128) + ks_first) * 2) * 64 + lane;
+#pragma unroll
+        for (int s = 0; s < 2 * KS; ++s) u.d[t * 2 * KS + s] = tf_stream_load(src + s * 64);
+        const uint8_t* sc = scales + (size_t)((ntile[t] * 16 + (lane & 15)) / bn) * (k / bk);
+#pragma unroll
+        for (int q = 0; q < SW; ++q) {
+            uint32_t word = 0x7f7f7f7fu;
+#pragma unroll
+            for (int b = 0; b < 4; ++b)
+                if (4 * q + b < KS) word = (word & ~(0xffu << (8 * b))) | ((uint32_t)sc[((ks_first + 4 * q + b) * 128 + 32 * g) / bk] << (8 * b));
+            u.scale[t * SW + q] = word;
+        }
+    }
+}
+#define TF_MFMA4(A, B, C, FMT, S, SA, SB)                                              \
+    switch ((S) & 3) {                                                                 \
+        case 0: C = TF_MFMA(A, B, C, FMT, 0, SA, SB); break;                            \
+        case 1: C = TF_MFMA(A, B, C, FMT, 1, SA, SB); break;                            \
+        case 2: C = TF_MFMA(A, B, C, FMT, 2, SA, SB); break;                            \
+        default: C = TF_MFMA(A, B, C, FMT, 3, SA, SB); break;                           \
+    }
+// Product of the A tile with weight tile `t` of a unit over the wave's k-steps.
+template <bool FP8, int TILES, int KS>
+__device__ __forceinline__ v4f tf_dot_unit(const ATile<KS>& a, const Unit<TILES, KS>& u, int t) {
+    constexpr int SW = (KS + 3) / 4;
     v4f acc = {0.f, 0.f, 0.f, 0.f};
 #pragma unroll
     for (int s = 0; s < KS; ++s) {
-        v8i bv;
-        if constexpr (FP8) bv = v8i{(int)b.lo[s][0], (int)b.lo[s][1], (int)b.lo[s][2], (int)b.lo[s][3], (int)b.hi[s][0],
-                                    (int)b.hi[s][1], (int)b.hi[s][2], (int)b.hi[s][3]};
-        else bv = v8i{(int)b.lo[s][0], (int)b.lo[s][1], (int)b.lo[s][2], (int)b.lo[s][3], 0, 0, 0, 0};
-        const int sa = (int)a.scale[s >> 2], sb = (int)b.scale[s >> 2];
-        constexpr int F = FP8 ? 0 : 4;
-        switch (s & 3) {
-            case 0: acc = TF_MFMA(a.a[s], bv, acc, F, 0, sa, sb); break;
-            case 1: acc = TF_MFMA(a.a[s], bv, acc, F, 1, sa, sb); break;
-            case 2: acc = TF_MFMA(a.a[s], bv, acc, F, 2, sa, sb); break;
-            default: acc = TF_MFMA(a.a[s], bv, acc, F, 3, sa, sb); break;
+        const int sa = (int)a.scale[s >> 2], sb = (int)u.scale[t * SW + (s >> 2)];
+        if constexpr (FP8) {
+            const u4v lo = u.d[(t * KS + s) * 2], hi = u.d[(t * KS + s) * 2 + 1];
+            const v8i bv = v8i{(int)lo[0], (int)lo[1], (int)lo[2], (int)lo[3], (int)hi[0], (int)hi[1], (int)hi[2], (int)hi[3]};
+            TF_MFMA4(a.a[s], bv, acc, 0, s, sa, sb)
+        } else {
+            const u4v lo = u.d[t * KS + s];
+            const v8i bv = v8i{(int)lo[0], (int)lo[1], (int)lo[2], (int)lo[3], 0, 0, 0, 0};
+            TF_MFMA4(a.a[s], bv, acc, 4, s, sa, sb)
         }
     }
     return acc;
 }
 
-// Description of one streamed projection over a list of M tiles.
+// Operands of one streamed projection (routed: FP4 weights through the plan; dense: FP8 weights over all rows).
 struct StreamArgs {
-    // activations: E4M3 codes [rows][k] + scales, or (FC2) BF16 rows to quantize first
-    const uint8_t* a_codes;
+    const uint8_t* a_codes;          // FC1: E4M3 token codes [rows][k]
     const uint8_t* a_scales;
-    const uint16_t* a_bf16;          // FC2: BF16 intermediate rows [phys_row][k] (quantized in the prologue)
+    const uint16_t* a_bf16;          // FC2: BF16 intermediate rows [phys_row][k] (quantized in the tile prologue)
     uint8_t* q_codes;                // FC2: where the prologue stores the codes it used ([phys_row][k]), may be null
     uint8_t* q_scales;
     float min_amax;                  // quantizer flavour of the FC2 prologue
-    // weights
     const uint8_t* w;                // prepared weights, expert-major
     const uint8_t* ws;               // prepared scales (FP4) or row-major block scales (FP8)
     long long w_expert_stride, ws_expert_stride;
     int bn, bk;                      // FP8 weight scale block
-    // plan (routed) or null (dense: tile t covers rows 16 t ..)
-    const int32_t* expert_tile_base; // [experts + 1]; tiles = expert_tile_base[experts]
-    const int32_t* task_expert;      // [tile * groups]
+    const int32_t* expert_tile_base; // routed: [experts + 1]; tiles = expert_tile_base[experts]
+    const int32_t* task_expert;      // routed: [tile * groups]; null: dense (tile t covers rows 16 t ..)
     const int32_t* task_valid_rows;
     const int32_t* token_map;        // [tile * 16 + m] -> route index
     const float* token_weights;
     int experts, groups, topk;
-    int dense_rows;                  // dense: number of rows
-    // shapes
+    int dense_rows;
     int k, inter, hidden, act_block;
     float limit;
-    // outputs
     uint16_t* out;                   // FC1: BF16 intermediate [phys_row][inter]; FC2: BF16 [route or row][hidden]
     uint16_t* tap;                   // FC1 dense: BF16 projections [row][2 inter] before the activation, may be null
 };
@@ -156,43 +168,60 @@ __device__ __forceinline__ ItemRef tf_item(const StreamArgs& p, int item, int pe
     }
     return r;
 }
+__device__ __forceinline__ int tf_tiles(const StreamArgs& p) {
+    return p.task_expert != nullptr ? p.expert_tile_base[p.experts] : (p.dense_rows + 15) / 16;
+}
 
-// FC1 + SwiGLU.  Item = (tile, j): weight tiles j ("up" for routed, "gate" for shared) and inter / 16 + j of the
-// expert's [2 inter][k] matrix; output intermediate columns 16 j .. 16 j + 15 of the tile's rows.
+// FC1 + SwiGLU.  Item = (tile, j): weight tiles j and inter / 16 + j of the expert's [2 inter][k] matrix; output
+// intermediate columns 16 j .. 16 j + 15 of the tile's rows.  A pipeline unit is 2 KS KiB a wave: both tiles of an FP4
+// item, or one tile of an FP8 item (units 2 item, 2 item + 1); the next unit's loads are issued before the current unit's
+// products run.
 // Routed (FP4): rows [0, inter) are up, [inter, 2 inter) gate; h = bf16((g * logistic(g)) * u), g = min(gate, limit),
 // u = clamp(up) in FP32.  Shared (FP8): rows [0, inter) gate, then up; both rounded to BF16 first, clamped in BF16.
-// The weights of the next item are requested before the current item's products run.
 template <bool FP8, int KS>
 __device__ __forceinline__ void tf_fc1_items(const StreamArgs& p, int item_first, int item_last, float (*red)[2][4][64]) {
     const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
     const int per_tile = p.inter / 16, ks_first = wave * KS;
     if (item_first >= item_last) return;
+    constexpr int PER_ITEM = FP8 ? 2 : 1;                    // units per item
+    const int unit_first = item_first * PER_ITEM, unit_last = item_last * PER_ITEM;
     int loaded_tile = -1;
     ATile<KS> a;
-    BTile<KS, FP8> b0, b1;
-    ItemRef cur = tf_item(p, item_first, per_tile);
-    tf_load_b<KS, FP8>(b0, p.w + (size_t)cur.expert * p.w_expert_stride, p.ws + (size_t)cur.expert * p.ws_expert_stride,
-                       cur.j, p.k, ks_first, lane, p.bn, p.bk);
-    tf_load_b<KS, FP8>(b1, p.w + (size_t)cur.expert * p.w_expert_stride, p.ws + (size_t)cur.expert * p.ws_expert_stride,
-                       per_tile + cur.j, p.k, ks_first, lane, p.bn, p.bk);
-    for (int item = item_first; item < item_last; ++item) {
-        if (cur.tile != loaded_tile) {
+    Unit<2, KS> cur, next;
+    auto load_unit = [&](Unit<2, KS>& u, int unit) {
+        const ItemRef r = tf_item(p, unit / PER_ITEM, per_tile);
+        const uint8_t* w = p.w + (size_t)r.expert * p.w_expert_stride;
+        const uint8_t* ws = p.ws + (size_t)r.expert * p.ws_expert_stride;
+        if constexpr (FP8) {
+            const int nt[2] = {(unit & 1) * per_tile + r.j, 0};
+            tf_load_fp8<2, KS>(u, w, ws, nt, p.k, ks_first, lane, p.bn, p.bk);
+        } else {
+            const int nt[2] = {r.j, per_tile + r.j};
+            tf_load_fp4<2, KS>(u, w, ws, nt, p.k, ks_first, lane);
+        }
+    };
+    load_unit(cur, unit_first);
+    v4f first_acc = {0.f, 0.f, 0.f, 0.f};
+    for (int unit = unit_first; unit < unit_last; ++unit) {
+        const int item = unit / PER_ITEM;
+        const ItemRef r = tf_item(p, item, per_tile);
+        if (r.tile != loaded_tile) {
             long long row = -1;
-            if ((lane & 15) < cur.valid)
-                row = p.task_expert != nullptr ? p.token_map[cur.tile * 16 + (lane & 15)] / p.topk : cur.tile * 16 + (lane & 15);
+            if ((lane & 15) < r.valid)
+                row = p.task_expert != nullptr ? p.token_map[r.tile * 16 + (lane & 15)] / p.topk : r.tile * 16 + (lane & 15);
             tf_load_a<KS>(a, p.a_codes, p.a_scales, row, p.k, p.act_block, ks_first, lane);
-            loaded_tile = cur.tile;
+            loaded_tile = r.tile;
         }
-        BTile<KS, FP8> n0, n1;
-        ItemRef next = cur;
-        if (item + 1 < item_last) {
-            next = tf_item(p, item + 1, per_tile);
-            const uint8_t* w = p.w + (size_t)next.expert * p.w_expert_stride;
-            const uint8_t* ws = p.ws + (size_t)next.expert * p.ws_expert_stride;
-            tf_load_b<KS, FP8>(n0, w, ws, next.j, p.k, ks_first, lane, p.bn, p.bk);
-            tf_load_b<KS, FP8>(n1, w, ws, per_tile + next.j, p.k, ks_first, lane, p.bn, p.bk);
+        if (unit + 1 < unit_last) load_unit(next, unit + 1);
+        v4f c0, c1;
+        if constexpr (FP8) {
+            const v4f c = tf_dot_unit<true, 2, KS>(a, cur, 0);
+            if ((unit & 1) == 0) { first_acc = c; if (unit + 1 < unit_last) cur = next; continue; }
+            c0 = first_acc; c1 = c;
+        } else {
+            c0 = tf_dot_unit<false, 2, KS>(a, cur, 0);
+            c1 = tf_dot_unit<false, 2, KS>(a, cur, 1);
         }
-        const v4f c0 = tf_dot_tile<KS, FP8>(a, b0), c1 = tf_dot_tile<KS, FP8>(a, b1);
         float (*slot)[2][4][64] = red + (item & 1) * 4;
 #pragma unroll
         for (int i = 0; i < 4; ++i) { slot[wave][0][i][lane] = c0[i]; slot[wave][1][i][lane] = c1[i]; }
@@ -201,7 +230,7 @@ __device__ __forceinline__ void tf_fc1_items(const StreamArgs& p, int item_first
 #pragma unroll
             for (int i = 0; i < 4; ++i) {
                 const int m = 4 * (lane >> 4) + i;
-                if (m < cur.valid) {
+                if (m < r.valid) {
                     float first = slot[0][0][i][lane], second = slot[0][1][i][lane];
 #pragma unroll
                     for (int w2 = 1; w2 < 4; ++w2) {
@@ -209,12 +238,12 @@ __device__ __forceinline__ void tf_fc1_items(const StreamArgs& p, int item_first
                         second = __fadd_rn(second, slot[w2][1][i][lane]);
                     }
                     float value;
-                    const size_t row = (size_t)(cur.tile * 16 + m);
+                    const size_t row = (size_t)(r.tile * 16 + m);
                     if constexpr (FP8) {
                         const uint16_t gb = tf_to_bf16(first), ub = tf_to_bf16(second);
                         if (p.tap != nullptr) {
-                            p.tap[row * 2 * p.inter + 16 * cur.j + (lane & 15)] = gb;
-                            p.tap[row * 2 * p.inter + p.inter + 16 * cur.j + (lane & 15)] = ub;
+                            p.tap[row * 2 * p.inter + 16 * r.j + (lane & 15)] = gb;
+                            p.tap[row * 2 * p.inter + p.inter + 16 * r.j + (lane & 15)] = ub;
                         }
                         const float hi = tf_bf16(tf_to_bf16(p.limit)), lo = tf_bf16(tf_to_bf16(-p.limit));
                         const float g = fminf(tf_bf16(gb), hi);
@@ -225,40 +254,50 @@ __device__ __forceinline__ void tf_fc1_items(const StreamArgs& p, int item_first
                         const float u = fminf(p.limit, fmaxf(-p.limit, first));
                         value = __fmul_rn(__fmul_rn(g, tf_logistic(g)), u);
                     }
-                    p.out[row * p.inter + 16 * cur.j + (lane & 15)] = tf_to_bf16(value);
+                    p.out[row * p.inter + 16 * r.j + (lane & 15)] = tf_to_bf16(value);
                 }
             }
         }
-        if (item + 1 < item_last) { b0 = n0; b1 = n1; }
-        cur = next;
+        if (unit + 1 < unit_last) cur = next;
     }
 }
 
-// FC2.  Item = (tile, j): weight tiles 4 j .. 4 j + 3 of the expert's [hidden][k] matrix (64 output columns).  The
-// prologue of a tile quantizes its BF16 intermediate rows (MXFP8, `act_block` columns a block) into LDS; every wave then
-// keeps its K share as the A operand.  Routed: out[route][c] = bf16(acc * token_weight); dense: out[row][c] = bf16(acc).
+// FC2.  Routed item = (tile, j): weight tiles 4 j .. 4 j + 3 of the expert's [hidden][k] FP4 matrix (64 output columns);
+// shared item: tiles 2 j, 2 j + 1 of the FP8 matrix (32 columns): 4 KS KiB a wave either way.  The prologue of a tile
+// quantizes its BF16 intermediate rows (MXFP8, `act_block` columns a block) into LDS; every wave then keeps its K share
+// as the A operand.  Routed: out[route][c] = bf16(acc * token_weight); dense: out[row][c] = bf16(acc).
 template <bool FP8, int KS>
 __device__ __forceinline__ void tf_fc2_items(const StreamArgs& p, int item_first, int item_last, float (*red)[2][4][64],
                                              uint8_t* s_codes, uint8_t* s_scales) {
     const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
-    const int per_tile = p.hidden / 64, ks_first = wave * KS;
+    constexpr int COLS = FP8 ? 32 : 64, NT = COLS / 16;
+    const int per_tile = p.hidden / COLS, ks_first = wave * KS;
     if (item_first >= item_last) return;
     int loaded_tile = -1;
     ATile<KS> a;
-    BTile<KS, FP8> b[4];
-    ItemRef cur = tf_item(p, item_first, per_tile);
-#pragma unroll
-    for (int t = 0; t < 4; ++t)
-        tf_load_b<KS, FP8>(b[t], p.w + (size_t)cur.expert * p.w_expert_stride, p.ws + (size_t)cur.expert * p.ws_expert_stride,
-                           4 * cur.j + t, p.k, ks_first, lane, p.bn, p.bk);
+    Unit<4, KS> cur, next;
+    auto load_unit = [&](Unit<4, KS>& u, int item) {
+        const ItemRef r = tf_item(p, item, per_tile);
+        const uint8_t* w = p.w + (size_t)r.expert * p.w_expert_stride;
+        const uint8_t* ws = p.ws + (size_t)r.expert * p.ws_expert_stride;
+        if constexpr (FP8) {
+            const int nt[4] = {2 * r.j, 2 * r.j + 1, 0, 0};
+            tf_load_fp8<4, KS>(u, w, ws, nt, p.k, ks_first, lane, p.bn, p.bk);
+        } else {
+            const int nt[4] = {4 * r.j, 4 * r.j + 1, 4 * r.j + 2, 4 * r.j + 3};
+            tf_load_fp4<4, KS>(u, w, ws, nt, p.k, ks_first, lane);
+        }
+    };
+    load_unit(cur, item_first);
     for (int item = item_first; item < item_last; ++item) {
-        if (cur.tile != loaded_tile) {
+        const ItemRef r = tf_item(p, item, per_tile);
+        if (r.tile != loaded_tile) {
             __syncthreads();
             // quantize rows [0, valid) of the tile: 8 values a lane-step, groups of act_block / 8 lanes
             const int per_row = p.k >> 3, group_lanes = p.act_block >> 3;
-            for (int q = threadIdx.x; q < cur.valid * per_row; q += blockDim.x) {
+            for (int q = threadIdx.x; q < r.valid * per_row; q += blockDim.x) {
                 const int m = q / per_row, c8 = q - m * per_row;
-                const u4v wv = reinterpret_cast<const u4v*>(p.a_bf16 + (size_t)(cur.tile * 16 + m) * p.k)[c8];
+                const u4v wv = reinterpret_cast<const u4v*>(p.a_bf16 + (size_t)(r.tile * 16 + m) * p.k)[c8];
                 float v[8];
 #pragma unroll
                 for (int i = 0; i < 4; ++i) { v[2 * i] = tf_bf16_lo(wv[i]); v[2 * i + 1] = tf_bf16_hi(wv[i]); }
@@ -266,78 +305,76 @@ __device__ __forceinline__ void tf_fc2_items(const StreamArgs& p, int item_first
                 const Quant8 c = tf_quant8(v, amax, p.min_amax);
                 reinterpret_cast<u2v*>(s_codes + (size_t)m * p.k)[c8] = u2v{c.lo, c.hi};
                 if ((c8 & (group_lanes - 1)) == 0) s_scales[m * (p.k / p.act_block) + c8 / group_lanes] = (uint8_t)c.exponent;
-                if (p.q_codes != nullptr && cur.j == 0) {
-                    reinterpret_cast<u2v*>(p.q_codes + (size_t)(cur.tile * 16 + m) * p.k)[c8] = u2v{c.lo, c.hi};
+                if (p.q_codes != nullptr && r.j == 0) {
+                    reinterpret_cast<u2v*>(p.q_codes + (size_t)(r.tile * 16 + m) * p.k)[c8] = u2v{c.lo, c.hi};
                     if ((c8 & (group_lanes - 1)) == 0)
-                        p.q_scales[(size_t)(cur.tile * 16 + m) * (p.k / p.act_block) + c8 / group_lanes] = (uint8_t)c.exponent;
+                        p.q_scales[(size_t)(r.tile * 16 + m) * (p.k / p.act_block) + c8 / group_lanes] = (uint8_t)c.exponent;
                 }
             }
             __syncthreads();
-            tf_load_a<KS>(a, s_codes, s_scales, (lane & 15) < cur.valid ? (lane & 15) : -1, p.k, p.act_block, ks_first, lane);
-            loaded_tile = cur.tile;
+            tf_load_a<KS>(a, s_codes, s_scales, (lane & 15) < r.valid ? (lane & 15) : -1, p.k, p.act_block, ks_first, lane);
+            loaded_tile = r.tile;
         }
-        BTile<KS, FP8> n[4];
-        ItemRef next = cur;
-        if (item + 1 < item_last) {
-            next = tf_item(p, item + 1, per_tile);
+        if (item + 1 < item_last) load_unit(next, item + 1);
 #pragma unroll
-            for (int t = 0; t < 4; ++t)
-                tf_load_b<KS, FP8>(n[t], p.w + (size_t)next.expert * p.w_expert_stride,
-                                   p.ws + (size_t)next.expert * p.ws_expert_stride, 4 * next.j + t, p.k, ks_first, lane, p.bn, p.bk);
-        }
-#pragma unroll
-        for (int t = 0; t < 4; ++t) {
-            const v4f c = tf_dot_tile<KS, FP8>(a, b[t]);
+        for (int t = 0; t < NT; ++t) {
+            const v4f c = tf_dot_unit<FP8, 4, KS>(a, cur, t);
 #pragma unroll
             for (int i = 0; i < 4; ++i) red[(t >> 1) * 4 + wave][t & 1][i][lane] = c[i];
         }
         __syncthreads();
-        // waves 0..3 each finish one of the four 16-column tiles
-        {
+        // wave w finishes 16-column tile w of the item (routed: 4 tiles; shared: 2)
+        if (wave < NT) {
             float (*slot)[2][4][64] = red + (wave >> 1) * 4;
             const int which = wave & 1;
 #pragma unroll
             for (int i = 0; i < 4; ++i) {
                 const int m = 4 * (lane >> 4) + i;
-                if (m < cur.valid) {
+                if (m < r.valid) {
                     float acc = slot[0][which][i][lane];
 #pragma unroll
                     for (int w2 = 1; w2 < 4; ++w2) acc = __fadd_rn(acc, slot[w2][which][i][lane]);
-                    const int col = 64 * cur.j + 16 * wave + (lane & 15);
+                    const int col = COLS * r.j + 16 * wave + (lane & 15);
                     if (p.task_expert != nullptr) {
-                        const int phys = cur.tile * 16 + m;
+                        const int phys = r.tile * 16 + m;
                         p.out[(size_t)p.token_map[phys] * p.hidden + col] = tf_to_bf16(__fmul_rn(acc, p.token_weights[phys]));
                     } else {
-                        p.out[(size_t)(cur.tile * 16 + m) * p.hidden + col] = tf_to_bf16(acc);
+                        p.out[(size_t)(r.tile * 16 + m) * p.hidden + col] = tf_to_bf16(acc);
                     }
                 }
             }
         }
         __syncthreads();
-        if (item + 1 < item_last) {
-#pragma unroll
-            for (int t = 0; t < 4; ++t) b[t] = n[t];
-        }
-        cur = next;
+        if (item + 1 < item_last) cur = next;
     }
 }
 
-__device__ __forceinline__ int tf_tiles(const StreamArgs& p) {
-    return p.task_expert != nullptr ? p.expert_tile_base[p.experts] : (p.dense_rows + 15) / 16;
-}
-// Persistent launch: workgroup b of G takes items [b W / G, (b + 1) W / G).  block = 256 threads (four waves).
-template <bool FP8, int KS>
-__global__ void __launch_bounds__(256) tf_fc1_stream(const StreamArgs p) {
+// Persistent launch of one phase over the routed experts and, optionally, the shared expert (`shared.w == nullptr`: routed
+// only; `routed.w == nullptr`: dense only).  Every item costs the same bytes (a shared FC1 item counts twice), so workgroup
+// b of G takes the cost range [b C / G, (b + 1) C / G) of the list "routed items, then shared items".  block = 256.
+template <int KSR, int KSS>
+__global__ void __launch_bounds__(256, 2) tf_phase1_stream(const StreamArgs routed, const StreamArgs shared) {
     __shared__ float red[8][2][4][64];
-    const long long items = (long long)tf_tiles(p) * (p.inter / 16);
-    const int first = (int)(items * blockIdx.x / gridDim.x), last = (int)(items * (blockIdx.x + 1) / gridDim.x);
-    tf_fc1_items<FP8, KS>(p, first, last, red);
+    const long long r_items = routed.w ? (long long)tf_tiles(routed) * (routed.inter / 16) : 0;
+    const long long s_units = shared.w ? (long long)tf_tiles(shared) * (shared.inter / 16) * 2 : 0;
+    const long long total = r_items + s_units;
+    const long long lo = total * blockIdx.x / gridDim.x, hi = total * (blockIdx.x + 1) / gridDim.x;
+    if (lo < r_items) tf_fc1_items<false, KSR>(routed, (int)lo, (int)(hi < r_items ? hi : r_items), red);
+    if (hi > r_items) {
+        const long long a = (lo > r_items ? lo - r_items : 0), b = hi - r_items;
+        __syncthreads();
+        tf_fc1_items<true, KSS>(shared, (int)((a + 1) / 2), (int)((b + 1) / 2), red);
+    }
 }
-template <bool FP8, int KS>
-__global__ void __launch_bounds__(256) tf_fc2_stream(const StreamArgs p) {
+template <int KSR, int KSS>
+__global__ void __launch_bounds__(256, 2) tf_phase2_stream(const StreamArgs routed, const StreamArgs shared) {
     __shared__ float red[8][2][4][64];
     extern __shared__ uint8_t dyn[];
-    const long long items = (long long)tf_tiles(p) * (p.hidden / 64);
-    const int first = (int)(items * blockIdx.x / gridDim.x), last = (int)(items * (blockIdx.x + 1) / gridDim.x);
-    tf_fc2_items<FP8, KS>(p, first, last, red, dyn, dyn + 16 * (size_t)p.k);
+    const long long r_items = routed.w ? (long long)tf_tiles(routed) * (routed.hidden / 64) : 0;
+    const long long s_items = shared.w ? (long long)tf_tiles(shared) * (shared.hidden / 32) : 0;
+    const long long total = r_items + s_items;
+    const long long lo = total * blockIdx.x / gridDim.x, hi = total * (blockIdx.x + 1) / gridDim.x;
+    const int kmax = routed.w && (!shared.w || routed.k > shared.k) ? routed.k : shared.k;
+    if (lo < r_items) tf_fc2_items<false, KSR>(routed, (int)lo, (int)(hi < r_items ? hi : r_items), red, dyn, dyn + 16 * (size_t)kmax);
+    if (hi > r_items) tf_fc2_items<true, KSS>(shared, (int)(lo > r_items ? lo - r_items : 0), (int)(hi - r_items), red, dyn, dyn + 16 * (size_t)kmax);
 }

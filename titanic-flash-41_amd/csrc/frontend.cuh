@@ -65,7 +65,7 @@ __device__ __forceinline__ void tf_plan_block(const int32_t* ids, const float* w
                                               int32_t* expert_tile_base, int pairs, int experts, int groups, int tile_m) {
     __shared__ int32_t s_ids[1024];
     __shared__ int32_t s_base[513];
-    __shared__ int32_t s_wave[16];
+    __shared__ int32_t s_wave[16];   // blocks of at most 1,024 threads
     const int t = threadIdx.x, lane = t & 63, wave = t >> 6;
     for (int p = t; p < pairs; p += blockDim.x) s_ids[p] = ids[p];
     __syncthreads();
@@ -122,7 +122,7 @@ __device__ __forceinline__ void tf_frontend_run(const uint16_t* input, const int
                      (long long)(blockIdx.x - first) * blockDim.x + threadIdx.x,
                      (long long)(gridDim.x - first) * blockDim.x);
 }
-extern "C" __global__ void __launch_bounds__(1024) ca_moe_frontend(
+extern "C" __global__ void __launch_bounds__(512) ca_moe_frontend(
     const uint16_t* input, const int32_t* ids, const float* weights, uint8_t* packed, uint8_t* scales,
     int32_t* token_map, float* token_weights, int32_t* task_expert, int32_t* task_valid_rows,
     int32_t* expert_tile_base, int32_t rows, int32_t topk, int32_t experts, int32_t cols, int32_t groups,
@@ -132,20 +132,57 @@ extern "C" __global__ void __launch_bounds__(1024) ca_moe_frontend(
 }
 // The front-end with the router's top-k inside: block 0 first routes every owner row from the gate's logits (and
 // applies padding routes), then plans; the other blocks quantize meanwhile (launch one block more).
-extern "C" __global__ void __launch_bounds__(1024) ca_moe_route_frontend(
+// With `gate_w` the gate product runs here too: `logit_blocks` further blocks (one wave per expert) compute the logits,
+// publish them and count themselves in at `sync`; block 0 waits for that count, bounded: if the count does not arrive it
+// computes the logits itself, so the kernel always ends.  All blocks of this small grid are resident together.
+extern "C" __global__ void __launch_bounds__(512) ca_moe_route_frontend(
     const uint16_t* input, int32_t* ids, float* weights, uint8_t* packed, uint8_t* scales, int32_t* token_map,
     float* token_weights, int32_t* task_expert, int32_t* task_valid_rows, int32_t* expert_tile_base,
-    const float* logits, const float* bias, const float* bias_alt, const long long* tokens, const int32_t* live,
+    float* logits, const float* bias, const float* bias_alt, const long long* tokens, const int32_t* live,
     const int32_t* padding, int32_t rows, int32_t topk, int32_t experts, int32_t cols, int32_t groups, int32_t tile_m,
     int32_t owner_rows, int32_t act_block, uint8_t* packed_min, uint8_t* scales_min, int32_t scoring,
-    float route_scale, long long alt_token) {
+    float route_scale, long long alt_token, const uint16_t* gate_w, uint32_t* sync, int32_t logit_blocks) {
+    const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6, waves = blockDim.x >> 6;
+    const int first_logit_block = (int)gridDim.x - logit_blocks;
+    if (gate_w != nullptr && (int)blockIdx.x >= first_logit_block) {
+        const int e = ((int)blockIdx.x - first_logit_block) * waves + wave;
+        if (e < experts) tf_logits_expert(input, gate_w, logits, owner_rows, cols, experts, e, lane);
+        __threadfence();
+        __syncthreads();
+        if (threadIdx.x == 0) atomicAdd(sync, 1u);
+        return;
+    }
     if (blockIdx.x == 0) {
+        if (gate_w != nullptr) {
+            __shared__ int arrived;
+            if (threadIdx.x == 0) {
+                int ok = 0;
+                for (int spin = 0; spin < (1 << 18); ++spin) {
+                    if (__hip_atomic_load(sync, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT) >= (uint32_t)logit_blocks) { ok = 1; break; }
+                    __builtin_amdgcn_s_sleep(2);
+                }
+                __hip_atomic_store(sync, 0u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+                arrived = ok;
+            }
+            __syncthreads();
+            if (!arrived)
+                for (int e = wave; e < experts; e += waves) tf_logits_expert(input, gate_w, logits, owner_rows, cols, experts, e, lane);
+            __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "agent");
+            __syncthreads();
+        }
         const RouteParams p{experts, topk, scoring, route_scale, alt_token};
         tf_route_block(logits, bias, bias_alt, tokens, live, padding, ids, weights, owner_rows, p, 0,
                        blockDim.x >> 6, true);
     }
-    tf_frontend_run(input, ids, weights, packed, scales, packed_min, scales_min, token_map, token_weights, task_expert,
-                    task_valid_rows, expert_tile_base, rows, topk, experts, cols, groups, tile_m, act_block, 1);
+    if ((int)blockIdx.x >= first_logit_block) return;
+    // quantizer blocks are blocks [1, first_logit_block)
+    if (blockIdx.x == 0) {
+        tf_plan_block(ids, weights, token_map, token_weights, task_expert, task_valid_rows, expert_tile_base, rows * topk, experts, groups, tile_m);
+        return;
+    }
+    const long long total = (long long)rows * (cols >> 3);
+    tf_quantize_span(input, packed, scales, packed_min, scales_min, total, act_block,
+                     (long long)(blockIdx.x - 1) * blockDim.x + threadIdx.x, (long long)(first_logit_block - 1) * blockDim.x);
 }
 // Row quantizer alone (any number of rows).
 extern "C" __global__ void __launch_bounds__(256) ca_quantize_rows(

@@ -4,41 +4,53 @@
 #pragma once
 #include "common.cuh"
 
-// logits[m][e] = sum_k x[m][k] * w[e][k], BF16 inputs, FP32 accumulate.  One wave per expert, up to 16 rows.
+// logits[m][e] = sum_k x[m][k] * w[e][k], BF16 inputs, FP32 accumulate, for one expert by one wave.
 // Fixed summation order: lane l accumulates the 8-element vectors at k = 512 j + 8 l (j ascending) with fma in k order,
-// then the 64 partials are combined by the xor butterfly 32, 16, 8, 4, 2, 1.  hidden % 512 == 0.
+// then the 64 partials are combined by the xor butterfly 32, 16, 8, 4, 2, 1.  hidden % 512 == 0, hidden <= 8192.
+// The expert's row is requested whole before any use, and the token rows four at a time.
+__device__ __forceinline__ void tf_logits_expert(const uint16_t* __restrict__ x, const uint16_t* __restrict__ w, float* __restrict__ out,
+                                                 int rows, int hidden, int experts, int e, int lane) {
+    const int nj = hidden >> 9;
+    u4v wv[16];
+    const u4v* wrow = reinterpret_cast<const u4v*>(w + (size_t)e * hidden);
+#pragma unroll
+    for (int j = 0; j < 16; ++j) if (j < nj) wv[j] = wrow[j * 64 + lane];
+    for (int m0 = 0; m0 < rows; m0 += 4) {
+        float acc[4] = {0.f, 0.f, 0.f, 0.f};
+#pragma unroll
+        for (int half = 0; half < 2; ++half) {               // eight vectors of four rows in flight
+            u4v xv[4][8];
+#pragma unroll
+            for (int r = 0; r < 4; ++r)
+#pragma unroll
+                for (int j = 0; j < 8; ++j)
+                    if (m0 + r < rows && half * 8 + j < nj) xv[r][j] = reinterpret_cast<const u4v*>(x + (size_t)(m0 + r) * hidden)[(half * 8 + j) * 64 + lane];
+#pragma unroll
+            for (int r = 0; r < 4; ++r)
+#pragma unroll
+                for (int j = 0; j < 8; ++j)
+                    if (m0 + r < rows && half * 8 + j < nj) {
+#pragma unroll
+                        for (int i = 0; i < 4; ++i) {
+                            acc[r] = __fmaf_rn(tf_bf16_lo(xv[r][j][i]), tf_bf16_lo(wv[half * 8 + j][i]), acc[r]);
+                            acc[r] = __fmaf_rn(tf_bf16_hi(xv[r][j][i]), tf_bf16_hi(wv[half * 8 + j][i]), acc[r]);
+                        }
+                    }
+        }
+#pragma unroll
+        for (int r = 0; r < 4; ++r) {
+            float v = acc[r];
+#pragma unroll
+            for (int o = 32; o > 0; o >>= 1) v = __fadd_rn(v, __shfl_xor(v, o));
+            if (lane == 0 && m0 + r < rows) out[(size_t)(m0 + r) * experts + e] = v;
+        }
+    }
+}
+// One wave per expert, up to 16 rows a launch.
 extern "C" __global__ void __launch_bounds__(64) ca_router_logits_rows(
     const uint16_t* __restrict__ x, const uint16_t* __restrict__ w, float* __restrict__ out, int rows, int hidden,
     int experts) {
-    const int e = blockIdx.x, lane = threadIdx.x;
-    if (e >= experts) return;
-    float acc[16];
-#pragma unroll
-    for (int m = 0; m < 16; ++m) acc[m] = 0.f;
-    const u4v* wrow = reinterpret_cast<const u4v*>(w + (size_t)e * hidden);
-    for (int j = 0; j < hidden / 512; ++j) {
-        const u4v wv = wrow[j * 64 + lane];
-#pragma unroll
-        for (int m = 0; m < 16; ++m) {
-            if (m < rows) {
-                const u4v xv = reinterpret_cast<const u4v*>(x + (size_t)m * hidden)[j * 64 + lane];
-#pragma unroll
-                for (int i = 0; i < 4; ++i) {
-                    acc[m] = __fmaf_rn(tf_bf16_lo(xv[i]), tf_bf16_lo(wv[i]), acc[m]);
-                    acc[m] = __fmaf_rn(tf_bf16_hi(xv[i]), tf_bf16_hi(wv[i]), acc[m]);
-                }
-            }
-        }
-    }
-#pragma unroll
-    for (int m = 0; m < 16; ++m) {
-        if (m < rows) {
-            float v = acc[m];
-#pragma unroll
-            for (int o = 32; o > 0; o >>= 1) v = __fadd_rn(v, __shfl_xor(v, o));
-            if (lane == 0) out[(size_t)m * experts + e] = v;
-        }
-    }
+    if ((int)blockIdx.x < experts) tf_logits_expert(x, w, out, rows, hidden, experts, blockIdx.x, threadIdx.x);
 }
 
 struct RouteParams {

@@ -27,7 +27,7 @@ def load():
         vp, cp, sz = ctypes.c_void_p, ctypes.c_char_p, ctypes.c_size_t
         lib.tfh_layer_create.restype = vp
         lib.tfh_layer_create.argtypes = [cp, ctypes.POINTER(native.Geometry), ctypes.c_int, ctypes.POINTER(vp), ctypes.c_int, ctypes.c_int,
-                                         ctypes.c_int, ctypes.c_int, ctypes.c_int, cp, sz]
+                                         ctypes.c_int, ctypes.c_int, ctypes.c_int, ctypes.c_int, ctypes.c_int, cp, sz]
         lib.tfh_layer_destroy.argtypes = [vp]
         lib.tfh_layer_destroy.restype = None
         lib.tfh_layer_set_tokens.argtypes = [vp, vp, ctypes.c_int, vp, cp, sz]
@@ -52,7 +52,7 @@ class HostError(RuntimeError):
 class Layer:
     """One LayerFfn + Workspace + TokenRows on cuda:0 for `rows` token rows."""
 
-    def __init__(self, geometry, operands, rows, overlap=True, sum_shared=True, route_front=True, code_scales=False):
+    def __init__(self, geometry, operands, rows, overlap=True, sum_shared=True, route_front=True, code_scales=False, fold_shared=True, gate_front=True):
         self.lib = load()
         native.load()
         self.g, self.rows = geometry, rows
@@ -66,7 +66,7 @@ class Layer:
             import torch
             torch.cuda.synchronize()
         self.h = self.lib.tfh_layer_create(native.KERNEL_LIB.encode(), ctypes.byref(geometry), rows, ptrs, int(on_device), int(overlap),
-                                           int(sum_shared), int(route_front), int(code_scales), self._err, 512)
+                                           int(sum_shared), int(route_front), int(code_scales), int(fold_shared), int(gate_front), self._err, 512)
         if not self.h:
             raise HostError(self._err.value.decode())
         self.h = ctypes.c_void_p(self.h)

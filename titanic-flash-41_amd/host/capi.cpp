@@ -28,7 +28,7 @@ extern "C" {
 
 // operands: gate_w, bias, bias_alt, w13, s13, w2, s2, sh_w13, sh_s13, sh_w2, sh_s2 (canonical checkpoint layout).
 void* tfh_layer_create(const char* kernel_library, const ca_geometry* geometry, int rows, const void* const* operands, int operands_on_device,
-                       int overlap, int sum_shared, int route_front, int code_scales, char* error, size_t error_len) {
+                       int overlap, int sum_shared, int route_front, int code_scales, int fold_shared, int gate_front, char* error, size_t error_len) {
     Handle* h = new Handle;
     const int status = guarded(error, error_len, [&] {
         h->native = std::make_shared<tf::Native>(kernel_library, *geometry);
@@ -39,7 +39,7 @@ void* tfh_layer_create(const char* kernel_library, const ca_geometry* geometry, 
         h->prepared = tf::prepare_layer(*h->native, *h->weights, 0);
         if (code_scales) h->scale_code = tf::code_layer_scales(*h->native, *h->weights, h->prepared);
         tf::LayerFfn::Options options;
-        options.overlap = overlap != 0; options.sum_shared = sum_shared != 0; options.route_front = route_front != 0;
+        options.overlap = overlap != 0; options.sum_shared = sum_shared != 0; options.route_front = route_front != 0; options.fold_shared = fold_shared != 0; options.gate_front = gate_front != 0;
         h->layer = std::make_unique<tf::LayerFfn>(h->native, h->weights, h->prepared, (size_t)rows, options);
         h->workspace = std::make_unique<tf::Workspace>(h->native, (size_t)rows);
         std::vector<int64_t> ids((size_t)rows, 0);

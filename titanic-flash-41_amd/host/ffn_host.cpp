@@ -244,13 +244,16 @@ Router::Router(std::shared_ptr<const Native> native, std::shared_ptr<Weights> we
            "router checkpoint shape/dtype mismatch");                                                        // src/ffn.rs:225-228
     census_.zero();
 }
-std::optional<RouteOperands> Router::run_routed(uint64_t input, size_t input_len, const TokenRows& tokens, bool fused, const Stream& stream) {
+std::optional<RouteOperands> Router::run_routed(uint64_t input, size_t input_len, const TokenRows& tokens, bool fused, const Stream& stream,
+                                                bool gate_front) {
     const ca_geometry& g = native_->geometry();
     ensure(input_len == rows_ * (size_t)g.hidden && tokens.rows() == rows_, "router shape/context mismatch");   // src/ffn.rs:331-339
     ensure(!stream_set_ || stream_ == stream.raw(), "router needs one ordered stream");                        // :340-345
     stream_ = stream.raw(); stream_set_ = true;
     const uint64_t gate = weights_->ptr("ffn.gate.weight");
-    if (rows_ <= 64) {
+    const bool gate_in_front = fused && gate_front && rows_ <= 16;
+    if (gate_in_front) {
+    } else if (rows_ <= 64) {
         for (size_t offset = 0; offset < rows_; offset += 16)                                                  // :351-364
             native_->router_logits((int)std::min<size_t>(16, rows_ - offset), input + offset * g.hidden * 2, gate,
                                    logits_.ptr() + offset * g.experts * 4, stream.raw());
@@ -261,7 +264,8 @@ std::optional<RouteOperands> Router::run_routed(uint64_t input, size_t input_len
     if (fused) {
         ensure(rows_ * g.topk <= 1024, "fused routing owner");                                                 // :370-371
         return RouteOperands{logits_.ptr(), bias, bias_alt, tokens.ids().ptr(), tokens.live().ptr(),
-                             tokens.padding_active() ? tokens.padding_sources().ptr() : 0, ids_.ptr(), routing_.ptr(), rows_};
+                             tokens.padding_active() ? tokens.padding_sources().ptr() : 0, ids_.ptr(), routing_.ptr(), rows_,
+                             gate_in_front ? gate : 0};
     }
     uint64_t lp = logits_.ptr(), tp = tokens.ids().ptr(), vp = tokens.live().ptr(), ip = ids_.ptr(), wp = routing_.ptr();
     uint64_t b = bias, ba = bias_alt;
@@ -306,6 +310,7 @@ Workspace::Workspace(std::shared_ptr<const Native> native, size_t rows) : native
     add("token_map_ptr", padded * 4); add("token_weights_ptr", padded * 4);
     add("scatter_ptr", pairs * H * 2);
     add("plan_scratch_ptr", ((pairs + 63) / 64 * g.experts + pairs) * 4);
+    add("sync_ptr", 256);
     scratch_ = Buffer<uint8_t>(at);
     scratch_.zero();                                                                                          // scratch_initializer "zero", src/moe.rs:440
     output_ = Buffer<uint16_t>(rows * H);
@@ -337,7 +342,8 @@ void Workspace::pointers(const Expert& expert, uint64_t input, const Buffer<int3
 }
 std::optional<std::pair<uint64_t, size_t>> Workspace::run_live_for_ffn(const Expert& expert, uint64_t input, size_t input_len, const Buffer<int32_t>& ids,
                                                                        const Buffer<float>& routing_weights, size_t live, bool fuse_sum,
-                                                                       const std::optional<RouteOperands>& route, const Stream& stream) {
+                                                                       const std::optional<RouteOperands>& route, const Stream& stream,
+                                                                       const SharedOperands* shared) {
     const ca_geometry& g = native_->geometry();
     ensure(live <= rows_, "MoE live row domain");                                                             // src/moe.rs:1045
     guard_stream(stream);
@@ -345,15 +351,29 @@ std::optional<std::pair<uint64_t, size_t>> Workspace::run_live_for_ffn(const Exp
     ensure(expert.layout().experts == (size_t)g.experts && expert.layout().hidden == (size_t)g.hidden &&
                expert.layout().intermediate == (size_t)g.intermediate && ids.len() == rows_ * g.topk && routing_weights.len() == rows_ * g.topk,
            "MoE input shape mismatch");                                                                       // :1103-1114
-    uint64_t p[27];
+    uint64_t p[38];
     pointers(expert, input, ids, routing_weights, p);
-    int32_t scalars[7] = {(int32_t)rows_, (int32_t)rows_, (int32_t)(max_tiles_ * tile_m_), (int32_t)max_tiles_, (int32_t)tile_m_, 1, 0};
-    if (route) {
+    int32_t scalars[7] = {(int32_t)rows_, (int32_t)rows_, (int32_t)(max_tiles_ * tile_m_), (int32_t)max_tiles_, (int32_t)tile_m_, 1, (int32_t)rows_};
+    if (shared) {
+        ensure(rows_ <= 64 && p[5] && p[6], "folded shared expert is for few-row owners");
+        for (int i = 21; i < 29; ++i) p[i] = 0;
+        if (route) {
+            ensure(route->ids == p[1] && route->weights == p[2] && route->owner_rows == rows_ && route->logits && route->bias && route->live,
+                   "fused routing domain");
+            p[21] = route->logits; p[22] = route->bias; p[23] = route->bias_alt; p[24] = route->tokens; p[25] = route->live; p[26] = route->padding;
+            p[27] = route->gate_w; p[28] = at("sync_ptr");
+        }
+        const uint64_t sh[9] = {shared->w13, shared->s13, shared->w2, shared->s2, shared->activation, shared->activation_codes,
+                                shared->activation_scales, shared->up_tap, shared->output};
+        for (int i = 0; i < 9; ++i) p[29 + i] = sh[i];
+        native_->primitive(9, p, 38, scalars, 7, stream.raw(), "ffn.experts_with_shared");
+    } else if (route) {
         ensure(route->ids == p[1] && route->weights == p[2] && route->owner_rows == rows_ && route->logits && route->bias && route->live,
                "fused routing domain");                                                                       // :1266-1269
         p[21] = route->logits; p[22] = route->bias; p[23] = route->bias_alt; p[24] = route->tokens; p[25] = route->live; p[26] = route->padding;
+        p[27] = route->gate_w; p[28] = at("sync_ptr");
         scalars[6] = (int32_t)route->owner_rows;
-        native_->primitive(1, p, 27, scalars, 7, stream.raw(), "integration.tp_moe.dynamic (route front)");
+        native_->primitive(1, p, 29, scalars, 7, stream.raw(), "integration.tp_moe.dynamic (route front)");
     } else {
         native_->primitive(0, p, 21, scalars, 6, stream.raw(), "integration.tp_moe.dynamic");
     }
@@ -411,17 +431,29 @@ void LayerFfn::run(Workspace& workspace, uint64_t input, size_t input_len, const
     const bool fused = options_.route_front && rows_ * g.topk <= 1024;                                          // :988-990
     // Dual-stream schedule (:1007-1010, :1028-1036): the shared branch forks before routing, quantizes the input itself
     // and joins before the sum.  Without the branch the front-end emits the shared-flavour codes beside the routed ones.
-    workspace.emit_shared_input(!branch_stream_);
-    if (branch_stream_) {
+    const bool fold = options_.fold_shared && rows_ <= 64;
+    const bool branch = branch_stream_ && !fold;
+    workspace.emit_shared_input(!branch);
+    if (fold) {
+        const SharedOperands shared{shared_w13_.values, shared_w13_.scales, shared_w2_.values, shared_w2_.scales, activation_.ptr(),
+                                    activation_codes_.ptr(), activation_scales_.ptr(), shared_up_.ptr(), shared_down_.ptr()};
+        const std::optional<RouteOperands> route = router_.run_routed(input, input_len, tokens, fused, stream, options_.gate_front);
+        const auto deferred = workspace.run_live_for_ffn(expert_, input, input_len, router_.ids(), router_.routing(), tokens.active_rows(),
+                                                         options_.sum_shared, route, stream, &shared);
+        if (deferred) sum_shared(workspace, deferred->second, stream);
+        else add_shared(workspace, stream);
+        return;
+    }
+    if (branch) {
         input_ready_->record(stream.raw());
         input_ready_->wait(branch_stream_->raw());
         run_shared(workspace, input, *branch_stream_);
         output_ready_->record(branch_stream_->raw());
     }
-    const std::optional<RouteOperands> route = router_.run_routed(input, input_len, tokens, fused, stream);
+    const std::optional<RouteOperands> route = router_.run_routed(input, input_len, tokens, fused, stream, options_.gate_front);
     const auto deferred = workspace.run_live_for_ffn(expert_, input, input_len, router_.ids(), router_.routing(), tokens.active_rows(),
                                                      options_.sum_shared, route, stream);
-    if (branch_stream_) output_ready_->wait(stream.raw());
+    if (branch) output_ready_->wait(stream.raw());
     else run_shared(workspace, 0, stream);
     if (deferred) sum_shared(workspace, deferred->second, stream);
     else add_shared(workspace, stream);

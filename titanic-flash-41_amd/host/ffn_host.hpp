@@ -126,14 +126,19 @@ private:
 };
 
 // Operands a router hands to the experts' front-end when its top-k runs there (src/moe.rs:181-200 RouteOperands).
-struct RouteOperands { uint64_t logits, bias, bias_alt, tokens, live, padding, ids, weights; size_t owner_rows; };
+// gate_w != 0: the gate product is left to the front-end too (owners of at most 16 rows).
+struct RouteOperands { uint64_t logits, bias, bias_alt, tokens, live, padding, ids, weights; size_t owner_rows; uint64_t gate_w; };
+// Operands of the shared expert when it is folded into the routed experts' launches (entry "ffn.experts_with_shared"):
+// prepared w13 / scales / w2 / scales, activation (BF16), its codes and scales, the up-projection tap, the output.
+struct SharedOperands { uint64_t w13, s13, w2, s2, activation, activation_codes, activation_scales, up_tap, output; };
 
 class Router {                                                                                      // src/ffn.rs:173-426
 public:
     Router(std::shared_ptr<const Native> native, std::shared_ptr<Weights> weights, size_t rows);
     void run(uint64_t input, size_t input_len, const TokenRows& tokens, const Stream& stream) { run_routed(input, input_len, tokens, false, stream); }
     // fused: the gate product only; returns the operands for the front-end that will route.
-    std::optional<RouteOperands> run_routed(uint64_t input, size_t input_len, const TokenRows& tokens, bool fused, const Stream& stream);
+    std::optional<RouteOperands> run_routed(uint64_t input, size_t input_len, const TokenRows& tokens, bool fused, const Stream& stream,
+                                            bool gate_front = false);
     const Buffer<float>& logits() const { return logits_; }
     const Buffer<int32_t>& ids() const { return ids_; }
     const Buffer<float>& routing() const { return routing_; }
@@ -162,7 +167,8 @@ public:
     // and row count; otherwise the topk_sum node runs and output() holds the reduced rows.
     std::optional<std::pair<uint64_t, size_t>> run_live_for_ffn(const Expert& expert, uint64_t input, size_t input_len, const Buffer<int32_t>& ids,
                                                                const Buffer<float>& routing_weights, size_t live, bool fuse_sum,
-                                                               const std::optional<RouteOperands>& route, const Stream& stream);
+                                                               const std::optional<RouteOperands>& route, const Stream& stream,
+                                                               const SharedOperands* shared = nullptr);
     void run(const Expert& expert, uint64_t input, size_t input_len, const Buffer<int32_t>& ids, const Buffer<float>& routing_weights,
              const Stream& stream) { run_live_for_ffn(expert, input, input_len, ids, routing_weights, rows_, false, std::nullopt, stream); }
     // Phase nodes alone (for per-kernel timing): 8 = front-end (plan + quantize), 6 = FC1 + SwiGLU, 7 = FC2.
@@ -192,6 +198,9 @@ public:
         bool overlap = true;        // FFN_OVERLAP: shared expert on an auxiliary stream beside the routed experts (:518-522)
         bool sum_shared = true;     // FFN_SUM_SHARED: fused route sum + shared addition (:1037-1046)
         bool route_front = true;    // MOE_ROUTE_FRONT: the router's top-k inside the experts' front-end (:986-990)
+        bool gate_front = true;     // the gate product inside the front-end launch as well (owners of at most 16 rows)
+        bool fold_shared = true;    // few rows: the shared expert's weights stream inside the routed experts' two launches
+                                    // (one queue, no cross-stream join); takes precedence over `overlap`
     };
     LayerFfn(std::shared_ptr<const Native> native, std::shared_ptr<Weights> weights, Prepared layout, size_t rows, Options options);
     void run(Workspace& workspace, uint64_t input, size_t input_len, const TokenRows& tokens, const Stream& stream);
