@@ -1,0 +1,90 @@
+"""CPU-side checks of the drop-in boundary: the shared libraries load without a GPU and export every symbol the header
+declares, the operator contracts agree with the library's entry table, and argument validation answers with the
+reference's error conventions before anything would touch a device."""
+import ctypes
+import importlib
+import json
+import os
+import re
+
+import pytest
+
+ROOT = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
+pkg = importlib.import_module("titanic-flash-41_amd")
+native = pkg.native
+contracts = importlib.import_module("titanic-flash-41_amd.contracts")
+
+
+def declared_symbols():
+    text = open(os.path.join(ROOT, "include", "titanic_moe.h")).read()
+    text = re.sub(r"/\*.*?\*/", "", text, flags=re.S)
+    return sorted(set(re.findall(r"\b(ca_[a-z0-9_]+)\s*\(", text)))
+
+
+def test_library_exports_every_declared_symbol():
+    lib = native.load()
+    names = declared_symbols()
+    assert len(names) >= 18
+    for name in names:
+        assert hasattr(lib, name), name
+    assert sorted(native.EXPORTS) == names
+
+
+def test_abi_versions_and_kernel_table():
+    lib = native.load()
+    assert lib.ca_ffn_abi() == 1 and lib.ca_primitives_abi() == 1
+    names = native.kernel_names()
+    for required in ["ca_route_padding_rows", "ca_ffn_sum_shared", "ca_moe_group_sum_rows", "ca_moe_frontend", "ca_moe_route_frontend",
+                     "ca_route_topk", "ca_route_census", "ca_expert_compact_words", "ca_expert_compact_scales", "ca_expert_scale_codes4",
+                     "ca_expert_scale_code1", "ca_expert_scale_code1_check", "ca_expert_scale_code1_census", "ca_shared_swiglu_quant"]:
+        assert required in names, required        # the names the reference resolves from its code modules (src/ffn.rs, src/expert_packing.rs)
+    assert lib.ca_kernel_name(len(names)) is None
+
+
+def test_contracts_match_the_entry_table():
+    lib = native.load()
+    b = contracts.bindings(native.KERNEL_LIB)
+    assert len(b["entries"]) == lib.ca_primitives_entries()
+    assert [e["index"] for e in b["entries"]] == list(range(len(b["entries"])))
+    # the node sequence the reference's workspace admits (src/moe.rs:378-383)
+    c = contracts.runtime_contract(contracts.BENCHMARK_GEOMETRY, 4, native.KERNEL_LIB)
+    assert [n["kernel_id"] for n in c["nodes"]] == ["integration.tp_moe.dynamic", "moe.w4a16.topk_sum"]
+    assert c["scratch_initializer"] == "zero" and c["deterministic"] and c["swiglu_limit"] == 10.0
+    node = c["nodes"][0]
+    assert sorted(node["pointers"]) == sorted(b["entries"][0]["pointers"]) and sorted(node["scalars"]) == sorted(b["entries"][0]["i32_scalars"])
+    for p in node["pointers"].values():
+        assert p["role"] in {"input", "ids", "routing_weights", "scratch", "w13", "s13", "w2", "s2"}
+        assert p["role"] != "scratch" or p["offset"] < c["scratch_bytes"]
+    assert node["scalars"]["rows_padded"] == node["scalars"]["max_phys_tiles"] * node["scalars"]["tile_m"]
+    committed = os.path.join(ROOT, "titanic-flash-41_amd", "contracts", "bindings.json")
+    if os.path.exists(committed):
+        on_disk = json.load(open(committed))
+        assert [(e["kernel_id"], e["pointers"], e["i32_scalars"]) for e in on_disk["entries"]] == \
+               [(e["kernel_id"], e["pointers"], e["i32_scalars"]) for e in b["entries"]]
+
+
+def test_argument_validation_needs_no_device():
+    lib = native.load()
+    bad = native.Geometry(1000, 16, 2, 512, 512, 0, 1.0, 128, 128, 128, -1, 10.0)
+    assert lib.ca_ffn_configure(ctypes.byref(bad)) == -4
+    assert lib.ca_ffn_configure(None) == -1
+    good = native.Geometry(1024, 16, 2, 512, 512, 0, 1.0, 128, 128, 128, -1, 10.0)
+    assert lib.ca_ffn_configure(ctypes.byref(good)) == 0
+    back = native.Geometry()
+    assert lib.ca_ffn_geometry(ctypes.byref(back)) == 0 and (back.hidden, back.experts, back.act_block) == (1024, 16, 128)
+    assert lib.ca_router_logits(0, None, None, None, None) == -1 and lib.ca_router_logits(17, None, None, None, None) == -1
+    assert lib.ca_shared_swiglu(0, None, None, None) == -1 and lib.ca_ffn_add(70000, None, None, None, None) == -1
+    assert lib.ca_moe_nibble_permute(None, 16, 0, None) == -1
+    assert lib.ca_primitives_launch(None, 0, None, 0, None, 0, None) == -1
+    grid = (ctypes.c_uint32 * 3)(1, 1, 1)
+    assert lib.ca_kernel_launch(b"no_such_kernel", grid, grid, 0, (ctypes.c_void_p * 1)(), None) == -3
+
+
+def test_host_library_loads_and_reports_a_missing_kernel_library():
+    host = pkg.host
+    lib = host.load()
+    err = ctypes.create_string_buffer(256)
+    g = native.Geometry(1024, 16, 2, 512, 512, 0, 1.0, 128, 128, 128, -1, 10.0)
+    ptrs = (ctypes.c_void_p * 11)()
+    handle = lib.tfh_layer_create(b"/nonexistent/libtitanic_moe_hip.so", ctypes.byref(g), 4, ptrs, 0, 1, 1, 1, 0, 1, 1, err, 256)
+    assert not handle and b"load kernel library" in err.value

@@ -7,33 +7,31 @@
 // logits[m][e] = sum_k x[m][k] * w[e][k], BF16 inputs, FP32 accumulate, for one expert by one wave.
 // Fixed summation order: lane l accumulates the 8-element vectors at k = 512 j + 8 l (j ascending) with fma in k order,
 // then the 64 partials are combined by the xor butterfly 32, 16, 8, 4, 2, 1.  hidden % 512 == 0, hidden <= 8192.
-// The expert's row is requested whole before any use, and the token rows four at a time.
+// Loads are issued sixteen at a time (four vectors of the expert's row, four of each of four token rows).
 __device__ __forceinline__ void tf_logits_expert(const uint16_t* __restrict__ x, const uint16_t* __restrict__ w, float* __restrict__ out,
                                                  int rows, int hidden, int experts, int e, int lane) {
     const int nj = hidden >> 9;
-    u4v wv[16];
     const u4v* wrow = reinterpret_cast<const u4v*>(w + (size_t)e * hidden);
-#pragma unroll
-    for (int j = 0; j < 16; ++j) if (j < nj) wv[j] = wrow[j * 64 + lane];
     for (int m0 = 0; m0 < rows; m0 += 4) {
         float acc[4] = {0.f, 0.f, 0.f, 0.f};
+        for (int j0 = 0; j0 < nj; j0 += 4) {                 // four vectors of the expert and of four rows in flight
+            u4v wv[4], xv[4][4];
 #pragma unroll
-        for (int half = 0; half < 2; ++half) {               // eight vectors of four rows in flight
-            u4v xv[4][8];
-#pragma unroll
-            for (int r = 0; r < 4; ++r)
-#pragma unroll
-                for (int j = 0; j < 8; ++j)
-                    if (m0 + r < rows && half * 8 + j < nj) xv[r][j] = reinterpret_cast<const u4v*>(x + (size_t)(m0 + r) * hidden)[(half * 8 + j) * 64 + lane];
+            for (int j = 0; j < 4; ++j) if (j0 + j < nj) wv[j] = wrow[(j0 + j) * 64 + lane];
 #pragma unroll
             for (int r = 0; r < 4; ++r)
 #pragma unroll
-                for (int j = 0; j < 8; ++j)
-                    if (m0 + r < rows && half * 8 + j < nj) {
+                for (int j = 0; j < 4; ++j)
+                    if (m0 + r < rows && j0 + j < nj) xv[r][j] = reinterpret_cast<const u4v*>(x + (size_t)(m0 + r) * hidden)[(j0 + j) * 64 + lane];
+#pragma unroll
+            for (int r = 0; r < 4; ++r)
+#pragma unroll
+                for (int j = 0; j < 4; ++j)
+                    if (m0 + r < rows && j0 + j < nj) {
 #pragma unroll
                         for (int i = 0; i < 4; ++i) {
-                            acc[r] = __fmaf_rn(tf_bf16_lo(xv[r][j][i]), tf_bf16_lo(wv[half * 8 + j][i]), acc[r]);
-                            acc[r] = __fmaf_rn(tf_bf16_hi(xv[r][j][i]), tf_bf16_hi(wv[half * 8 + j][i]), acc[r]);
+                            acc[r] = __fmaf_rn(tf_bf16_lo(xv[r][j][i]), tf_bf16_lo(wv[j][i]), acc[r]);
+                            acc[r] = __fmaf_rn(tf_bf16_hi(xv[r][j][i]), tf_bf16_hi(wv[j][i]), acc[r]);
                         }
                     }
         }

@@ -32,7 +32,7 @@ def load():
         lib.tfh_layer_destroy.restype = None
         lib.tfh_layer_set_tokens.argtypes = [vp, vp, ctypes.c_int, vp, cp, sz]
         lib.tfh_layer_run.argtypes = [vp, ctypes.c_uint64, cp, sz]
-        lib.tfh_layer_capture.argtypes = [vp, ctypes.c_uint64, cp, sz]
+        lib.tfh_layer_capture.argtypes = [vp, ctypes.POINTER(ctypes.c_uint64), ctypes.c_int, cp, sz]
         lib.tfh_layer_time.argtypes = [vp, ctypes.POINTER(ctypes.c_int), ctypes.c_int, ctypes.c_int, ctypes.c_int, ctypes.POINTER(ctypes.c_float), cp, sz]
         lib.tfh_layer_time_phase.argtypes = [vp, ctypes.c_int, ctypes.c_uint64, ctypes.c_int, ctypes.POINTER(ctypes.c_float), cp, sz]
         lib.tfh_layer_profile_step.argtypes = [vp, ctypes.c_uint64, ctypes.POINTER(ctypes.c_float), cp, sz]
@@ -91,9 +91,12 @@ class Layer:
         assert x.is_cuda and x.is_contiguous() and x.numel() == self.rows * self.g.hidden
         self._check(self.lib.tfh_layer_run(self.h, x.data_ptr(), self._err, 512))
 
-    def capture(self, x):
-        assert x.is_cuda and x.is_contiguous()
-        return self._check(self.lib.tfh_layer_capture(self.h, x.data_ptr(), self._err, 512))
+    def capture(self, xs):
+        """Captures one pass over each tensor of `xs` (or the single tensor `xs`), in order, into one graph."""
+        xs = [xs] if not isinstance(xs, (list, tuple)) else list(xs)
+        assert all(x.is_cuda and x.is_contiguous() for x in xs)
+        ptrs = (ctypes.c_uint64 * len(xs))(*[x.data_ptr() for x in xs])
+        return self._check(self.lib.tfh_layer_capture(self.h, ptrs, len(xs), self._err, 512))
 
     def time(self, order, warmup, steps):
         ms = ctypes.c_float(0)

@@ -67,13 +67,18 @@ int tfh_layer_run(void* handle, uint64_t input, char* error, size_t error_len) {
         h->stream->synchronize();
     });
 }
-// Captures one pass into a graph (src/probe.rs:1527-1542 replays the layer the same way); returns the graph's index.
-int tfh_layer_capture(void* handle, uint64_t input, char* error, size_t error_len) {
+// Captures one pass over each of `count` inputs, in order, into one graph (the reference captures its whole forward, forty
+// layers' passes, into one graph and replays it: src/probe.rs:1527-1542, src/cuda.rs:2068-2153); returns the graph's index.
+int tfh_layer_capture(void* handle, const uint64_t* inputs, int count, char* error, size_t error_len) {
     Handle* h = (Handle*)handle;
     int index = -1;
     const int status = guarded(error, error_len, [&] {
+        tf::ensure(count >= 1, "capture needs an input");
         auto graph = std::make_unique<tf::Graph>();
-        graph->capture(*h->stream, [&] { h->layer->run(*h->workspace, input, h->rows * (size_t)h->native->geometry().hidden, *h->tokens, *h->stream); });
+        graph->capture(*h->stream, [&] {
+            for (int i = 0; i < count; ++i)
+                h->layer->run(*h->workspace, inputs[i], h->rows * (size_t)h->native->geometry().hidden, *h->tokens, *h->stream);
+        });
         h->graphs.push_back(std::move(graph));
         index = (int)h->graphs.size() - 1;
     });
