@@ -30,13 +30,18 @@ CONFIGS = {
                workload="decode step, 4 requests x 1 token; H 4096, E 256, top-6, I 2048, 1 shared expert (I 2048)"),
     "c3": dict(rows=32, hidden=4096, experts=256, topk=6, inter=2048, shared=2048,
                workload="speculative verify, 4 requests x 8 draft tokens = 32 rows; H 4096, E 256, top-6, I 2048, 1 shared expert"),
+    "c4": dict(rows=4096, hidden=4096, experts=256, topk=6, inter=2048, shared=2048,
+               workload="prefill chunk of 4096 tokens, uniform routing; H 4096, E 256, top-6, I 2048, 1 shared expert"),
+    "c5": dict(rows=16384, hidden=4096, experts=256, topk=6, inter=2048, shared=2048,
+               workload="long prefill of 16384 tokens, Zipf(1.1) expert popularity; H 4096, E 256, top-6, I 2048, 1 shared expert"),
 }
+MFMA_FP8_PEAK_TFLOPS, MFMA_FP4_PEAK_TFLOPS = 5000.0, 10100.0
 
 
-def make_inputs(synth, name, cfg, device):
+def make_inputs(synth, name, cfg, device, batches=BATCHES):
     import torch
     xs = []
-    for step in range(BATCHES):
+    for step in range(batches):
         if name == "c3":   # tokens of a request share a base vector: correlated router logits
             base = synth.normal("c3/base.%d" % step, (4, 1, cfg["hidden"]), device=device)
             noise = synth.normal("c3/noise.%d" % step, (4, 8, cfg["hidden"]), std=0.3, device=device)
@@ -57,10 +62,10 @@ def cpu_baseline(pkg, g, ops, xs, taps_ids, budget_s=20.0):
     oracle.set_threads(threads)
     rows = xs[0].shape[0]
     done, spent = 0, 0.0
-    while done < len(xs) and (done == 0 or spent + spent / done < budget_s):
-        x = xs[done]
+    while done < 4 * len(xs) and (done == 0 or spent + spent / done < budget_s):
+        x = xs[done % len(xs)]
         # gather the operands the step touches outside the timed region (the oracle reads host memory)
-        small_ops = _HostSubset(ops, taps_ids[done], g)
+        small_ops = _HostSubset(ops, taps_ids[done % len(xs)], g)
         t0 = time.perf_counter()
         helpers.oracle_layer(g, small_ops, x.cpu())
         spent += time.perf_counter() - t0
@@ -118,8 +123,14 @@ def main():
     g = native.Geometry(cfg["hidden"], cfg["experts"], cfg["topk"], cfg["inter"], cfg["shared"], 0, 1.0, 128, 128, 128, -1, 10.0)
     torch.cuda.set_device(0)
     t0 = time.time()
+    wide = cfg["rows"] > 64
+    batches = 2 if wide else BATCHES
+    if wide:
+        args.steps, args.warmup, args.profile_steps = min(args.steps, 200), min(args.warmup, 20), min(args.profile_steps, 8)
     ops = synth.LayerOperands(g, args.config, device="cuda")
-    xs = make_inputs(synth, args.config, cfg, "cuda")
+    if args.config == "c5":      # expert popularity ~ rank^-1.1: the busiest experts take more than ten times the mean load
+        ops.bias = synth.zipf_bias(g.experts, 1.1, 0.06, device="cuda")
+    xs = make_inputs(synth, args.config, cfg, "cuda", batches)
     layer = host.Layer(g, ops, cfg["rows"])
     layer.set_tokens()
     setup_s = time.time() - t0
@@ -131,10 +142,10 @@ def main():
         layer.profile_step(x)
     passes = 0
     for i in range(args.profile_steps):
-        x = xs[i % BATCHES]
+        x = xs[i % batches]
         parts += np.array(layer.profile_step(x))
         passes += 1
-        if i < BATCHES:
+        if i < batches:
             ids_per_batch.append(layer.tap("ids").reshape(cfg["rows"], cfg["topk"]).copy())
             tiles_per_batch.append(int(layer.tap("tile_base")[-1]))
     parts /= passes
@@ -149,13 +160,17 @@ def main():
     step_bytes = fc1_bytes + fc2_bytes + shared_bytes + router_bytes + rows * (K + 2) * H * 2
     fc1_ms = float(parts[2])
     achieved = fc1_bytes / (fc1_ms * 1e-3) / 1e9
+    routes = float(np.mean([(ids >= 0).sum() for ids in ids_per_batch]))
+    fc1_flops, fc2_flops = routes * 2 * (2 * I) * H, routes * 2 * H * I
+    step_flops = fc1_flops + fc2_flops + rows * (6 * H * S + 2 * H * E)
+    max_load = float(np.mean([np.bincount(ids[ids >= 0].ravel(), minlength=E).max() for ids in ids_per_batch]))
 
     # whole-layer throughput: one graph holds a pass over each of the sixteen batches (as the reference's graph holds its forty
     # layers' passes); a step is one pass, so steps and warmup are rounded up to whole replays
     graph = layer.capture(xs)
     torch.cuda.synchronize()
-    replays, warm = -(-args.steps // BATCHES), -(-args.warmup // BATCHES)
-    args.steps, args.warmup = replays * BATCHES, warm * BATCHES
+    replays, warm = -(-args.steps // batches), -(-args.warmup // batches)
+    args.steps, args.warmup = replays * batches, warm * batches
     ms = layer.time([graph], warm, replays)
     torch.cuda.synchronize()
     ms_per_step = ms / args.steps
@@ -166,9 +181,16 @@ def main():
         "ms_per_step": ms_per_step, "higher_is_better": True, "scaling": "weak", "vs_baseline": None,
         "dtype": "fp4 (e2m1 weights, ue8m0 scales) x fp8 (e4m3 activations), f32 accumulate",
         "data": "synthetic", "config": {"workload": args.config + ": " + cfg["workload"], "numerics": "sigmoid top-k renormalised, 128-wide activation blocks",
-                                        "input_batches": BATCHES, "distinct_experts_per_step": distinct, "schedule": "HIP graph replay (16 passes a graph), shared expert folded into the routed experts' launches"},
-        "roofline": {"bound": "hbm", "kernel": "tf_fc1_stream<fp4> (routed FC1 + SwiGLU)", "achieved": achieved, "peak": HBM_PEAK_GBS, "unit": "GB/s",
-                     "frac": achieved / HBM_PEAK_GBS, "traffic": None, "bytes_per_launch": fc1_bytes, "avg_launch_ms": fc1_ms},
+                                        "input_batches": batches, "distinct_experts_per_step": distinct, "schedule": "HIP graph replay (%d passes a graph)" % batches},
+        "roofline": ({"bound": "mfma", "kernel": "tf_gemm<fp4, FC1> (routed FC1 + SwiGLU + FP8 requantization)",
+                      "achieved": fc1_flops / (fc1_ms * 1e-3) / 1e12, "peak": MFMA_FP8_PEAK_TFLOPS, "unit": "TFLOP/s",
+                      "frac": fc1_flops / (fc1_ms * 1e-3) / 1e12 / MFMA_FP8_PEAK_TFLOPS,
+                      "frac_of_fp4_peak": fc1_flops / (fc1_ms * 1e-3) / 1e12 / MFMA_FP4_PEAK_TFLOPS,
+                      "operands": "A = FP8 E4M3 activations, B = FP4 E2M1 weights: issues at the FP8 rate (measured)", "traffic": None,
+                      "flops_per_launch": fc1_flops, "avg_launch_ms": fc1_ms, "weight_gbs": fc1_bytes / (fc1_ms * 1e-3) / 1e9} if wide else
+                     {"bound": "hbm", "kernel": "tf_phase1_stream (routed FC1 + SwiGLU, measured alone)", "achieved": achieved, "peak": HBM_PEAK_GBS,
+                      "unit": "GB/s", "frac": achieved / HBM_PEAK_GBS, "traffic": None, "bytes_per_launch": fc1_bytes, "avg_launch_ms": fc1_ms}),
+        "step_tflops": step_flops / (ms_per_step * 1e-3) / 1e12, "busiest_expert_rows": max_load, "phys_tiles": tiles,
         "step_bytes": step_bytes, "step_gbs": step_bytes / (ms_per_step * 1e-3) / 1e9, "step_hbm_frac": step_bytes / (ms_per_step * 1e-3) / 1e9 / HBM_PEAK_GBS,
         "kernel_ms": {"router": float(parts[0]), "front_end": float(parts[1]), "fc1_swiglu": fc1_ms, "fc2": float(parts[3]),
                       "shared_expert": float(parts[4]), "sum_shared": float(parts[5]), "eager_pass": float(parts[6])},

@@ -14,6 +14,7 @@ namespace {
 ca_geometry g_geometry = {5120, 384, 6, 576, 576, 1, 1.5f, 32, 32, 32, 129264, 10.f};   // src/ffn.rs:65-66, 245-258
 
 bool supported_k(int k) { return k == 512 || k == 1024 || k == 2048 || k == 4096; }
+constexpr size_t kSyncBytes = 16384;   // arrival word + queue / dependency counters of the streaming launch
 int check_geometry(const ca_geometry& g) {
     if (g.hidden <= 0 || g.hidden % 512 || g.experts <= 0 || g.experts > 512 || g.topk <= 0 || g.topk > 8 ||
         g.topk > g.experts || g.intermediate <= 0 || g.intermediate % 512 || g.shared_intermediate <= 0 ||
@@ -29,6 +30,7 @@ struct Context {
     ca_geometry g;
     int cus;
     int stream_wgs;    // persistent workgroups of the streaming kernels
+    bool single_launch; // FC1 + FC2 + sum in one launch with in-kernel dependencies (experimental: slower than two launches so far)
 };
 
 // Phase launches of the streaming kernels; either operand set may be absent (w == nullptr).
@@ -88,7 +90,11 @@ void shared_stream_args(const Context& c, const uint64_t* p, int m, StreamArgs& 
 }
 // phases: 1 front-end (plan + quantize), 2 FC1 + SwiGLU, 4 FC2.  `sh` (may be null): the shared expert's operands (SharedPtr
 // order, its input codes taken from the front-end's shared-flavour output), folded into the same phase launches.
-int launch_dynamic(const Context& c, bool route, const uint64_t* p, const int32_t* sc, hipStream_t s, int phases = 7, const uint64_t* sh = nullptr) {
+// `sum` (may be null, needs `sh`): {routed output, layer output} device pointers and the live row count: the ordered sum and the
+// shared addition run as well (inside the single streaming launch when the shapes allow it).
+struct SumArgs { uint64_t routed_out, output; int live; uint64_t sync; };
+int launch_dynamic(const Context& c, bool route, const uint64_t* p, const int32_t* sc, hipStream_t s, int phases = 7, const uint64_t* sh = nullptr,
+                   const SumArgs* sum = nullptr) {
     const ca_geometry& g = c.g;
     const int rows = sc[S_TOKENS], tile_m = sc[S_TILE_M], groups = sc[S_GROUPS], max_tiles = sc[S_MAX_TILES];
     if (rows < 1 || rows > sc[S_MAX_ROWS] || groups < 1 || max_tiles < 1 || sc[S_ROWS_PADDED] != max_tiles * tile_m) return -1;
@@ -102,6 +108,10 @@ int launch_dynamic(const Context& c, bool route, const uint64_t* p, const int32_
     const bool few = rows <= TF_STREAM_MAX_ROWS;
     if (few ? tile_m != 16 : tile_m != TF_GEMM_TILE_M) return -1;
 
+    // single streaming launch: one unit is 16 loads a lane in both projections
+    const bool mega = c.single_launch && few && sh && sum && sum->sync && phases == 7 && (g.hidden == 1024 || g.hidden == 4096) && g.hidden == 2 * g.intermediate && g.shared_intermediate == g.intermediate;
+    const int counter_words = mega ? 8 + max_tiles + 4 + g.hidden / 64 : 0;
+    uint32_t* counters = mega ? (uint32_t*)sum->sync + 16 : nullptr;
     const uint16_t* x = (const uint16_t*)p[P_A];
     int32_t* ids = (int32_t*)p[P_IDS];
     float* weights = (float*)p[P_WEIGHTS];
@@ -122,12 +132,12 @@ int launch_dynamic(const Context& c, bool route, const uint64_t* p, const int32_
                 (const float*)p[P_BIAS], (const float*)p[P_BIAS_ALT], (const long long*)p[P_TOKENS], (const int32_t*)p[P_LIVE],
                 (const int32_t*)p[P_PADDING], rows, g.topk, g.experts, g.hidden, groups, tile_m, owner, g.act_block,
                 (uint8_t*)p[P_PACKED_MIN], (uint8_t*)p[P_SCALES_MIN], g.scoring, g.route_scale, (long long)g.alt_token,
-                (const uint16_t*)p[P_GATE_W], (uint32_t*)p[P_SYNC], logit_blocks);
+                (const uint16_t*)p[P_GATE_W], (uint32_t*)p[P_SYNC], logit_blocks, counters, counter_words);
         } else {
             ca_moe_frontend<<<quant_blocks, 512, 0, s>>>(
                 x, ids, weights, (uint8_t*)p[P_PACKED], (uint8_t*)p[P_SCALES], (int32_t*)p[P_TOKEN_MAP], (float*)p[P_TOKEN_WEIGHTS],
                 (int32_t*)p[P_TASK_EXPERT], (int32_t*)p[P_TASK_VALID], (int32_t*)p[P_TILE_BASE], rows, g.topk, g.experts, g.hidden,
-                groups, tile_m, g.act_block, (uint8_t*)p[P_PACKED_MIN], (uint8_t*)p[P_SCALES_MIN]);
+                groups, tile_m, g.act_block, (uint8_t*)p[P_PACKED_MIN], (uint8_t*)p[P_SCALES_MIN], counters, counter_words);
         }
     } else {
         if (route || !p[P_PLAN_SCRATCH]) return -1;   // wide owners route with ca_route_topk first
@@ -168,18 +178,36 @@ int launch_dynamic(const Context& c, bool route, const uint64_t* p, const int32_
             if (!supported_k(g.shared_intermediate)) return -4;
             shared_stream_args(c, sh, rows, sa, sb);
         }
-        if (phases & 2) {
-            status = launch_phase1(a, sa, c.stream_wgs, s);
-            if (status) return status;
-        }
-        if (!(phases & 4)) return 0;
         StreamArgs b = a;
         b.a_codes = nullptr; b.a_scales = nullptr; b.a_bf16 = (const uint16_t*)p[P_INTER];
         b.q_codes = (uint8_t*)p[P_INTER_CODES]; b.q_scales = (uint8_t*)p[P_INTER_SCALES]; b.min_amax = 0.f;
         b.w = (const uint8_t*)p[P_W2]; b.ws = (const uint8_t*)p[P_S2];
         b.w_expert_stride = w2_stride; b.ws_expert_stride = s2_stride;
         b.k = g.intermediate; b.out = (uint16_t*)p[P_SCATTER];
-        return launch_phase2(b, sb, c.stream_wgs, s);
+        if (mega) {
+            MegaArgs m{};
+            m.r1 = a; m.s1 = sa; m.r2 = b; m.s2 = sb;
+            m.counters = counters; m.max_tiles = max_tiles;
+            m.routes = (const uint16_t*)p[P_SCATTER]; m.shared_down = (const uint16_t*)sh[H_OUT];
+            m.routed_out = (uint16_t*)sum->routed_out; m.output = (uint16_t*)sum->output;
+            m.rows = rows; m.live = sum->live < rows ? sum->live : rows; m.topk = g.topk;
+            const size_t lds = 16 * (size_t)g.intermediate + 16 * (size_t)(g.intermediate / g.act_block);
+            // one workgroup a CU keeps every operand in registers (the 4096-wide unit does not fit twice); the grid is what is resident
+            if (g.hidden == 1024) tf_moe_stream<2, 1, 2><<<c.cus * 2, 256, lds, s>>>(m);
+            else tf_moe_stream<8, 4, 1><<<c.cus, 256, lds, s>>>(m);
+            return launch_status();
+        }
+        if (phases & 2) {
+            status = launch_phase1(a, sa, c.stream_wgs, s);
+            if (status) return status;
+        }
+        if (!(phases & 4)) return 0;
+        status = launch_phase2(b, sb, c.stream_wgs, s);
+        if (status || !sum) return status;
+        const int n = rows * g.hidden;
+        ca_ffn_sum_shared<<<(n / 8 + 255) / 256, 256, 0, s>>>((const uint16_t*)p[P_SCATTER], (const uint16_t*)sh[H_OUT], (uint16_t*)sum->routed_out,
+                                                               (uint16_t*)sum->output, n, sum->live < rows ? sum->live : rows, g.topk, g.hidden);
+        return launch_status();
     }
     if (sh) return -4;   // many rows: the shared expert runs through its own entry
     if (!p[P_INTER_CODES] || !p[P_INTER_SCALES]) return -1;
@@ -286,7 +314,7 @@ const EntryShape kEntries[] = {
     {"moe.w4a8.phase1", P_DYN_COUNT, S_DYN_COUNT},
     {"moe.w4a8.phase2", P_DYN_COUNT, S_DYN_COUNT},
     {"moe.front_end", P_DYN_COUNT, S_DYN_COUNT},
-    {"ffn.experts_with_shared", P_ROUTE_COUNT + H_COUNT - 2, S_ROUTE_COUNT},
+    {"ffn.experts_with_shared", P_ROUTE_COUNT + H_COUNT - 2 + 2, S_ROUTE_COUNT + 1},
 };
 constexpr int kEntryCount = sizeof(kEntries) / sizeof(kEntries[0]);
 
@@ -377,7 +405,8 @@ void* ca_primitives_open(int32_t* status) {
     hipError_t e = hipGetDevice(&device);
     if (e == hipSuccess) e = hipDeviceGetAttribute(&cus, hipDeviceAttributeMultiprocessorCount, device);
     if (e != hipSuccess) { *status = (int32_t)e; return nullptr; }
-    Context* c = new Context{g_geometry, cus, cus * 2};
+    Context* c = new Context{g_geometry, cus, cus * 2, false};
+    if (const char* v = std::getenv("TITANIC_MOE_SINGLE_LAUNCH")) c->single_launch = v[0] == '1';
     if (const char* v = std::getenv("TITANIC_MOE_STREAM_WGS_PER_CU")) {
         const int n = std::atoi(v);
         if (n >= 1 && n <= 8) c->stream_wgs = cus * n;
@@ -407,7 +436,11 @@ int32_t ca_primitives_launch(void* context, int32_t index, const uint64_t* point
             sh[H_A] = pointers[P_PACKED_MIN]; sh[H_AS] = pointers[P_SCALES_MIN];
             for (int i = 2; i < H_COUNT; ++i) sh[i] = pointers[P_ROUTE_COUNT + i - 2];
             if (!sh[H_A] || !sh[H_AS]) return -1;
-            return launch_dynamic(c, pointers[P_LOGITS] != 0, pointers, scalars, s, 7, sh);
+            // + routed output, layer output (both or neither) and the live row count: the sum and the shared addition run too
+            const uint64_t routed_out = pointers[P_ROUTE_COUNT + H_COUNT - 2], output = pointers[P_ROUTE_COUNT + H_COUNT - 1];
+            if (!routed_out != !output) return -1;
+            const SumArgs sum{routed_out, output, scalars[S_ROUTE_COUNT], pointers[P_SYNC]};
+            return launch_dynamic(c, pointers[P_LOGITS] != 0, pointers, scalars, s, 7, sh, output ? &sum : nullptr);
         }
         default: return -3;
     }

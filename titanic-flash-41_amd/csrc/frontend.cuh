@@ -62,13 +62,15 @@ __device__ __forceinline__ void tf_quantize_span(const uint16_t* __restrict__ in
 // Route plan of at most 1,024 routes by one block (the block's first `experts` threads own one expert each).
 __device__ __forceinline__ void tf_plan_block(const int32_t* ids, const float* weights, int32_t* token_map,
                                               float* token_weights, int32_t* task_expert, int32_t* task_valid_rows,
-                                              int32_t* expert_tile_base, int pairs, int experts, int groups, int tile_m) {
-    __shared__ int32_t s_ids[1024];
+                                              int32_t* expert_tile_base, int pairs, int experts, int groups, int tile_m,
+                                              int32_t* s_ids, float* s_weights, bool preloaded) {
     __shared__ int32_t s_base[513];
     __shared__ int32_t s_wave[16];   // blocks of at most 1,024 threads
     const int t = threadIdx.x, lane = t & 63, wave = t >> 6;
-    for (int p = t; p < pairs; p += blockDim.x) s_ids[p] = ids[p];
-    __syncthreads();
+    if (!preloaded) {
+        for (int p = t; p < pairs; p += blockDim.x) { s_ids[p] = ids[p]; s_weights[p] = weights[p]; }
+        __syncthreads();
+    }
     int count = 0;
     if (t < experts) for (int p = 0; p < pairs; ++p) count += s_ids[p] == t;
     const int tiles = (count + tile_m - 1) / tile_m;
@@ -101,7 +103,7 @@ __device__ __forceinline__ void tf_plan_block(const int32_t* ids, const float* w
             for (int q = 0; q < p; ++q) rank += s_ids[q] == expert;
             const int row = (s_base[expert] + rank / tile_m) * tile_m + rank % tile_m;
             token_map[row] = p;
-            token_weights[row] = weights[p];
+            token_weights[row] = s_weights[p];
         }
     }
 }
@@ -113,9 +115,11 @@ __device__ __forceinline__ void tf_frontend_run(const uint16_t* input, const int
                                                 int32_t* token_map, float* token_weights, int32_t* task_expert,
                                                 int32_t* task_valid_rows, int32_t* expert_tile_base, int rows, int topk,
                                                 int experts, int cols, int groups, int tile_m, int act_block, int first) {
+    __shared__ int32_t s_ids[1024];
+    __shared__ float s_weights[1024];
     if (blockIdx.x == 0)
         tf_plan_block(ids, weights, token_map, token_weights, task_expert, task_valid_rows, expert_tile_base,
-                      rows * topk, experts, groups, tile_m);
+                      rows * topk, experts, groups, tile_m, s_ids, s_weights, false);
     if ((int)blockIdx.x < first) return;
     const long long total = (long long)rows * (cols >> 3);
     tf_quantize_span(input, packed, scales, packed_min, scales_min, total, act_block,
@@ -126,7 +130,9 @@ extern "C" __global__ void __launch_bounds__(512) ca_moe_frontend(
     const uint16_t* input, const int32_t* ids, const float* weights, uint8_t* packed, uint8_t* scales,
     int32_t* token_map, float* token_weights, int32_t* task_expert, int32_t* task_valid_rows,
     int32_t* expert_tile_base, int32_t rows, int32_t topk, int32_t experts, int32_t cols, int32_t groups,
-    int32_t tile_m, int32_t act_block, uint8_t* packed_min, uint8_t* scales_min) {
+    int32_t tile_m, int32_t act_block, uint8_t* packed_min, uint8_t* scales_min, uint32_t* counters, int32_t counter_words) {
+    if (blockIdx.x == 0 && counters != nullptr)      // the queue and dependency counters of the streaming launch that follows
+        for (int i = threadIdx.x; i < counter_words; i += blockDim.x) counters[i] = 0u;
     tf_frontend_run(input, ids, weights, packed, scales, packed_min, scales_min, token_map, token_weights, task_expert,
                     task_valid_rows, expert_tile_base, rows, topk, experts, cols, groups, tile_m, act_block, 0);
 }
@@ -141,13 +147,18 @@ extern "C" __global__ void __launch_bounds__(512) ca_moe_route_frontend(
     float* logits, const float* bias, const float* bias_alt, const long long* tokens, const int32_t* live,
     const int32_t* padding, int32_t rows, int32_t topk, int32_t experts, int32_t cols, int32_t groups, int32_t tile_m,
     int32_t owner_rows, int32_t act_block, uint8_t* packed_min, uint8_t* scales_min, int32_t scoring,
-    float route_scale, long long alt_token, const uint16_t* gate_w, uint32_t* sync, int32_t logit_blocks) {
+    float route_scale, long long alt_token, const uint16_t* gate_w, uint32_t* sync, int32_t logit_blocks, uint32_t* counters,
+    int32_t counter_words) {
+    __shared__ int32_t s_ids[1024];
+    if (blockIdx.x == 0 && counters != nullptr)      // the queue and dependency counters of the streaming launch that follows
+        for (int i = threadIdx.x; i < counter_words; i += blockDim.x) counters[i] = 0u;
+    __shared__ float s_weights[1024];
     const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6, waves = blockDim.x >> 6;
     const int first_logit_block = (int)gridDim.x - logit_blocks;
     if (gate_w != nullptr && (int)blockIdx.x >= first_logit_block) {
         const int e = ((int)blockIdx.x - first_logit_block) * waves + wave;
         if (e < experts) tf_logits_expert(input, gate_w, logits, owner_rows, cols, experts, e, lane);
-        __threadfence();
+        tf_stores_done();
         __syncthreads();
         if (threadIdx.x == 0) atomicAdd(sync, 1u);
         return;
@@ -167,17 +178,19 @@ extern "C" __global__ void __launch_bounds__(512) ca_moe_route_frontend(
             __syncthreads();
             if (!arrived)
                 for (int e = wave; e < experts; e += waves) tf_logits_expert(input, gate_w, logits, owner_rows, cols, experts, e, lane);
-            __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "agent");
+            tf_stores_done();
             __syncthreads();
         }
         const RouteParams p{experts, topk, scoring, route_scale, alt_token};
         tf_route_block(logits, bias, bias_alt, tokens, live, padding, ids, weights, owner_rows, p, 0,
-                       blockDim.x >> 6, true);
+                       blockDim.x >> 6, true, s_ids, s_weights);
     }
     if ((int)blockIdx.x >= first_logit_block) return;
     // quantizer blocks are blocks [1, first_logit_block)
     if (blockIdx.x == 0) {
-        tf_plan_block(ids, weights, token_map, token_weights, task_expert, task_valid_rows, expert_tile_base, rows * topk, experts, groups, tile_m);
+        // the executed rows are the owner's first `rows` rows, so their routes are the first rows * topk of the LDS copy
+        tf_plan_block(ids, weights, token_map, token_weights, task_expert, task_valid_rows, expert_tile_base, rows * topk, experts, groups, tile_m,
+                      s_ids, s_weights, true);
         return;
     }
     const long long total = (long long)rows * (cols >> 3);

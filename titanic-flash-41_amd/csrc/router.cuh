@@ -40,7 +40,7 @@ __device__ __forceinline__ void tf_logits_expert(const uint16_t* __restrict__ x,
             float v = acc[r];
 #pragma unroll
             for (int o = 32; o > 0; o >>= 1) v = __fadd_rn(v, __shfl_xor(v, o));
-            if (lane == 0 && m0 + r < rows) out[(size_t)(m0 + r) * experts + e] = v;
+            if (lane == 0 && m0 + r < rows) tf_publish_f32(out + (size_t)(m0 + r) * experts + e, v);   // may be read by another block of the same launch
         }
     }
 }
@@ -68,7 +68,7 @@ __device__ __forceinline__ void tf_route_row(const float* logits, const float* b
         score[i] = 0.f;
         biased[i] = -INFINITY;
         if (e < p.experts) {
-            const float x = logits[e];
+            const float x = tf_acquire_f32(logits + e);
             float s;
             if (p.scoring == 1) s = __builtin_sqrtf(x > 20.f ? x : tf_log1p_pos(tf_exp(x)));
             else s = tf_logistic(x);
@@ -118,7 +118,8 @@ __device__ __forceinline__ void tf_route_row(const float* logits, const float* b
 __device__ __forceinline__ void tf_route_block(const float* logits, const float* bias, const float* bias_alt,
                                                const long long* tokens, const int32_t* live, const int32_t* padding,
                                                int32_t* ids, float* weights, int rows, const RouteParams& p,
-                                               int first_row, int row_stride, bool apply_padding) {
+                                               int first_row, int row_stride, bool apply_padding, int32_t* s_ids = nullptr,
+                                               float* s_weights = nullptr) {
     const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
     const int n_live = min(rows, live[0]);
     for (int row = first_row + wave; row < rows; row += row_stride) {
@@ -134,6 +135,10 @@ __device__ __forceinline__ void tf_route_block(const float* logits, const float*
             if (k < p.topk && lane == k) {
                 ids[row * p.topk + k] = is_live ? chosen[k] : -1;
                 weights[row * p.topk + k] = is_live ? share[k] : 0.f;
+                if (s_ids != nullptr) {      // a copy in LDS for the plan that follows in the same block
+                    s_ids[row * p.topk + k] = is_live ? chosen[k] : -1;
+                    s_weights[row * p.topk + k] = is_live ? share[k] : 0.f;
+                }
             }
     }
     if (apply_padding) {
@@ -142,7 +147,12 @@ __device__ __forceinline__ void tf_route_block(const float* logits, const float*
         if (padding != nullptr)
             for (int i = threadIdx.x; i < rows * p.topk; i += blockDim.x) {
                 const int r = i / p.topk, s = padding[r];
-                if (s >= 0) { ids[i] = ids[s * p.topk + (i - r * p.topk)]; weights[i] = 0.f; }
+                if (s >= 0) {
+                    const int32_t from = s_ids != nullptr ? s_ids[s * p.topk + (i - r * p.topk)] : ids[s * p.topk + (i - r * p.topk)];
+                    ids[i] = from;
+                    weights[i] = 0.f;
+                    if (s_ids != nullptr) { s_ids[i] = from; s_weights[i] = 0.f; }
+                }
             }
         __syncthreads();
     }

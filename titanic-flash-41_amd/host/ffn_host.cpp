@@ -310,7 +310,7 @@ Workspace::Workspace(std::shared_ptr<const Native> native, size_t rows) : native
     add("token_map_ptr", padded * 4); add("token_weights_ptr", padded * 4);
     add("scatter_ptr", pairs * H * 2);
     add("plan_scratch_ptr", ((pairs + 63) / 64 * g.experts + pairs) * 4);
-    add("sync_ptr", 256);
+    add("sync_ptr", 16384);
     scratch_ = Buffer<uint8_t>(at);
     scratch_.zero();                                                                                          // scratch_initializer "zero", src/moe.rs:440
     output_ = Buffer<uint16_t>(rows * H);
@@ -351,9 +351,9 @@ std::optional<std::pair<uint64_t, size_t>> Workspace::run_live_for_ffn(const Exp
     ensure(expert.layout().experts == (size_t)g.experts && expert.layout().hidden == (size_t)g.hidden &&
                expert.layout().intermediate == (size_t)g.intermediate && ids.len() == rows_ * g.topk && routing_weights.len() == rows_ * g.topk,
            "MoE input shape mismatch");                                                                       // :1103-1114
-    uint64_t p[38];
+    uint64_t p[40];
     pointers(expert, input, ids, routing_weights, p);
-    int32_t scalars[7] = {(int32_t)rows_, (int32_t)rows_, (int32_t)(max_tiles_ * tile_m_), (int32_t)max_tiles_, (int32_t)tile_m_, 1, (int32_t)rows_};
+    int32_t scalars[8] = {(int32_t)rows_, (int32_t)rows_, (int32_t)(max_tiles_ * tile_m_), (int32_t)max_tiles_, (int32_t)tile_m_, 1, (int32_t)rows_, (int32_t)live};
     if (shared) {
         ensure(rows_ <= 64 && p[5] && p[6], "folded shared expert is for few-row owners");
         for (int i = 21; i < 29; ++i) p[i] = 0;
@@ -361,12 +361,16 @@ std::optional<std::pair<uint64_t, size_t>> Workspace::run_live_for_ffn(const Exp
             ensure(route->ids == p[1] && route->weights == p[2] && route->owner_rows == rows_ && route->logits && route->bias && route->live,
                    "fused routing domain");
             p[21] = route->logits; p[22] = route->bias; p[23] = route->bias_alt; p[24] = route->tokens; p[25] = route->live; p[26] = route->padding;
-            p[27] = route->gate_w; p[28] = at("sync_ptr");
+            p[27] = route->gate_w;
         }
+        p[28] = at("sync_ptr");
+        ensure((8 + max_tiles_ + 4 + g.hidden / 64 + 16) * 4 <= bytes_of("sync_ptr"), "streaming counters exceed the sync region");
         const uint64_t sh[9] = {shared->w13, shared->s13, shared->w2, shared->s2, shared->activation, shared->activation_codes,
                                 shared->activation_scales, shared->up_tap, shared->output};
         for (int i = 0; i < 9; ++i) p[29 + i] = sh[i];
-        native_->primitive(9, p, 38, scalars, 7, stream.raw(), "ffn.experts_with_shared");
+        p[38] = shared->routed_output; p[39] = shared->layer_output;
+        native_->primitive(9, p, 40, scalars, 8, stream.raw(), "ffn.experts_with_shared");
+        if (shared->layer_output) return std::nullopt;      // summed and added inside the entry
     } else if (route) {
         ensure(route->ids == p[1] && route->weights == p[2] && route->owner_rows == rows_ && route->logits && route->bias && route->live,
                "fused routing domain");                                                                       // :1266-1269
@@ -436,10 +440,12 @@ void LayerFfn::run(Workspace& workspace, uint64_t input, size_t input_len, const
     workspace.emit_shared_input(!branch);
     if (fold) {
         const SharedOperands shared{shared_w13_.values, shared_w13_.scales, shared_w2_.values, shared_w2_.scales, activation_.ptr(),
-                                    activation_codes_.ptr(), activation_scales_.ptr(), shared_up_.ptr(), shared_down_.ptr()};
+                                    activation_codes_.ptr(), activation_scales_.ptr(), shared_up_.ptr(), shared_down_.ptr(),
+                                    options_.sum_shared ? workspace.output().ptr() : 0, options_.sum_shared ? output_.ptr() : 0};
         const std::optional<RouteOperands> route = router_.run_routed(input, input_len, tokens, fused, stream, options_.gate_front);
         const auto deferred = workspace.run_live_for_ffn(expert_, input, input_len, router_.ids(), router_.routing(), tokens.active_rows(),
                                                          options_.sum_shared, route, stream, &shared);
+        if (options_.sum_shared) return;                    // the entry summed and added
         if (deferred) sum_shared(workspace, deferred->second, stream);
         else add_shared(workspace, stream);
         return;

@@ -130,7 +130,8 @@ private:
 struct RouteOperands { uint64_t logits, bias, bias_alt, tokens, live, padding, ids, weights; size_t owner_rows; uint64_t gate_w; };
 // Operands of the shared expert when it is folded into the routed experts' launches (entry "ffn.experts_with_shared"):
 // prepared w13 / scales / w2 / scales, activation (BF16), its codes and scales, the up-projection tap, the output.
-struct SharedOperands { uint64_t w13, s13, w2, s2, activation, activation_codes, activation_scales, up_tap, output; };
+// layer_output != 0: the entry also runs the ordered sum and the shared addition into routed_output / layer_output.
+struct SharedOperands { uint64_t w13, s13, w2, s2, activation, activation_codes, activation_scales, up_tap, output, routed_output, layer_output; };
 
 class Router {                                                                                      // src/ffn.rs:173-426
 public:
