@@ -107,6 +107,7 @@ int launch_dynamic(const Context& c, bool route, const uint64_t* p, const int32_
     if (need_tiles > max_tiles) return -1;
     const bool few = rows <= TF_STREAM_MAX_ROWS;
     if (few ? tile_m != 16 : tile_m != TF_GEMM_TILE_M) return -1;
+    if (few && max_tiles > TF_LDS_TILES) return -1;
 
     // single streaming launch: one unit is 16 loads a lane in both projections
     const bool mega = c.single_launch && few && sh && sum && sum->sync && phases == 7 && (g.hidden == 1024 || g.hidden == 4096) && g.hidden == 2 * g.intermediate && g.shared_intermediate == g.intermediate;
@@ -172,6 +173,7 @@ int launch_dynamic(const Context& c, bool route, const uint64_t* p, const int32_
         a.experts = g.experts; a.groups = groups; a.topk = g.topk;
         a.k = g.hidden; a.inter = g.intermediate; a.hidden = g.hidden; a.act_block = g.act_block; a.limit = g.swiglu_limit;
         a.out = (uint16_t*)p[P_INTER];
+        a.table_tiles = max_tiles;
         StreamArgs sa{}, sb{};
         if (sh) {
             for (int i = 0; i < H_COUNT; ++i) if (!sh[i] && i != H_UP_TAP && i != H_ACT_CODES && i != H_ACT_SCALES) return -1;

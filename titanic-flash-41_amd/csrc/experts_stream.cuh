@@ -153,8 +153,38 @@ struct StreamArgs {
     float limit;
     uint16_t* out;                   // FC1: BF16 intermediate [phys_row][inter]; FC2: BF16 [route or row][hidden]
     uint16_t* tap;                   // FC1 dense: BF16 projections [row][2 inter] before the activation, may be null
+    int table_tiles;                 // routed: capacity of the plan tables in tiles (phase kernels: at most TF_LDS_TILES)
 };
+// A workgroup walks the plan's tile table for every item; read in place that is three dependent round trips (tile count,
+// the tile's expert, the tile's rows) before the first weight load can be issued.  The phase kernels copy the table into
+// LDS with one round of independent loads instead (expert and row count packed in one word).
+constexpr int TF_LDS_TILES = 576;       // rows <= 64, topk <= 8, experts <= 512: at most 32 + 512 tiles
+struct PlanLds {
+    int32_t tiles;
+    uint32_t tile[TF_LDS_TILES];        // expert | valid rows << 16
+};
+// Block barrier inside.  `v` must be a routed operand set with table_tiles in [1, TF_LDS_TILES].
+__device__ __forceinline__ void tf_plan_preload(const StreamArgs& v, PlanLds& t) {
+    if (threadIdx.x == 0) t.tiles = v.expert_tile_base[v.experts];
+    for (int i = threadIdx.x; i < v.table_tiles; i += blockDim.x)
+        t.tile[i] = (uint32_t)v.task_expert[i * v.groups] | ((uint32_t)v.task_valid_rows[i * v.groups] << 16);
+    __syncthreads();
+}
 struct ItemRef { int tile, j, expert, valid; };
+__device__ __forceinline__ ItemRef tf_item(const StreamArgs& p, int item, int per_tile, const PlanLds& t) {
+    ItemRef r;
+    r.tile = item / per_tile;
+    r.j = item - r.tile * per_tile;
+    if (p.task_expert != nullptr) {
+        const uint32_t word = t.tile[r.tile];
+        r.expert = (int)(word & 0xffffu);
+        r.valid = (int)(word >> 16);
+    } else {
+        r.expert = 0;
+        r.valid = min(16, p.dense_rows - r.tile * 16);
+    }
+    return r;
+}
 __device__ __forceinline__ ItemRef tf_item(const StreamArgs& p, int item, int per_tile) {
     ItemRef r;
     r.tile = item / per_tile;
@@ -179,7 +209,8 @@ __device__ __forceinline__ int tf_tiles(const StreamArgs& p) {
 // Routed (FP4): rows [0, inter) are up, [inter, 2 inter) gate; h = bf16((g * logistic(g)) * u), g = min(gate, limit),
 // u = clamp(up) in FP32.  Shared (FP8): rows [0, inter) gate, then up; both rounded to BF16 first, clamped in BF16.
 template <bool FP8, int KS>
-__device__ __forceinline__ void tf_fc1_items(const StreamArgs& p, int item_first, int item_last, float (*red)[2][4][64]) {
+__device__ __forceinline__ void tf_fc1_items(const StreamArgs& p, int item_first, int item_last, float (*red)[2][4][64],
+                                             const PlanLds& plan) {
     const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
     const int per_tile = p.inter / 16, ks_first = wave * KS;
     if (item_first >= item_last) return;
@@ -189,7 +220,7 @@ __device__ __forceinline__ void tf_fc1_items(const StreamArgs& p, int item_first
     ATile<KS> a;
     Unit<2, KS> cur, next;
     auto load_unit = [&](Unit<2, KS>& u, int unit) {
-        const ItemRef r = tf_item(p, unit / PER_ITEM, per_tile);
+        const ItemRef r = tf_item(p, unit / PER_ITEM, per_tile, plan);
         const uint8_t* w = p.w + (size_t)r.expert * p.w_expert_stride;
         const uint8_t* ws = p.ws + (size_t)r.expert * p.ws_expert_stride;
         if constexpr (FP8) {
@@ -204,7 +235,7 @@ __device__ __forceinline__ void tf_fc1_items(const StreamArgs& p, int item_first
     v4f first_acc = {0.f, 0.f, 0.f, 0.f};
     for (int unit = unit_first; unit < unit_last; ++unit) {
         const int item = unit / PER_ITEM;
-        const ItemRef r = tf_item(p, item, per_tile);
+        const ItemRef r = tf_item(p, item, per_tile, plan);
         if (r.tile != loaded_tile) {
             long long row = -1;
             if ((lane & 15) < r.valid)
@@ -268,16 +299,18 @@ __device__ __forceinline__ void tf_fc1_items(const StreamArgs& p, int item_first
 // as the A operand.  Routed: out[route][c] = bf16(acc * token_weight); dense: out[row][c] = bf16(acc).
 template <bool FP8, int KS>
 __device__ __forceinline__ void tf_fc2_items(const StreamArgs& p, int item_first, int item_last, float (*red)[2][4][64],
-                                             uint8_t* s_codes, uint8_t* s_scales) {
+                                             uint8_t* s_codes, uint8_t* s_scales, const PlanLds& plan) {
     const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
     constexpr int COLS = FP8 ? 32 : 64, NT = COLS / 16;
     const int per_tile = p.hidden / COLS, ks_first = wave * KS;
     if (item_first >= item_last) return;
     int loaded_tile = -1;
+    int route[4] = {0, 0, 0, 0};
+    float share[4] = {0.f, 0.f, 0.f, 0.f};
     ATile<KS> a;
     Unit<4, KS> cur, next;
     auto load_unit = [&](Unit<4, KS>& u, int item) {
-        const ItemRef r = tf_item(p, item, per_tile);
+        const ItemRef r = tf_item(p, item, per_tile, plan);
         const uint8_t* w = p.w + (size_t)r.expert * p.w_expert_stride;
         const uint8_t* ws = p.ws + (size_t)r.expert * p.ws_expert_stride;
         if constexpr (FP8) {
@@ -290,8 +323,15 @@ __device__ __forceinline__ void tf_fc2_items(const StreamArgs& p, int item_first
     };
     load_unit(cur, item_first);
     for (int item = item_first; item < item_last; ++item) {
-        const ItemRef r = tf_item(p, item, per_tile);
+        const ItemRef r = tf_item(p, item, per_tile, plan);
         if (r.tile != loaded_tile) {
+            if (p.task_expert != nullptr) {      // where rows 4 (lane / 16) + i of the tile go, and their weights
+#pragma unroll
+                for (int i = 0; i < 4; ++i) {
+                    const int m = 4 * (lane >> 4) + i;
+                    if (m < r.valid) { route[i] = p.token_map[r.tile * 16 + m]; share[i] = p.token_weights[r.tile * 16 + m]; }
+                }
+            }
             __syncthreads();
             // quantize rows [0, valid) of the tile: 8 values a lane-step, groups of act_block / 8 lanes
             const int per_row = p.k >> 3, group_lanes = p.act_block >> 3;
@@ -336,8 +376,7 @@ __device__ __forceinline__ void tf_fc2_items(const StreamArgs& p, int item_first
                     for (int w2 = 1; w2 < 4; ++w2) acc = __fadd_rn(acc, slot[w2][which][i][lane]);
                     const int col = COLS * r.j + 16 * wave + (lane & 15);
                     if (p.task_expert != nullptr) {
-                        const int phys = r.tile * 16 + m;
-                        p.out[(size_t)p.token_map[phys] * p.hidden + col] = tf_to_bf16(__fmul_rn(acc, p.token_weights[phys]));
+                        p.out[(size_t)route[i] * p.hidden + col] = tf_to_bf16(__fmul_rn(acc, share[i]));
                     } else {
                         p.out[(size_t)(r.tile * 16 + m) * p.hidden + col] = tf_to_bf16(acc);
                     }
@@ -355,28 +394,32 @@ __device__ __forceinline__ void tf_fc2_items(const StreamArgs& p, int item_first
 template <int KSR, int KSS>
 __global__ void __launch_bounds__(256, 2) tf_phase1_stream(const StreamArgs routed, const StreamArgs shared) {
     __shared__ float red[8][2][4][64];
-    const long long r_items = routed.w ? (long long)tf_tiles(routed) * (routed.inter / 16) : 0;
+    __shared__ PlanLds plan;
+    if (routed.w) tf_plan_preload(routed, plan);
+    const long long r_items = routed.w ? (long long)plan.tiles * (routed.inter / 16) : 0;
     const long long s_units = shared.w ? (long long)tf_tiles(shared) * (shared.inter / 16) * 2 : 0;
     const long long total = r_items + s_units;
     const long long lo = total * blockIdx.x / gridDim.x, hi = total * (blockIdx.x + 1) / gridDim.x;
-    if (lo < r_items) tf_fc1_items<false, KSR>(routed, (int)lo, (int)(hi < r_items ? hi : r_items), red);
+    if (lo < r_items) tf_fc1_items<false, KSR>(routed, (int)lo, (int)(hi < r_items ? hi : r_items), red, plan);
     if (hi > r_items) {
         const long long a = (lo > r_items ? lo - r_items : 0), b = hi - r_items;
         __syncthreads();
-        tf_fc1_items<true, KSS>(shared, (int)((a + 1) / 2), (int)((b + 1) / 2), red);
+        tf_fc1_items<true, KSS>(shared, (int)((a + 1) / 2), (int)((b + 1) / 2), red, plan);
     }
 }
 template <int KSR, int KSS>
 __global__ void __launch_bounds__(256, 2) tf_phase2_stream(const StreamArgs routed, const StreamArgs shared) {
     __shared__ float red[8][2][4][64];
     extern __shared__ uint8_t dyn[];
-    const long long r_items = routed.w ? (long long)tf_tiles(routed) * (routed.hidden / 64) : 0;
+    __shared__ PlanLds plan;
+    if (routed.w) tf_plan_preload(routed, plan);
+    const long long r_items = routed.w ? (long long)plan.tiles * (routed.hidden / 64) : 0;
     const long long s_items = shared.w ? (long long)tf_tiles(shared) * (shared.hidden / 32) : 0;
     const long long total = r_items + s_items;
     const long long lo = total * blockIdx.x / gridDim.x, hi = total * (blockIdx.x + 1) / gridDim.x;
     const int kmax = routed.w && (!shared.w || routed.k > shared.k) ? routed.k : shared.k;
-    if (lo < r_items) tf_fc2_items<false, KSR>(routed, (int)lo, (int)(hi < r_items ? hi : r_items), red, dyn, dyn + 16 * (size_t)kmax);
-    if (hi > r_items) tf_fc2_items<true, KSS>(shared, (int)(lo > r_items ? lo - r_items : 0), (int)(hi - r_items), red, dyn, dyn + 16 * (size_t)kmax);
+    if (lo < r_items) tf_fc2_items<false, KSR>(routed, (int)lo, (int)(hi < r_items ? hi : r_items), red, dyn, dyn + 16 * (size_t)kmax, plan);
+    if (hi > r_items) tf_fc2_items<true, KSS>(shared, (int)(lo > r_items ? lo - r_items : 0), (int)(hi - r_items), red, dyn, dyn + 16 * (size_t)kmax, plan);
 }
 
 // ---- One persistent launch for FC1 + SwiGLU, FC2 and the ordered sum (few rows) ---------------------------------------------
