@@ -8,9 +8,13 @@ expert, ordered sum + shared addition) over one batch of synthetic token rows th
 as a captured HIP graph as the reference replays its layer (src/probe.rs:1527-1542).  Sixteen distinct input batches
 are cycled so every step routes to other experts and streams their weights from HBM, not from the last step's cache.
 
-Prints one JSON line: whole-layer tokens/s, the roofline of the dominant kernel (routed FC1 + SwiGLU; algorithmic bytes
-over its average duration, measured with HIP events on its launch stream), and the CPU baseline (the C oracle, a port
-of the reference semantics: the reference has no CPU path) timed on a bounded sample of the same workload.
+Prints one JSON line: whole-layer tokens/s, the roofline of the dominant kernel (FC1 + SwiGLU of the routed experts and
+the shared expert, one launch; algorithmic bytes over its average duration, measured with HIP events recorded between
+the launches on the launch stream), and the CPU baseline (the C oracle, a port of the reference semantics: the
+reference has no CPU path) timed on a bounded sample of the same workload.
+
+--copy-probe appends four plain device copies of 256 MiB after the timed region: a counter run (rocprofv3 --pmc
+FETCH_SIZE / WRITE_SIZE) then holds a kernel of known traffic to scale the counters by.
 """
 import argparse
 import importlib
@@ -36,6 +40,11 @@ CONFIGS = {
                workload="long prefill of 16384 tokens, Zipf(1.1) expert popularity; H 4096, E 256, top-6, I 2048, 1 shared expert"),
 }
 MFMA_FP8_PEAK_TFLOPS, MFMA_FP4_PEAK_TFLOPS = 5000.0, 10100.0
+# Measured HBM traffic of the dominant kernel over its algorithmic bytes, from the counter runs summarized under profiles/
+# (rocprofv3 --pmc FETCH_SIZE, then WRITE_SIZE, on tf_layer_probe: the same geometry, rows and schedule with random operands;
+# each counter scaled by its reading for a 256 MiB copy kernel).  The line's `traffic` is this ratio times the algorithmic
+# bytes of this run's launches; None where no counter run exists for the configuration.
+TRAFFIC_OVER_ALGORITHMIC = {"c2": 1.008}
 
 
 def make_inputs(synth, name, cfg, device, batches=BATCHES):
@@ -109,6 +118,7 @@ def main():
     ap.add_argument("--warmup", type=int, default=200)
     ap.add_argument("--config", default="c2", choices=sorted(CONFIGS))
     ap.add_argument("--no-cpu-baseline", action="store_true")
+    ap.add_argument("--copy-probe", action="store_true", help="append four 256 MiB device copies (counter calibration)")
     ap.add_argument("--profile-steps", type=int, default=64, help="eager passes with per-kernel HIP events for the roofline")
     args = ap.parse_args()
     if args.gpus != 1:
@@ -138,17 +148,29 @@ def main():
     # per-kernel durations (HIP events on the launch stream) and the routing of every batch
     ids_per_batch, parts = [], np.zeros(7)
     tiles_per_batch = []
-    for x in xs:                      # warm every batch once
-        layer.profile_step(x)
-    passes = 0
-    for i in range(args.profile_steps):
-        x = xs[i % batches]
-        parts += np.array(layer.profile_step(x))
-        passes += 1
-        if i < batches:
+    if wide:
+        # many rows: one eager pass at a time, events around each part (router, front-end, FC1, FC2, shared expert, sum)
+        for x in xs:                      # warm every batch once
+            layer.profile_step(x)
+        passes = 0
+        for i in range(args.profile_steps):
+            x = xs[i % batches]
+            parts += np.array(layer.profile_step(x))
+            passes += 1
+            if i < batches:
+                ids_per_batch.append(layer.tap("ids").reshape(cfg["rows"], cfg["topk"]).copy())
+                tiles_per_batch.append(int(layer.tap("tile_base")[-1]))
+        parts /= passes
+    else:
+        # few rows: the schedule of the timed region itself (front-end, FC1 and FC2 with the shared expert inside, sum), eager,
+        # every pass enqueued before the first wait, the library's marks between the launches
+        for x in xs:
+            layer.run(x)
             ids_per_batch.append(layer.tap("ids").reshape(cfg["rows"], cfg["topk"]).copy())
             tiles_per_batch.append(int(layer.tap("tile_base")[-1]))
-    parts /= passes
+        layer.profile_marks(xs, batches)
+        front, fc1, fc2, total, whole = layer.profile_marks(xs, max(args.profile_steps, batches) * 4)
+        parts = np.array([0.0, front, fc1, fc2, 0.0, total, whole])
     H, I, S, E, K, rows = cfg["hidden"], cfg["inter"], cfg["shared"], cfg["experts"], cfg["topk"], cfg["rows"]
     distinct = float(np.mean([len(set(ids.ravel().tolist())) for ids in ids_per_batch]))
     tiles = float(np.mean(tiles_per_batch))
@@ -158,8 +180,13 @@ def main():
     shared_bytes = 3 * H * S + rows * (H + 2 * S * 2 + S * 2 + H * 2)
     router_bytes = 2 * E * H + rows * H * 2
     step_bytes = fc1_bytes + fc2_bytes + shared_bytes + router_bytes + rows * (K + 2) * H * 2
+    # few rows: the shared expert's projections stream inside the same two launches
+    shared_fc1_bytes = 2 * S * H + (2 * S // 128) * (H // 128) + rows * (H + H // 128) + rows * S * 2
+    shared_fc2_bytes = H * S + (H // 128) * (S // 128) + rows * S * 2 + rows * H * 2
+    phase1_bytes = fc1_bytes + (0 if wide else shared_fc1_bytes)
+    phase2_bytes = fc2_bytes + (0 if wide else shared_fc2_bytes)
     fc1_ms = float(parts[2])
-    achieved = fc1_bytes / (fc1_ms * 1e-3) / 1e9
+    achieved = phase1_bytes / (fc1_ms * 1e-3) / 1e9
     routes = float(np.mean([(ids >= 0).sum() for ids in ids_per_batch]))
     fc1_flops, fc2_flops = routes * 2 * (2 * I) * H, routes * 2 * H * I
     step_flops = fc1_flops + fc2_flops + rows * (6 * H * S + 2 * H * E)
@@ -188,17 +215,25 @@ def main():
                       "frac_of_fp4_peak": fc1_flops / (fc1_ms * 1e-3) / 1e12 / MFMA_FP4_PEAK_TFLOPS,
                       "operands": "A = FP8 E4M3 activations, B = FP4 E2M1 weights: issues at the FP8 rate (measured)", "traffic": None,
                       "flops_per_launch": fc1_flops, "avg_launch_ms": fc1_ms, "weight_gbs": fc1_bytes / (fc1_ms * 1e-3) / 1e9} if wide else
-                     {"bound": "hbm", "kernel": "tf_phase1_stream (routed FC1 + SwiGLU, measured alone)", "achieved": achieved, "peak": HBM_PEAK_GBS,
-                      "unit": "GB/s", "frac": achieved / HBM_PEAK_GBS, "traffic": None, "bytes_per_launch": fc1_bytes, "avg_launch_ms": fc1_ms}),
+                     {"bound": "hbm", "kernel": "tf_phase1_stream (FC1 + SwiGLU of the routed experts and the shared expert in one launch)",
+                      "achieved": achieved, "peak": HBM_PEAK_GBS, "unit": "GB/s", "frac": achieved / HBM_PEAK_GBS,
+                      "traffic": (TRAFFIC_OVER_ALGORITHMIC[args.config] * phase1_bytes if args.config in TRAFFIC_OVER_ALGORITHMIC else None),
+                      "bytes_per_launch": phase1_bytes, "avg_launch_ms": fc1_ms}),
         "step_tflops": step_flops / (ms_per_step * 1e-3) / 1e12, "busiest_expert_rows": max_load, "phys_tiles": tiles,
         "step_bytes": step_bytes, "step_gbs": step_bytes / (ms_per_step * 1e-3) / 1e9, "step_hbm_frac": step_bytes / (ms_per_step * 1e-3) / 1e9 / HBM_PEAK_GBS,
         "kernel_ms": {"router": float(parts[0]), "front_end": float(parts[1]), "fc1_swiglu": fc1_ms, "fc2": float(parts[3]),
                       "shared_expert": float(parts[4]), "sum_shared": float(parts[5]), "eager_pass": float(parts[6])},
-        "kernel_gbs": {"fc2": fc2_bytes / (float(parts[3]) * 1e-3) / 1e9, "shared_expert": shared_bytes / (float(parts[4]) * 1e-3) / 1e9},
+        "kernel_gbs": {"fc2": phase2_bytes / (float(parts[3]) * 1e-3) / 1e9},
         "setup_s": setup_s,
     }
     if not args.no_cpu_baseline:
         line["cpu_baseline"] = cpu_baseline(pkg, g, ops, xs, ids_per_batch)
+    if args.copy_probe:
+        src = torch.empty(256 << 20, dtype=torch.uint8, device="cuda").random_(0, 255)
+        dst = torch.empty_like(src)
+        for _ in range(4):
+            dst.copy_(src)
+        torch.cuda.synchronize()
     layer.close()
     print(json.dumps(line))
 

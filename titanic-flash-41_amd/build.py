@@ -3,6 +3,7 @@
   libtitanic_moe_hip.so      kernels + the C ABI of include/titanic_moe.h
   titanic_moe_gfx950.hsaco   the same kernels as a code object for hosts that load modules by name
   libtitanic_ffn_host.so     the C++ host mirror of the reference's Rust FFN operators (needs only the HIP runtime)
+  tf_layer_probe             stand-alone driver of the layer for profilers (no Python in the process)
 """
 import os
 import subprocess
@@ -14,6 +15,7 @@ HOST = os.path.join(HERE, "host")
 KERNEL_LIB = os.path.join(HERE, "libtitanic_moe_hip.so")
 CODE_OBJECT = os.path.join(HERE, "titanic_moe_gfx950.hsaco")
 HOST_LIB = os.path.join(HERE, "libtitanic_ffn_host.so")
+PROBE = os.path.join(HERE, "tf_layer_probe")
 
 # -ffp-contract=off: bit-exact steps are written as explicit fma / mul / add.  Packed FP32 instructions stay off.
 DEVICE_FLAGS = ["-O3", "--offload-arch=gfx950", "-std=c++17", "-ffp-contract=off", "-Xclang", "-target-feature", "-Xclang",
@@ -45,8 +47,14 @@ def build_host():
     return HOST_LIB
 
 
+def build_probe():
+    src = os.path.join(HOST, "probe", "layer_probe.hip")
+    _run(["hipcc", *DEVICE_FLAGS, src, "-o", PROBE, "-L", HERE, "-ltitanic_ffn_host", "-Wl,-rpath,$ORIGIN"])
+    return PROBE
+
+
 def build():
-    return build_kernels(), build_host()
+    return build_kernels(), build_host(), build_probe()
 
 
 if __name__ == "__main__":

@@ -30,8 +30,15 @@ struct Context {
     ca_geometry g;
     int cus;
     int stream_wgs;    // persistent workgroups of the streaming kernels
+    hipEvent_t marks[5];   // profiling aid: see ca_primitives_marks
+    bool marking;
     bool single_launch; // FC1 + FC2 + sum in one launch with in-kernel dependencies (experimental: slower than two launches so far)
 };
+
+// Records mark `i` on the launch stream when the caller asked for marks (never while a stream is captured: the caller's duty).
+void mark(const Context& c, int i, hipStream_t s) {
+    if (c.marking) (void)hipEventRecord(c.marks[i], s);
+}
 
 // Phase launches of the streaming kernels; either operand set may be absent (w == nullptr).
 int launch_phase1(const StreamArgs& routed, const StreamArgs& shared, int wgs, hipStream_t s) {
@@ -113,6 +120,7 @@ int launch_dynamic(const Context& c, bool route, const uint64_t* p, const int32_
     const bool mega = c.single_launch && few && sh && sum && sum->sync && phases == 7 && (g.hidden == 1024 || g.hidden == 4096) && g.hidden == 2 * g.intermediate && g.shared_intermediate == g.intermediate;
     const int counter_words = mega ? 8 + max_tiles + 4 + g.hidden / 64 : 0;
     uint32_t* counters = mega ? (uint32_t*)sum->sync + 16 : nullptr;
+    mark(c, 0, s);
     const uint16_t* x = (const uint16_t*)p[P_A];
     int32_t* ids = (int32_t*)p[P_IDS];
     float* weights = (float*)p[P_WEIGHTS];
@@ -159,6 +167,7 @@ int launch_dynamic(const Context& c, bool route, const uint64_t* p, const int32_
     }
     int status = launch_status();
     if (status) return status;
+    mark(c, 1, s);
 
     const long long w13_stride = (long long)g.intermediate * g.hidden, s13_stride = w13_stride / 16;   // 2 I x H / 2, / 32
     const long long w2_stride = (long long)g.hidden * g.intermediate / 2, s2_stride = w2_stride / 16;
@@ -203,12 +212,15 @@ int launch_dynamic(const Context& c, bool route, const uint64_t* p, const int32_
             status = launch_phase1(a, sa, c.stream_wgs, s);
             if (status) return status;
         }
+        mark(c, 2, s);
         if (!(phases & 4)) return 0;
         status = launch_phase2(b, sb, c.stream_wgs, s);
+        mark(c, 3, s);
         if (status || !sum) return status;
         const int n = rows * g.hidden;
         ca_ffn_sum_shared<<<(n / 8 + 255) / 256, 256, 0, s>>>((const uint16_t*)p[P_SCATTER], (const uint16_t*)sh[H_OUT], (uint16_t*)sum->routed_out,
                                                                (uint16_t*)sum->output, n, sum->live < rows ? sum->live : rows, g.topk, g.hidden);
+        mark(c, 4, s);
         return launch_status();
     }
     if (sh) return -4;   // many rows: the shared expert runs through its own entry
@@ -407,7 +419,8 @@ void* ca_primitives_open(int32_t* status) {
     hipError_t e = hipGetDevice(&device);
     if (e == hipSuccess) e = hipDeviceGetAttribute(&cus, hipDeviceAttributeMultiprocessorCount, device);
     if (e != hipSuccess) { *status = (int32_t)e; return nullptr; }
-    Context* c = new Context{g_geometry, cus, cus * 2, false};
+    Context* c = new Context{};
+    c->g = g_geometry; c->cus = cus; c->stream_wgs = cus * 2;
     if (const char* v = std::getenv("TITANIC_MOE_SINGLE_LAUNCH")) c->single_launch = v[0] == '1';
     if (const char* v = std::getenv("TITANIC_MOE_STREAM_WGS_PER_CU")) {
         const int n = std::atoi(v);
@@ -416,6 +429,16 @@ void* ca_primitives_open(int32_t* status) {
     return c;
 }
 void ca_primitives_close(void* context) { delete (Context*)context; }
+int32_t ca_primitives_marks(void* context, void* const* events, size_t count) {
+    if (!context || (count != 0 && (count != 5 || !events))) return -1;
+    Context* c = (Context*)context;
+    c->marking = count == 5;
+    for (size_t i = 0; i < count; ++i) {
+        if (!events[i]) { c->marking = false; return -1; }
+        c->marks[i] = (hipEvent_t)events[i];
+    }
+    return 0;
+}
 int32_t ca_primitives_launch(void* context, int32_t index, const uint64_t* pointers, size_t np, const int32_t* scalars, size_t ns,
                              void* stream) {
     if (!context || !pointers || !scalars) return -1;

@@ -36,6 +36,7 @@ def load():
         lib.tfh_layer_time.argtypes = [vp, ctypes.POINTER(ctypes.c_int), ctypes.c_int, ctypes.c_int, ctypes.c_int, ctypes.POINTER(ctypes.c_float), cp, sz]
         lib.tfh_layer_time_phase.argtypes = [vp, ctypes.c_int, ctypes.c_uint64, ctypes.c_int, ctypes.POINTER(ctypes.c_float), cp, sz]
         lib.tfh_layer_profile_step.argtypes = [vp, ctypes.c_uint64, ctypes.POINTER(ctypes.c_float), cp, sz]
+        lib.tfh_layer_profile_marks.argtypes = [vp, ctypes.POINTER(ctypes.c_uint64), ctypes.c_int, ctypes.c_int, ctypes.POINTER(ctypes.c_float), cp, sz]
         lib.tfh_layer_tap.restype = ctypes.c_longlong
         lib.tfh_layer_tap.argtypes = [vp, cp, vp, sz, cp, sz]
         lib.tfh_layer_census.argtypes = [vp, vp, cp, sz]
@@ -113,6 +114,14 @@ class Layer:
         """Milliseconds of (router, front-end, FC1, FC2, shared expert, sum, whole pass) of one eager pass."""
         ms = (ctypes.c_float * 7)()
         self._check(self.lib.tfh_layer_profile_step(self.h, x.data_ptr(), ms, self._err, 512))
+        return list(ms)
+
+    def profile_marks(self, xs, passes):
+        """Mean milliseconds of (front-end, FC1 + SwiGLU, FC2, sum, first mark to last) over `passes` eager passes of the
+        layer's own schedule cycling through the inputs `xs`; events are recorded between the launches on the launch stream."""
+        ptrs = (ctypes.c_uint64 * len(xs))(*[x.data_ptr() for x in xs])
+        ms = (ctypes.c_float * 5)()
+        self._check(self.lib.tfh_layer_profile_marks(self.h, ptrs, len(xs), passes, ms, self._err, 512))
         return list(ms)
 
     def tap(self, name):

@@ -149,6 +149,35 @@ int tfh_layer_profile_step(void* handle, uint64_t input, float* milliseconds, ch
         milliseconds[6] = e[6]->elapsed_since(*e[0]);
     });
 }
+// `passes` eager passes of the layer's own schedule over the `count` inputs in turn, all enqueued before the first wait, with
+// the library's marks around every launch of the dynamic entry: mean milliseconds of [0] front-end (gate product, top-k, plan,
+// quantizers), [1] FC1 + SwiGLU, [2] FC2, [3] ordered sum + shared addition, [4] first mark to last.  Needs the schedule that
+// keeps the shared expert inside the routed launches (otherwise there is no sum mark).
+int tfh_layer_profile_marks(void* handle, const uint64_t* inputs, int count, int passes, float* milliseconds, char* error, size_t error_len) {
+    Handle* h = (Handle*)handle;
+    return guarded(error, error_len, [&] {
+        tf::ensure(count >= 1 && passes >= 1, "profile needs inputs and passes");
+        std::vector<std::unique_ptr<tf::Event>> events;
+        for (int i = 0; i < 5 * passes; ++i) events.push_back(std::make_unique<tf::Event>(true));
+        const size_t n = h->rows * (size_t)h->native->geometry().hidden;
+        try {
+            for (int pass = 0; pass < passes; ++pass) {
+                hipEvent_t raw[5];
+                for (int i = 0; i < 5; ++i) raw[i] = events[5 * pass + i]->raw();
+                h->native->marks(raw);
+                h->layer->run(*h->workspace, inputs[pass % count], n, *h->tokens, *h->stream);
+            }
+        } catch (...) { h->native->marks(nullptr); throw; }
+        h->native->marks(nullptr);
+        h->stream->synchronize();
+        double sum[5] = {0, 0, 0, 0, 0};
+        for (int pass = 0; pass < passes; ++pass) {
+            for (int i = 0; i < 4; ++i) sum[i] += events[5 * pass + i + 1]->elapsed_since(*events[5 * pass + i]);
+            sum[4] += events[5 * pass + 4]->elapsed_since(*events[5 * pass]);
+        }
+        for (int i = 0; i < 5; ++i) milliseconds[i] = (float)(sum[i] / passes);
+    });
+}
 // Copies a named tap to the host.  Returns the tap's size in bytes (or -1); copies min(bytes, size).
 long long tfh_layer_tap(void* handle, const char* name, void* out, size_t bytes, char* error, size_t error_len) {
     Handle* h = (Handle*)handle;

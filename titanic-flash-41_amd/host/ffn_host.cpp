@@ -31,6 +31,7 @@ Native::Native(const std::string& library, const ca_geometry& geometry) : g_(geo
     close_ = symbol<decltype(close_)>(lib_, "ca_primitives_close");
     launch_ = symbol<decltype(launch_)>(lib_, "ca_primitives_launch");
     scratch_bytes_ = symbol<decltype(scratch_bytes_)>(lib_, "ca_primitives_scratch_bytes");
+    marks_ = symbol<decltype(marks_)>(lib_, "ca_primitives_marks");
     int32_t status = 0;
     ctx_ = symbol<void* (*)(int32_t*)>(lib_, "ca_primitives_open")(&status);
     if (status != 0 || !ctx_) throw Error("initialize primitive library: " + std::to_string(status));   // src/primitives.rs:116-119
@@ -38,6 +39,9 @@ Native::Native(const std::string& library, const ca_geometry& geometry) : g_(geo
 Native::~Native() {
     if (ctx_ && close_) close_(ctx_);
     if (lib_) dlclose(lib_);
+}
+void Native::marks(hipEvent_t* events) const {
+    ensure(marks_(ctx_, (void* const*)events, events ? 5 : 0) == 0, "profiling marks rejected");
 }
 void Native::router_logits(int rows, uint64_t x, uint64_t w, uint64_t out, hipStream_t s) const {
     ensure(router_logits_(rows, (const void*)x, (const void*)w, (void*)out, s) == 0, "tiny router GPU launch failed");   // src/ffn.rs:352-363

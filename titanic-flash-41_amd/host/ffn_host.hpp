@@ -38,6 +38,8 @@ public:
     // Primitives::launch (src/primitives.rs:122-151)
     void primitive(int index, const uint64_t* pointers, size_t np, const int32_t* scalars, size_t ns, hipStream_t s, const char* what) const;
     int64_t scratch_bytes(int index, int rows) const;
+    // five events recorded around the launches of the dynamic entries (null: off)
+    void marks(hipEvent_t* events) const;
 private:
     void* lib_ = nullptr;
     void* ctx_ = nullptr;
@@ -50,6 +52,7 @@ private:
     void (*close_)(void*) = nullptr;
     int32_t (*launch_)(void*, int32_t, const uint64_t*, size_t, const int32_t*, size_t, void*) = nullptr;
     int64_t (*scratch_bytes_)(void*, int32_t, int32_t) = nullptr;
+    int32_t (*marks_)(void*, void* const*, size_t) = nullptr;
 };
 
 // ---- device atlas (src/weights.rs:276-417: contiguous expert groups, 256-byte aligned views) --------------------------

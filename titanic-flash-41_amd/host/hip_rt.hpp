@@ -39,6 +39,7 @@ public:
     void record(hipStream_t s) const { check(hipEventRecord(e_, s), "event record"); }
     void wait(hipStream_t s) const { check(hipStreamWaitEvent(s, e_, 0), "event wait"); }
     void synchronize() const { check(hipEventSynchronize(e_), "event synchronize"); }
+    hipEvent_t raw() const { return e_; }
     float elapsed_since(const Event& earlier) const { float ms = 0; check(hipEventElapsedTime(&ms, earlier.e_, e_), "elapsed"); return ms; }
 private:
     hipEvent_t e_ = nullptr;
