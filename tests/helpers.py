@@ -79,7 +79,7 @@ class GpuLayer:
         self.sh_s13, self.sh_s2 = ops.sh_s13.to(d), ops.sh_s2.to(d)
         self.tile_m = 16 if rows <= STREAM_MAX_ROWS else GEMM_TILE_M
         pairs = rows * K
-        self.max_tiles = pairs // self.tile_m + min(E, pairs)
+        self.max_tiles = -(-pairs // self.tile_m) - 1 + min(E, pairs)
         padded = self.max_tiles * self.tile_m
         z = lambda shape, dt: torch.zeros(shape, dtype=dt, device=d)
         self.logits = z((rows, E), torch.float32)

@@ -78,7 +78,7 @@ def test_wide_plan_bit_exact(rows, experts, topk, tile_m):
     weights = rng.random((rows, topk), dtype=np.float32)
     pairs = rows * topk
     waves = (pairs + 63) // 64
-    max_tiles = pairs // tile_m + min(experts, pairs)
+    max_tiles = -(-pairs // tile_m) - 1 + min(experts, pairs)
     d_ids, d_w = dev(ids), dev(weights)
     wave_counts = torch.zeros(waves * experts, dtype=torch.int32, device="cuda")
     local_rank = torch.zeros(pairs, dtype=torch.int32, device="cuda")

@@ -46,11 +46,17 @@ def align256(n):
     return (n + 255) // 256 * 256
 
 
+def max_phys_tiles(pairs, tile_m, experts):
+    """Tile capacity of a launch, as the reference's contracts state it (runtime-contract.json `max_phys_tiles`;
+    src/moe.rs:1253-1257 checks it): min(E, pairs) experts open a tile each, the other routes fill ceil(pairs / tile_m) - 1 more."""
+    return -(-pairs // tile_m) - 1 + min(experts, pairs)
+
+
 def scratch_layout(g, rows):
     """The Workspace's scratch regions (same order and formulas as tf::Workspace in host/ffn_host.cpp)."""
     tile_m = 16 if rows <= 64 else 128
     pairs = rows * g["topk"]
-    tiles = pairs // tile_m + min(g["experts"], pairs)
+    tiles = max_phys_tiles(pairs, tile_m, g["experts"])
     padded = tiles * tile_m
     H, I, B = g["hidden"], g["intermediate"], g["act_block"]
     sizes = [("packed_a_storage_ptr", rows * H), ("scale_storage_ptr", rows * H // B), ("shared_a_storage_ptr", rows * H),

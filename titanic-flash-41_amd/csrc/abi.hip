@@ -109,8 +109,9 @@ int launch_dynamic(const Context& c, bool route, const uint64_t* p, const int32_
         if (!p[i] && i != P_PACKED_MIN && i != P_SCALES_MIN && i != P_INTER_CODES && i != P_INTER_SCALES && i != P_PLAN_SCRATCH) return -1;
     if (!supported_k(g.hidden) || !supported_k(g.intermediate)) return -4;
     const long long pairs = (long long)rows * g.topk;
-    // worst case tiles: every expert opens one partial tile
-    const long long need_tiles = (pairs / tile_m) + (g.experts < pairs ? g.experts : pairs);
+    // capacity of the reference's contracts (max_phys_tiles): A = min(E, pairs) experts open a tile each and the other routes fill
+    // at most floor((pairs - A) / tile_m) <= ceil(pairs / tile_m) - 1 more
+    const long long need_tiles = (pairs + tile_m - 1) / tile_m - 1 + (g.experts < pairs ? g.experts : pairs);
     if (need_tiles > max_tiles) return -1;
     const bool few = rows <= TF_STREAM_MAX_ROWS;
     if (few ? tile_m != 16 : tile_m != TF_GEMM_TILE_M) return -1;
@@ -484,7 +485,7 @@ int64_t ca_primitives_scratch_bytes(void* context, int32_t index, int32_t rows) 
     const ca_geometry& g = ((const Context*)context)->g;
     const long long pairs = (long long)rows * g.topk;
     const int tile_m = rows <= TF_STREAM_MAX_ROWS ? 16 : TF_GEMM_TILE_M;
-    const long long tiles = pairs / tile_m + (g.experts < pairs ? g.experts : pairs), padded = tiles * tile_m;
+    const long long tiles = (pairs + tile_m - 1) / tile_m - 1 + (g.experts < pairs ? g.experts : pairs), padded = tiles * tile_m;
     long long bytes = 0;
     auto add = [&](long long n) { bytes += (n + 255) / 256 * 256; };
     add(2ll * rows * g.hidden); add(2ll * rows * g.hidden / g.act_block);              // packed + scales, both flavours

@@ -303,7 +303,7 @@ Workspace::Workspace(std::shared_ptr<const Native> native, size_t rows) : native
     ensure(rows >= 1, "MoE workspace rows");
     tile_m_ = rows <= 64 ? 16 : 128;
     const size_t pairs = rows * g.topk;
-    max_tiles_ = pairs / tile_m_ + std::min<size_t>(g.experts, pairs);
+    max_tiles_ = (pairs + tile_m_ - 1) / tile_m_ - 1 + std::min<size_t>(g.experts, pairs);   // the reference contracts' capacity (runtime-contract.json max_phys_tiles)
     const size_t padded = max_tiles_ * tile_m_, H = g.hidden, I = g.intermediate, B = g.act_block;
     size_t at = 0;
     auto add = [&](const char* name, size_t bytes) { regions_[name] = View{at, bytes}; at += align256(bytes); };
