@@ -17,6 +17,7 @@
 // for the shared expert (src/fp8_linear.rs:782-806).
 #pragma once
 #include "experts_stream.cuh"
+#include <type_traits>
 
 #define TF_STREAM_MAX_ROWS 64
 #define TF_GEMM_TILE_M 128
@@ -78,26 +79,29 @@ __global__ void __launch_bounds__(256) tf_gemm(const GemmArgs p) {
         const uint8_t* ws = p.ws + (size_t)expert * p.ws_expert_stride;
         __syncthreads();
         if (tid < 128) {
-            long long src = -1;
-            if (tid < valid) {
-                if (MODE == TF_GEMM_FC1_ROUTED) src = p.token_map[tile * 128 + tid] / p.topk;
-                else src = (long long)tile * 128 + tid;
-            }
+            // rows past the last valid one re-read the last valid row: every load of the main loop is then unconditional (the
+            // number of loads in flight is the same for every wave and k-step) and their products are never stored
+            const int t = min(tid, valid - 1);
+            long long src;
+            if (MODE == TF_GEMM_FC1_ROUTED) src = p.token_map[tile * 128 + t] / p.topk;
+            else src = (long long)tile * 128 + t;
             s_row[tid] = src;
         }
         __syncthreads();
-        // this thread's four 16-byte chunks of every k-step's A tile: chunk id c = tid + 256 i -> row c / 8, piece c % 8
+        // this thread's four 16-byte chunks of every k-step's A tile: chunk id c = tid + 256 i is LDS slot c (a wave fills one
+        // 1 KiB fragment block with consecutive 16-byte slots: no bank conflicts), i.e. fragment c / 128, K half (c / 64) % 2,
+        // row c % 16 of the fragment, 16-byte piece (c % 64) / 16 of the half
         const uint8_t* a_src[4];
         int a_dst[4];
 #pragma unroll
         for (int i = 0; i < 4; ++i) {
-            const int c = tid + 256 * i, row = c >> 3, piece = c & 7;
+            const int c = tid + 256 * i, block = c >> 6, slot = c & 63;
+            const int row = (block >> 1) * 16 + (slot & 15), piece = (block & 1) * 4 + (slot >> 4);
             const long long src = s_row[row];
-            a_src[i] = src >= 0 ? p.a_codes + src * p.k + piece * 16 : nullptr;
-            a_dst[i] = (((row >> 4) * 2 + (piece >> 2)) * 64 + (piece & 3) * 16 + (row & 15)) * 16;
+            a_src[i] = p.a_codes + src * p.k + piece * 16;
+            a_dst[i] = c * 16;
         }
-        const long long my_row = tid < 128 ? s_row[tid] : -1;
-        const uint8_t* as_src = my_row >= 0 ? p.a_scales + my_row * (p.k / p.act_block) : nullptr;
+        const uint8_t* as_src = p.a_scales + s_row[tid & 127] * (p.k / p.act_block);
         // weight row tiles of this wave: FC1 routed: up tiles then gate tiles; FC1 shared: gate tiles then up tiles
         int ntile[4];
 #pragma unroll
@@ -107,32 +111,33 @@ __global__ void __launch_bounds__(256) tf_gemm(const GemmArgs p) {
         }
         auto load_a = [&](int ks, u4v (&ra)[4], uint32_t& rs) {
 #pragma unroll
-            for (int i = 0; i < 4; ++i) ra[i] = a_src[i] ? *reinterpret_cast<const u4v*>(a_src[i] + (size_t)ks * 128) : u4v{0, 0, 0, 0};
-            rs = 0x7f7f7f7fu;
-            if (as_src) {
-                if (p.act_block == 32) rs = *reinterpret_cast<const uint32_t*>(as_src + ks * 4);
-                else rs = 0x01010101u * as_src[ks];
-            }
+            for (int i = 0; i < 4; ++i) ra[i] = *reinterpret_cast<const u4v*>(a_src[i] + (size_t)ks * 128);
+            if (p.act_block == 32) rs = *reinterpret_cast<const uint32_t*>(as_src + ks * 4);
+            else rs = 0x01010101u * as_src[ks];
         };
         auto store_a = [&](int stage, const u4v (&ra)[4], uint32_t rs) {
 #pragma unroll
             for (int i = 0; i < 4; ++i) *reinterpret_cast<u4v*>(&s_a[stage][a_dst[i]]) = ra[i];
             if (tid < 128) s_as[stage][tid] = rs;
         };
+        // B operand of one k-step: plain loads (an expert's weight slice is re-read by the expert's other tiles from this
+        // XCD's L2).  FP8: with the lane's block scale of the k-step; FP4: scales come a word per four k-steps (load_b_scales).
         auto load_b = [&](int ks, BFrag<FP8> (&b)[4], uint32_t (&sb)[4]) {
 #pragma unroll
             for (int j = 0; j < 4; ++j) {
                 if constexpr (FP8) {
                     const u4v* src = reinterpret_cast<const u4v*>(w) + (((size_t)ntile[j] * ksteps + ks) * 2) * 64 + lane;
-                    b[j].lo = tf_stream_load(src);
-                    b[j].hi = tf_stream_load(src + 64);
+                    b[j].lo = src[0];
+                    b[j].hi = src[64];
                     sb[j] = ws[(size_t)((ntile[j] * 16 + r16) / p.bn) * (p.k / p.bk) + (ks * 128 + 32 * g) / p.bk];
                 } else {
-                    b[j].lo = tf_stream_load(reinterpret_cast<const u4v*>(w) + ((size_t)ntile[j] * ksteps + ks) * 64 + lane);
-                    if ((ks & 3) == 0)
-                        sb[j] = __builtin_nontemporal_load(reinterpret_cast<const uint32_t*>(ws) + ((size_t)ntile[j] * (p.k / 512) + ks / 4) * 64 + lane);
+                    b[j].lo = reinterpret_cast<const u4v*>(w)[((size_t)ntile[j] * ksteps + ks) * 64 + lane];
                 }
             }
+        };
+        auto load_b_scales = [&](int ks, uint32_t (&sb)[4]) {
+#pragma unroll
+            for (int j = 0; j < 4; ++j) sb[j] = reinterpret_cast<const uint32_t*>(ws)[((size_t)ntile[j] * (p.k / 512) + ks / 4) * 64 + lane];
         };
         v4f acc[8][4];
 #pragma unroll
@@ -141,47 +146,70 @@ __global__ void __launch_bounds__(256) tf_gemm(const GemmArgs p) {
             for (int j = 0; j < 4; ++j) acc[f][j] = v4f{0.f, 0.f, 0.f, 0.f};
         const int frags = (valid + 15) >> 4;
 
-        u4v ra[4];
-        uint32_t rs;
-        BFrag<FP8> b[4], bn[4];
-        uint32_t sb[4] = {0, 0, 0, 0};
-        load_a(0, ra, rs);
-        load_b(0, b, sb);
-        store_a(0, ra, rs);
-        __syncthreads();
-        for (int ks = 0; ks < ksteps; ++ks) {
-            const int stage = ks & 1;
-            uint32_t sbn[4] = {sb[0], sb[1], sb[2], sb[3]};
-            if (ks + 1 < ksteps) { load_a(ks + 1, ra, rs); load_b(ks + 1, bn, sbn); }
+        // Main loop, compiled for 2, 4, 6 or 8 row fragments so that its products sit under no branch.  Operands of k-step
+        // ks + D - 1 are requested while k-step ks is multiplied (a ring of D register sets, indexed statically by unrolling
+        // D times): the token tile goes registers -> LDS one k-step ahead of its use (two LDS stages, one barrier a k-step),
+        // the weights stay in registers.
+        auto main_loop = [&](auto fr_constant) {
+            constexpr int FR = decltype(fr_constant)::value;
+            constexpr int D = FP8 ? 3 : 4;
+            u4v ra[D][4];
+            uint32_t rs[D];
+            BFrag<FP8> b[D][4];
+            uint32_t sbk[D][4];                  // FP8: the slot's scale bytes
+            uint32_t sb[4] = {0, 0, 0, 0}, sb_next[4] = {0, 0, 0, 0};   // FP4: scale words of the current / next four k-steps
 #pragma unroll
-            for (int f = 0; f < 8; ++f) {
-                if (f < frags) {
-                    const u4v lo = *reinterpret_cast<const u4v*>(&s_a[stage][((f * 2) * 64 + lane) * 16]);
-                    const u4v hi = *reinterpret_cast<const u4v*>(&s_a[stage][((f * 2 + 1) * 64 + lane) * 16]);
-                    const v8i av = v8i{(int)lo[0], (int)lo[1], (int)lo[2], (int)lo[3], (int)hi[0], (int)hi[1], (int)hi[2], (int)hi[3]};
-                    const int sa = (int)((s_as[stage][f * 16 + r16] >> (8 * g)) & 0xffu);
+            for (int d = 0; d < D - 1; ++d) {
+                if (d < ksteps) { load_a(d, ra[d], rs[d]); load_b(d, b[d], sbk[d]); }
+            }
+            if constexpr (!FP8) load_b_scales(0, sb);
+            store_a(0, ra[0], rs[0]);
+            __syncthreads();
+            for (int ks0 = 0; ks0 < ksteps; ks0 += D) {
 #pragma unroll
-                    for (int j = 0; j < 4; ++j) {
-                        v8i bv;
-                        if constexpr (FP8) bv = v8i{(int)b[j].lo[0], (int)b[j].lo[1], (int)b[j].lo[2], (int)b[j].lo[3], (int)b[j].hi[0],
-                                                    (int)b[j].hi[1], (int)b[j].hi[2], (int)b[j].hi[3]};
-                        else bv = v8i{(int)b[j].lo[0], (int)b[j].lo[1], (int)b[j].lo[2], (int)b[j].lo[3], 0, 0, 0, 0};
-                        if constexpr (FP8) {
-                            acc[f][j] = __builtin_amdgcn_mfma_scale_f32_16x16x128_f8f6f4(av, bv, acc[f][j], 0, 0, 0, sa, 0, (int)sb[j]);
-                        } else {
-                            const int sbj = (int)(sb[j] >> (8 * (ks & 3)));
-                            acc[f][j] = __builtin_amdgcn_mfma_scale_f32_16x16x128_f8f6f4(av, bv, acc[f][j], 0, 4, 0, sa, 0, sbj);
+                for (int u = 0; u < D; ++u) {
+                    const int ks = ks0 + u;
+                    if (ks < ksteps) {
+                        const int stage = ks & 1, ahead = ks + D - 1;
+                        if (ahead < ksteps) {
+                            load_a(ahead, ra[(u + D - 1) % D], rs[(u + D - 1) % D]);
+                            load_b(ahead, b[(u + D - 1) % D], sbk[(u + D - 1) % D]);
+                            if constexpr (!FP8) { if (u == 1) load_b_scales(ahead, sb_next); }       // ahead % 4 == 0 (D == 4, ksteps % 4 == 0)
                         }
+                        if constexpr (!FP8) {
+                            if (u == 0 && ks > 0) {
+#pragma unroll
+                                for (int j = 0; j < 4; ++j) sb[j] = sb_next[j];
+                            }
+                        }
+#pragma unroll
+                        for (int f = 0; f < FR; ++f) {
+                            const u4v lo = *reinterpret_cast<const u4v*>(&s_a[stage][((f * 2) * 64 + lane) * 16]);
+                            const u4v hi = *reinterpret_cast<const u4v*>(&s_a[stage][((f * 2 + 1) * 64 + lane) * 16]);
+                            const v8i av = v8i{(int)lo[0], (int)lo[1], (int)lo[2], (int)lo[3], (int)hi[0], (int)hi[1], (int)hi[2], (int)hi[3]};
+                            const int sa = (int)((s_as[stage][f * 16 + r16] >> (8 * g)) & 0xffu);
+#pragma unroll
+                            for (int j = 0; j < 4; ++j) {
+                                const BFrag<FP8>& bj = b[u][j];
+                                if constexpr (FP8) {
+                                    const v8i bv = v8i{(int)bj.lo[0], (int)bj.lo[1], (int)bj.lo[2], (int)bj.lo[3], (int)bj.hi[0], (int)bj.hi[1], (int)bj.hi[2], (int)bj.hi[3]};
+                                    acc[f][j] = __builtin_amdgcn_mfma_scale_f32_16x16x128_f8f6f4(av, bv, acc[f][j], 0, 0, 0, sa, 0, (int)sbk[u][j]);
+                                } else {
+                                    const v8i bv = v8i{(int)bj.lo[0], (int)bj.lo[1], (int)bj.lo[2], (int)bj.lo[3], 0, 0, 0, 0};
+                                    acc[f][j] = __builtin_amdgcn_mfma_scale_f32_16x16x128_f8f6f4(av, bv, acc[f][j], 0, 4, 0, sa, 0, (int)(sb[j] >> (8 * u)));
+                                }
+                            }
+                        }
+                        if (ks + 1 < ksteps) store_a(stage ^ 1, ra[(u + 1) % D], rs[(u + 1) % D]);
+                        __syncthreads();
                     }
                 }
             }
-            if (ks + 1 < ksteps) {
-                store_a(stage ^ 1, ra, rs);
-#pragma unroll
-                for (int j = 0; j < 4; ++j) { b[j] = bn[j]; sb[j] = sbn[j]; }
-            }
-            __syncthreads();
-        }
+        };
+        if (frags > 6) main_loop(std::integral_constant<int, 8>{});
+        else if (frags > 4) main_loop(std::integral_constant<int, 6>{});
+        else if (frags > 2) main_loop(std::integral_constant<int, 4>{});
+        else main_loop(std::integral_constant<int, 2>{});
 
         // ---- epilogue --------------------------------------------------------------------------------------------------
         if constexpr (FC1) {
@@ -216,9 +244,7 @@ __global__ void __launch_bounds__(256) tf_gemm(const GemmArgs p) {
                         hv[f][j][i] = value;
                         m = fmaxf(m, fabsf(value));
                     }
-#pragma unroll
-                    for (int o = 1; o < 16; o <<= 1) m = fmaxf(m, __shfl_xor(m, o));
-                    amax[f][i] = m;
+                    amax[f][i] = tf_row16_max(m);
                 }
             if (p.act_block == 128) {
 #pragma unroll

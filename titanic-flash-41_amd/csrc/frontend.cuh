@@ -21,6 +21,9 @@ __device__ __forceinline__ float tf_group_amax(const float (&v)[8], int group_la
     float amax = 0.f;
 #pragma unroll
     for (int i = 0; i < 8; ++i) amax = fmaxf(amax, fabsf(v[i]));
+    // groups are 4 lanes (32-wide blocks) or 16 lanes (128-wide blocks), aligned to their size
+    if (group_lanes == 16) return tf_row16_max(amax);
+    if (group_lanes == 4) return tf_quad_max(amax);
     for (int o = 1; o < group_lanes; o <<= 1) amax = fmaxf(amax, __shfl_xor(amax, o));
     return amax;
 }
