@@ -90,8 +90,7 @@ __device__ __forceinline__ void tf_route_row(const float* logits, const float* b
 #pragma unroll
             for (int i = 0; i < 8; ++i)
                 if (i * 64 + lane < p.experts && biased[i] == best) winner = min(winner, i * 64 + lane);
-#pragma unroll
-            for (int o = 32; o > 0; o >>= 1) winner = min(winner, __shfl_xor(winner, o));
+            winner = tf_wave_min(winner);
             float mine = 0.f;
 #pragma unroll
             for (int i = 0; i < 8; ++i)
