@@ -67,3 +67,30 @@ def test_graph_replay_matches_eager_and_oracle(config):
         check_layer(g, ops, xs[which], taps)
         layer.run(xs[1 - which])
     layer.close()
+
+
+def test_paired_owners_pool_into_one_launch():
+    # Paired::run (src/paired_ffn.rs:65-120): two owners of one layer, different live prefixes; every owner's live rows must
+    # come out exactly as when the owner runs alone (a row's arithmetic does not depend on which tile row it occupies)
+    g, ops, xa, rows = make("c1", "reference", "cpu")
+    xb = synth.activations("c1-paired-b", rows, g.hidden)
+    tokens_a, tokens_b = [5, 129264, 7, 9, 1, 2, 3, 4], [11, 12, 129264, 14, 15, 16, 17, 18]
+    live_a, live_b = 5, 3
+    layer = host.Layer(g, ops, rows, overlap=False, sum_shared=False, route_front=False, fold_shared=False)
+    alone = []
+    for x, tokens, live in [(xa, tokens_a, live_a), (xb, tokens_b, live_b)]:
+        layer.set_tokens(tokens, live=live)
+        layer.run(x.cuda())
+        alone.append(layer.tap("out").reshape(rows, g.hidden).copy())
+    xa_d, xb_d = xa.cuda(), xb.cuda()
+    out_a, out_b = layer.pair_run(xa_d, tokens_a, live_a, xb_d, tokens_b, live_b)
+    assert np.array_equal(out_a[:live_a], alone[0][:live_a]), "owner A differs from its own run"
+    assert np.array_equal(out_b[:live_b], alone[1][:live_b]), "owner B differs from its own run"
+    # and against the oracle, like any other schedule
+    from helpers import error_stats, oracle_layer
+    want = oracle_layer(g, ops, xb, tokens_b, live_b)["out"]
+    rel, mean = error_stats(out_b[:live_b], want[:live_b])
+    assert rel <= 2e-2 and mean <= 1e-3, (rel, mean)
+    with pytest.raises(host.HostError, match="paired FFN needs two live prefixes"):
+        layer.pair_run(xa_d, tokens_a, 0, xb_d, tokens_b, live_b)
+    layer.close()

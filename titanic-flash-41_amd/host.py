@@ -37,6 +37,8 @@ def load():
         lib.tfh_layer_time_phase.argtypes = [vp, ctypes.c_int, ctypes.c_uint64, ctypes.c_int, ctypes.POINTER(ctypes.c_float), cp, sz]
         lib.tfh_layer_profile_step.argtypes = [vp, ctypes.c_uint64, ctypes.POINTER(ctypes.c_float), cp, sz]
         lib.tfh_layer_profile_marks.argtypes = [vp, ctypes.POINTER(ctypes.c_uint64), ctypes.c_int, ctypes.c_int, ctypes.POINTER(ctypes.c_float), cp, sz]
+        lib.tfh_layer_pair_run.argtypes = [vp, ctypes.c_uint64, ctypes.POINTER(ctypes.c_int64), ctypes.c_int, ctypes.c_uint64, ctypes.POINTER(ctypes.c_int64),
+                                           ctypes.c_int, vp, vp, cp, sz]
         lib.tfh_layer_tap.restype = ctypes.c_longlong
         lib.tfh_layer_tap.argtypes = [vp, cp, vp, sz, cp, sz]
         lib.tfh_layer_census.argtypes = [vp, vp, cp, sz]
@@ -123,6 +125,16 @@ class Layer:
         ms = (ctypes.c_float * 5)()
         self._check(self.lib.tfh_layer_profile_marks(self.h, ptrs, len(xs), passes, ms, self._err, 512))
         return list(ms)
+
+    def pair_run(self, xa, tokens_a, live_a, xb, tokens_b, live_b):
+        """Two owners of this layer through the pooled launch (Paired::run): returns both owners' outputs [rows][hidden] (BF16 bits)."""
+        ia = (ctypes.c_int64 * self.rows)(*[int(t) for t in tokens_a])
+        ib = (ctypes.c_int64 * self.rows)(*[int(t) for t in tokens_b])
+        oa = np.empty((self.rows, self.g.hidden), np.uint16)
+        ob = np.empty((self.rows, self.g.hidden), np.uint16)
+        self._check(self.lib.tfh_layer_pair_run(self.h, xa.data_ptr(), ia, live_a, xb.data_ptr(), ib, live_b,
+                                                oa.ctypes.data_as(ctypes.c_void_p), ob.ctypes.data_as(ctypes.c_void_p), self._err, 512))
+        return oa, ob
 
     def tap(self, name):
         size = self._check(self.lib.tfh_layer_tap(self.h, name.encode(), None, 0, self._err, 512))

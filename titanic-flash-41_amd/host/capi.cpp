@@ -16,6 +16,11 @@ struct Handle {
     std::vector<std::unique_ptr<tf::Graph>> graphs;
     tf::ScaleCodeReport scale_code;
     size_t rows = 0;
+    tf::LayerFfn::Options options;
+    // a second owner of the same layer and the pool both owners run through (src/paired_ffn.rs)
+    std::unique_ptr<tf::LayerFfn> layer_b;
+    std::unique_ptr<tf::TokenRows> tokens_b;
+    std::unique_ptr<tf::Paired> paired;
 };
 template <class F>
 int guarded(char* error, size_t error_len, F&& body) {
@@ -40,6 +45,7 @@ void* tfh_layer_create(const char* kernel_library, const ca_geometry* geometry, 
         if (code_scales) h->scale_code = tf::code_layer_scales(*h->native, *h->weights, h->prepared);
         tf::LayerFfn::Options options;
         options.overlap = overlap != 0; options.sum_shared = sum_shared != 0; options.route_front = route_front != 0; options.fold_shared = fold_shared != 0; options.gate_front = gate_front != 0;
+        h->options = options;
         h->layer = std::make_unique<tf::LayerFfn>(h->native, h->weights, h->prepared, (size_t)rows, options);
         h->workspace = std::make_unique<tf::Workspace>(h->native, (size_t)rows);
         std::vector<int64_t> ids((size_t)rows, 0);
@@ -176,6 +182,27 @@ int tfh_layer_profile_marks(void* handle, const uint64_t* inputs, int count, int
             sum[4] += events[5 * pass + 4]->elapsed_since(*events[5 * pass]);
         }
         for (int i = 0; i < 5; ++i) milliseconds[i] = (float)(sum[i] / passes);
+    });
+}
+// Paired owners: a second LayerFfn over the same prepared layer and the pooled workspace.  Runs owner A (the handle's layer,
+// input `a_input`, token ids / live count as given) and owner B through Paired::run and copies both owners' layer outputs
+// ([rows][hidden] BF16 each) to the host.
+int tfh_layer_pair_run(void* handle, uint64_t a_input, const int64_t* a_ids, int a_live, uint64_t b_input, const int64_t* b_ids, int b_live,
+                       uint16_t* a_output, uint16_t* b_output, char* error, size_t error_len) {
+    Handle* h = (Handle*)handle;
+    return guarded(error, error_len, [&] {
+        if (!h->paired) {
+            h->layer_b = std::make_unique<tf::LayerFfn>(h->native, h->weights, h->prepared, h->rows, h->options);
+            std::vector<int64_t> ids(h->rows, 0);
+            h->tokens_b = std::make_unique<tf::TokenRows>(ids.data(), h->rows, h->rows);
+            h->paired = std::make_unique<tf::Paired>(h->native, h->rows);
+        }
+        h->tokens->update(a_ids, h->rows, (size_t)a_live);
+        h->tokens_b->update(b_ids, h->rows, (size_t)b_live);
+        h->paired->run(*h->layer, a_input, *h->tokens, *h->layer_b, b_input, *h->tokens_b, *h->stream);
+        h->stream->synchronize();
+        h->layer->output().download(a_output, h->layer->output().len());
+        h->layer_b->output().download(b_output, h->layer_b->output().len());
     });
 }
 // Copies a named tap to the host.  Returns the tap's size in bytes (or -1); copies min(bytes, size).

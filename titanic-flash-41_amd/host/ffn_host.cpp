@@ -391,6 +391,21 @@ std::optional<std::pair<uint64_t, size_t>> Workspace::run_live_for_ffn(const Exp
     native_->primitive(2, sp, 3, ss, 3, stream.raw(), "moe.w4a16.topk_sum");
     return std::nullopt;
 }
+void Workspace::run_live(const Expert& expert, uint64_t input, size_t input_len, const Buffer<int32_t>& ids, const Buffer<float>& routing_weights,
+                         size_t live, const Stream& stream) {                                                 // src/moe.rs:1011-1043
+    const ca_geometry& g = native_->geometry();
+    ensure(live >= 1 && live <= rows_, "MoE live row domain");
+    guard_stream(stream);
+    ensure(input_len == rows_ * (size_t)g.hidden && ids.len() == rows_ * g.topk && routing_weights.len() == rows_ * g.topk, "MoE input shape mismatch");
+    uint64_t p[21];
+    pointers(expert, input, ids, routing_weights, p);
+    // num_tokens patched to the live prefix (:1221-1237): the rows past it are outside the launch
+    const int32_t scalars[6] = {(int32_t)live, (int32_t)rows_, (int32_t)(max_tiles_ * tile_m_), (int32_t)max_tiles_, (int32_t)tile_m_, 1};
+    native_->primitive(0, p, 21, scalars, 6, stream.raw(), "integration.tp_moe.dynamic");
+    const uint64_t sp[3] = {at("scatter_ptr"), output_.ptr(), 0};
+    const int32_t ss[3] = {(int32_t)live, 0, 0};
+    native_->primitive(2, sp, 3, ss, 3, stream.raw(), "moe.w4a16.topk_sum");
+}
 void Workspace::run_phase(int entry, const Expert& expert, uint64_t input, const Buffer<int32_t>& ids, const Buffer<float>& routing_weights,
                           const Stream& stream) {
     ensure(entry == 6 || entry == 7 || entry == 8, "phase entry");
@@ -474,6 +489,38 @@ void LayerFfn::sum_shared(const Workspace& workspace, size_t live_rows, const St
     int n = (int)(rows_ * g.hidden), live = (int)live_rows, topk = g.topk, hidden = g.hidden;
     void* args[] = {&routes, &shared, &routed, &output, &n, &live, &topk, &hidden};
     native_->launch("ca_ffn_sum_shared", (uint32_t)((n / 8 + 255) / 256), 1, 256, 0, args, stream.raw());
+}
+
+// ---- Paired ------------------------------------------------------------------------------------------------------------------
+Paired::Paired(std::shared_ptr<const Native> native, size_t owner_rows)
+    : native_(native), rows_(owner_rows), workspace_(native, 2 * owner_rows), shared_scratch_{Workspace(native, owner_rows), Workspace(native, owner_rows)},
+      input_(2 * owner_rows * native->geometry().hidden), ids_(2 * owner_rows * native->geometry().topk),
+      routing_(2 * owner_rows * native->geometry().topk) {
+    ensure(owner_rows >= 1 && 2 * owner_rows <= 64, "paired owners pool into one few-row launch");
+    input_.zero(); ids_.zero(); routing_.zero();                                                               // src/paired_ffn.rs:21-23
+}
+void Paired::run(LayerFfn& a, uint64_t a_input, const TokenRows& a_tokens, LayerFfn& b, uint64_t b_input, const TokenRows& b_tokens,
+                 const Stream& stream) {                                                                       // :65-120
+    const ca_geometry& g = native_->geometry();
+    const size_t a_live = a_tokens.active_rows(), b_live = b_tokens.active_rows(), H = g.hidden, K = g.topk;
+    ensure(a.rows() == rows_ && b.rows() == rows_ && a_live >= 1 && a_live <= rows_ && b_live >= 1 && b_live <= rows_ && a_input && b_input &&
+               a.expert().same_layer_weights(b.expert()),
+           "paired FFN needs two live prefixes of one canonical layer");                                       // :70-75
+    a.router().run(a_input, rows_ * H, a_tokens, stream);                                                      // :79-80: each owner routes privately
+    b.router().run(b_input, rows_ * H, b_tokens, stream);
+    struct Owner { size_t offset, live; LayerFfn* ffn; uint64_t input; };
+    const Owner owners[2] = {{0, a_live, &a, a_input}, {a_live, b_live, &b, b_input}};
+    for (const Owner& o : owners) {                                                                            // :84-90: six capturable copies on the one stream
+        check(hipMemcpyAsync((void*)(input_.ptr() + o.offset * H * 2), (const void*)o.input, o.live * H * 2, hipMemcpyDeviceToDevice, stream.raw()), "pool rows");
+        check(hipMemcpyAsync((void*)(ids_.ptr() + o.offset * K * 4), (const void*)o.ffn->router().ids().ptr(), o.live * K * 4, hipMemcpyDeviceToDevice, stream.raw()), "pool ids");
+        check(hipMemcpyAsync((void*)(routing_.ptr() + o.offset * K * 4), (const void*)o.ffn->router().routing().ptr(), o.live * K * 4, hipMemcpyDeviceToDevice, stream.raw()), "pool weights");
+    }
+    workspace_.run_live(a.expert(), input_.ptr(), input_.len(), ids_, routing_, a_live + b_live, stream);      // :91
+    for (int i = 0; i < 2; ++i) {                                                                              // :108-115: every owner's shared expert on its own rows
+        const Owner& o = owners[i];
+        o.ffn->run_shared(shared_scratch_[i], o.input, stream);
+        native_->ffn_add((int)o.live, workspace_.output().ptr() + o.offset * H * 2, o.ffn->shared_down().ptr(), o.ffn->output().ptr(), stream.raw());   // :116-121
+    }
 }
 
 }  // namespace tf

@@ -100,6 +100,8 @@ public:
     std::pair<uint64_t, size_t> region(const std::string& role) const;
     const Prepared& layout() const { return layout_; }
     const Weights& weights() const { return *weights_; }
+    // same_layer_weights (src/moe.rs:150-155): both views name the same prepared layer of the same atlas
+    bool same_layer_weights(const Expert& other) const { return weights_ == other.weights_ && layout_.layer == other.layout_.layer; }
 private:
     std::shared_ptr<Weights> weights_;
     Prepared layout_;
@@ -175,6 +177,9 @@ public:
                                                                const SharedOperands* shared = nullptr);
     void run(const Expert& expert, uint64_t input, size_t input_len, const Buffer<int32_t>& ids, const Buffer<float>& routing_weights,
              const Stream& stream) { run_live_for_ffn(expert, input, input_len, ids, routing_weights, rows_, false, std::nullopt, stream); }
+    // run_live (:1011-1043): only the first `live` rows are launched (ids / weights given); output() holds their reduced rows.
+    void run_live(const Expert& expert, uint64_t input, size_t input_len, const Buffer<int32_t>& ids, const Buffer<float>& routing_weights,
+                  size_t live, const Stream& stream);
     // Phase nodes alone (for per-kernel timing): 8 = front-end (plan + quantize), 6 = FC1 + SwiGLU, 7 = FC2.
     void run_phase(int entry, const Expert& expert, uint64_t input, const Buffer<int32_t>& ids, const Buffer<float>& routing_weights, const Stream& stream);
     // scratch regions by role name (the runtime contract's pointer table)
@@ -216,6 +221,7 @@ public:
     const Buffer<uint8_t>& activation_codes() const { return activation_codes_; }
     const Buffer<uint8_t>& activation_scales() const { return activation_scales_; }
     const Expert& expert() const { return expert_; }
+    const Native& native() const { return *native_; }
     size_t rows() const { return rows_; }
     // input != 0: quantize it first (the branch's own quantizer); 0: use the codes the front-end left in the workspace.
     void run_shared(const Workspace& workspace, uint64_t input, const Stream& stream);
@@ -232,6 +238,27 @@ private:
     Options options_;
     std::unique_ptr<Stream> branch_stream_;
     std::unique_ptr<Event> input_ready_, output_ready_;
+};
+
+// ---- two owners pooled into one routed-experts launch (src/paired_ffn.rs:5-120) ---------------------------------------------
+// Each owner routes privately; the live prefixes of both owners' rows, ids and routing weights are concatenated (device
+// copies on the one ordered stream, capturable), one launch runs the pooled rows, every owner's shared expert runs on its own
+// rows, and the routed sums are split back by the two shared additions.  No padding row of A becomes a live row of B.
+class Paired {
+public:
+    Paired(std::shared_ptr<const Native> native, size_t owner_rows);
+    void run(LayerFfn& a, uint64_t a_input, const TokenRows& a_tokens, LayerFfn& b, uint64_t b_input, const TokenRows& b_tokens,
+             const Stream& stream);
+    const Workspace& workspace() const { return workspace_; }
+    const Buffer<int32_t>& ids() const { return ids_; }
+private:
+    std::shared_ptr<const Native> native_;
+    size_t rows_;
+    Workspace workspace_;
+    Workspace shared_scratch_[2];      // the owners' shared-branch quantizer scratch
+    Buffer<uint16_t> input_;
+    Buffer<int32_t> ids_;
+    Buffer<float> routing_;
 };
 
 }  // namespace tf
