@@ -243,3 +243,41 @@ def test_error_conventions():
     assert lib.ca_ffn_configure(ctypes.byref(bad)) == -4
     with pytest.raises(RuntimeError):
         native.launch("no_such_kernel", 1, 64, [])
+
+
+def test_code_object_loads_and_resolves_every_kernel_by_name():
+    # the reference resolves its kernels by name from a code module (src/cuda.rs:199-226 Module::function / Function::launch);
+    # the same names must resolve from titanic_moe_gfx950.hsaco through the HIP module interface, and a launch through it
+    # must give the library's own result
+    import ctypes
+    import os
+    hip = ctypes.CDLL("libamdhip64.so")
+    assert os.path.exists(native.CODE_OBJECT), "build the package first (python -m __graft_entry__ or build.py)"
+    torch.cuda.init()
+    torch.zeros(1, device="cuda")
+    module = ctypes.c_void_p()
+    assert hip.hipModuleLoad(ctypes.byref(module), native.CODE_OBJECT.encode()) == 0
+    lib = native.load()
+    lib.ca_kernel_name.restype = ctypes.c_char_p
+    functions = {}
+    for i in range(lib.ca_kernel_count()):
+        name = lib.ca_kernel_name(i)
+        f = ctypes.c_void_p()
+        assert hip.hipModuleGetFunction(ctypes.byref(f), module, name) == 0, name
+        functions[name.decode()] = f
+    assert {"ca_route_padding_rows", "ca_ffn_sum_shared", "ca_moe_frontend", "ca_moe_route_frontend", "ca_route_topk",
+            "ca_expert_compact_words", "ca_expert_compact_scales", "ca_expert_scale_code1"} <= set(functions)
+    n = 8 * 1024
+    a = synth.activations("module/a", 8, 1024).cuda()
+    b = synth.activations("module/b", 8, 1024).cuda()
+    out = torch.zeros_like(a)
+    args = (ctypes.c_void_p * 4)()
+    held = [ctypes.c_void_p(a.data_ptr()), ctypes.c_void_p(b.data_ptr()), ctypes.c_void_p(out.data_ptr()), ctypes.c_longlong(n // 8)]
+    for i, v in enumerate(held):
+        args[i] = ctypes.cast(ctypes.pointer(v), ctypes.c_void_p)
+    hip.hipModuleLaunchKernel.argtypes = [ctypes.c_void_p] + [ctypes.c_uint] * 7 + [ctypes.c_void_p, ctypes.c_void_p, ctypes.c_void_p]
+    assert hip.hipModuleLaunchKernel(functions["ca_ffn_add_rows"], (n // 8 + 255) // 256, 1, 1, 256, 1, 1, 0, None, args, None) == 0
+    assert hip.hipDeviceSynchronize() == 0
+    want = oracle.ffn_add(u16(a), u16(b))
+    assert np.array_equal(u16(out), want)
+    assert hip.hipModuleUnload(module) == 0
