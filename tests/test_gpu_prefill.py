@@ -45,16 +45,21 @@ def test_wide_live_rows_and_skewed_routing():
     layer.close()
 
 
-@pytest.mark.parametrize("config", ["c4"])
+@pytest.mark.parametrize("config", ["c4", "c5"])
 def test_full_size_prefill(config):
     c = CONFIGS[config]
     g = geometry(c["hidden"], c["experts"], c["topk"], c["inter"], c["shared"], "benchmark")
     ops = synth.LayerOperands(g, config, device="cuda")
+    if config == "c5":       # expert popularity ~ rank^-1.1 through the selection bias, as the benchmark sets it
+        ops.bias = synth.zipf_bias(g.experts, 1.1, 0.06, device="cuda")
     rows = c["rows"]
     x = synth.activations(config, rows, g.hidden, device="cuda")
     layer = GpuLayer(g, ops, rows)
     taps = layer.run(x)
     # the oracle is evaluated on a sample of rows (all their routes), against the GPU's own routing
+    if config == "c5":
+        counts = np.bincount(taps["ids"].ravel(), minlength=g.experts)
+        assert counts.max() > 10 * counts.mean(), "the busiest expert must take more than ten times the mean load"
     sample = np.arange(0, rows, rows // 16)[:16]
     sub_taps = subset(taps, sample, g, rows)
     print(config, check_rows(g, ops, x[torch.as_tensor(sample, device=x.device)], sub_taps, taps, sample))
