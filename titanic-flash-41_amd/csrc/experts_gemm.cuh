@@ -237,8 +237,11 @@ __global__ void __launch_bounds__(256) tf_gemm(const GemmArgs p) {
                             const float gv = fminf(tf_bf16(gb), hi_lim), uv = fminf(fmaxf(tf_bf16(ub), lo_lim), hi_lim);
                             value = __fmul_rn(gv / __fadd_rn(1.0f, tf_exp(-gv)), uv);
                         } else {
+                            // routed experts: no bit-level definition of this step exists (the reference's is inside a binary), the
+                            // result is rounded to BF16 next; the many-row path spends as long here as in the matrix instructions
+                            // with the exact sequence, so it takes the hardware exponential and reciprocal
                             const float gv = fminf(acc[f][2 + j][i], p.limit), uv = fminf(p.limit, fmaxf(-p.limit, acc[f][j][i]));
-                            value = __fmul_rn(__fmul_rn(gv, tf_logistic(gv)), uv);
+                            value = __fmul_rn(__fmul_rn(gv, tf_logistic_fast(gv)), uv);
                         }
                         value = tf_bf16(tf_to_bf16(value));
                         hv[f][j][i] = value;
