@@ -51,15 +51,16 @@ template <bool FP8>
 struct BFrag { u4v lo; u4v hi; };
 
 template <bool FP8, int MODE>
-__global__ void __launch_bounds__(256) tf_gemm(const GemmArgs p) {
+__global__ void __launch_bounds__(512) tf_gemm(const GemmArgs p) {
     constexpr bool FC1 = MODE == TF_GEMM_FC1_ROUTED || MODE == TF_GEMM_FC1_SHARED;
     constexpr bool ROUTED = MODE == TF_GEMM_FC1_ROUTED || MODE == TF_GEMM_FC2_ROUTED;
     constexpr int GROUP_COLS = FC1 ? 128 : 256;          // output columns a task covers
     __shared__ __attribute__((aligned(16))) uint8_t s_a[2][16384];     // [stage][m-frag 8][half 2][lane 64][16 B]
     __shared__ uint32_t s_as[2][128];                                   // [stage][row]: scale bytes of the row's four K32 blocks
     __shared__ float s_amax[4][128];
-    __shared__ long long s_row[128];                                    // source row of each tile row (-1: unused)
-    const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6, g = lane >> 4, r16 = lane & 15;
+    __shared__ long long s_row[128];                                    // source row of each tile row
+    // eight waves: row half mh (64 rows = four 16-row fragments) x column quarter nq (64 weight rows = four 16-row tiles)
+    const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6, mh = wave >> 2, nq = wave & 3, g = lane >> 4, r16 = lane & 15;
     const int ksteps = p.k / 128;
     const int n_cols = FC1 ? p.inter : p.hidden, groups = n_cols / GROUP_COLS;
     const int tiles = ROUTED ? p.expert_tile_base[p.experts] : (p.dense_rows + 127) / 128;
@@ -79,8 +80,8 @@ __global__ void __launch_bounds__(256) tf_gemm(const GemmArgs p) {
         const uint8_t* ws = p.ws + (size_t)expert * p.ws_expert_stride;
         __syncthreads();
         if (tid < 128) {
-            // rows past the last valid one re-read the last valid row: every load of the main loop is then unconditional (the
-            // number of loads in flight is the same for every wave and k-step) and their products are never stored
+            // rows past the last valid one re-read the last valid row (no load of the main loop is conditional); their products
+            // are never stored
             const int t = min(tid, valid - 1);
             long long src;
             if (MODE == TF_GEMM_FC1_ROUTED) src = p.token_map[tile * 128 + t] / p.topk;
@@ -88,37 +89,38 @@ __global__ void __launch_bounds__(256) tf_gemm(const GemmArgs p) {
             s_row[tid] = src;
         }
         __syncthreads();
-        // this thread's four 16-byte chunks of every k-step's A tile: chunk id c = tid + 256 i is LDS slot c (a wave fills one
+        // this thread's two 16-byte chunks of every k-step's A tile: chunk id c = tid + 512 i is LDS slot c (a wave fills one
         // 1 KiB fragment block with consecutive 16-byte slots: no bank conflicts), i.e. fragment c / 128, K half (c / 64) % 2,
         // row c % 16 of the fragment, 16-byte piece (c % 64) / 16 of the half
-        const uint8_t* a_src[4];
-        int a_dst[4];
+        const uint8_t* a_src[2];
+        int a_dst[2];
 #pragma unroll
-        for (int i = 0; i < 4; ++i) {
-            const int c = tid + 256 * i, block = c >> 6, slot = c & 63;
+        for (int i = 0; i < 2; ++i) {
+            const int c = tid + 512 * i, block = c >> 6, slot = c & 63;
             const int row = (block >> 1) * 16 + (slot & 15), piece = (block & 1) * 4 + (slot >> 4);
-            const long long src = s_row[row];
-            a_src[i] = p.a_codes + src * p.k + piece * 16;
+            a_src[i] = p.a_codes + s_row[row] * p.k + piece * 16;
             a_dst[i] = c * 16;
         }
         const uint8_t* as_src = p.a_scales + s_row[tid & 127] * (p.k / p.act_block);
-        // weight row tiles of this wave: FC1 routed: up tiles then gate tiles; FC1 shared: gate tiles then up tiles
+        // weight row tiles of this wave: FC1 routed: two "up" tiles then two "gate" tiles of the same 32 intermediate columns;
+        // FC1 shared: gate tiles then up tiles; FC2 / dense: four tiles of 64 output columns
         int ntile[4];
 #pragma unroll
         for (int j = 0; j < 4; ++j) {
-            if (FC1) ntile[j] = (j >> 1) * (p.inter / 16) + (ng * 128 + wave * 32) / 16 + (j & 1);
-            else ntile[j] = (ng * 256 + wave * 64) / 16 + j;
+            if (FC1) ntile[j] = (j >> 1) * (p.inter / 16) + (ng * 128 + nq * 32) / 16 + (j & 1);
+            else ntile[j] = (ng * 256 + nq * 64) / 16 + j;
         }
-        auto load_a = [&](int ks, u4v (&ra)[4], uint32_t& rs) {
+        auto load_a = [&](int ks, u4v (&ra)[2], uint32_t& rs) {
 #pragma unroll
-            for (int i = 0; i < 4; ++i) ra[i] = *reinterpret_cast<const u4v*>(a_src[i] + (size_t)ks * 128);
+            for (int i = 0; i < 2; ++i) ra[i] = *reinterpret_cast<const u4v*>(a_src[i] + (size_t)ks * 128);
+            // the raw scale bytes only: arithmetic on a value just requested would make this a wait for every load in flight
             if (p.act_block == 32) rs = *reinterpret_cast<const uint32_t*>(as_src + ks * 4);
-            else rs = 0x01010101u * as_src[ks];
+            else rs = as_src[ks];
         };
-        auto store_a = [&](int stage, const u4v (&ra)[4], uint32_t rs) {
+        auto store_a = [&](int stage, const u4v (&ra)[2], uint32_t rs) {
 #pragma unroll
-            for (int i = 0; i < 4; ++i) *reinterpret_cast<u4v*>(&s_a[stage][a_dst[i]]) = ra[i];
-            if (tid < 128) s_as[stage][tid] = rs;
+            for (int i = 0; i < 2; ++i) *reinterpret_cast<u4v*>(&s_a[stage][a_dst[i]]) = ra[i];
+            if (tid < 128) s_as[stage][tid] = p.act_block == 32 ? rs : 0x01010101u * rs;      // one byte per K32 block of the k-step
         };
         // B operand of one k-step: plain loads (an expert's weight slice is re-read by the expert's other tiles from this
         // XCD's L2).  FP8: with the lane's block scale of the k-step; FP4: scales come a word per four k-steps (load_b_scales).
@@ -139,29 +141,29 @@ __global__ void __launch_bounds__(256) tf_gemm(const GemmArgs p) {
 #pragma unroll
             for (int j = 0; j < 4; ++j) sb[j] = reinterpret_cast<const uint32_t*>(ws)[((size_t)ntile[j] * (p.k / 512) + ks / 4) * 64 + lane];
         };
-        v4f acc[8][4];
+        v4f acc[4][4];
 #pragma unroll
-        for (int f = 0; f < 8; ++f)
+        for (int f = 0; f < 4; ++f)
 #pragma unroll
             for (int j = 0; j < 4; ++j) acc[f][j] = v4f{0.f, 0.f, 0.f, 0.f};
-        const int frags = (valid + 15) >> 4;
+        const int frags = (valid + 15) >> 4;                       // of the tile
+        const int my_frags = min(4, max(0, frags - 4 * mh));       // of this wave's row half
 
-        // Main loop, compiled for 2, 4, 6 or 8 row fragments so that its products sit under no branch.  Operands of k-step
-        // ks + D - 1 are requested while k-step ks is multiplied (a ring of D register sets, indexed statically by unrolling
-        // D times): the token tile goes registers -> LDS one k-step ahead of its use (two LDS stages, one barrier a k-step),
-        // the weights stay in registers.
+        // Main loop, compiled for 0, 2 or 4 row fragments of the wave's half so that its products sit under no branch (every
+        // wave runs the same loads, LDS stores and barriers whatever its count).  Operands of k-step ks + D - 1 are requested
+        // while k-step ks is multiplied (a ring of D register sets, indexed statically by unrolling D times): the token tile
+        // goes registers -> LDS one k-step ahead of its use (two LDS stages, one barrier a k-step), the weights stay in
+        // registers.  Two waves share a SIMD, so one wave's loads, LDS traffic and scalar work run under the other's products.
         auto main_loop = [&](auto fr_constant) {
             constexpr int FR = decltype(fr_constant)::value;
-            constexpr int D = FP8 ? 3 : 4;
-            u4v ra[D][4];
+            constexpr int D = FP8 ? 2 : 4;         // ksteps % 4 == 0
+            u4v ra[D][2];
             uint32_t rs[D];
             BFrag<FP8> b[D][4];
             uint32_t sbk[D][4];                  // FP8: the slot's scale bytes
             uint32_t sb[4] = {0, 0, 0, 0}, sb_next[4] = {0, 0, 0, 0};   // FP4: scale words of the current / next four k-steps
 #pragma unroll
-            for (int d = 0; d < D - 1; ++d) {
-                if (d < ksteps) { load_a(d, ra[d], rs[d]); load_b(d, b[d], sbk[d]); }
-            }
+            for (int d = 0; d < D - 1; ++d) { load_a(d, ra[d], rs[d]); load_b(d, b[d], sbk[d]); }
             if constexpr (!FP8) load_b_scales(0, sb);
             store_a(0, ra[0], rs[0]);
             __syncthreads();
@@ -169,13 +171,14 @@ __global__ void __launch_bounds__(256) tf_gemm(const GemmArgs p) {
 #pragma unroll
                 for (int u = 0; u < D; ++u) {
                     const int ks = ks0 + u;
-                    if (ks < ksteps) {
-                        const int stage = ks & 1, ahead = ks + D - 1;
-                        if (ahead < ksteps) {
-                            load_a(ahead, ra[(u + D - 1) % D], rs[(u + D - 1) % D]);
-                            load_b(ahead, b[(u + D - 1) % D], sbk[(u + D - 1) % D]);
-                            if constexpr (!FP8) { if (u == 1) load_b_scales(ahead, sb_next); }       // ahead % 4 == 0 (D == 4, ksteps % 4 == 0)
-                        }
+                    {
+                        // No load sits under a condition (the last D - 1 k-steps request the last k-step again rather than
+                        // nothing): the compiler counts outstanding loads statically, and a load that may or may not have been
+                        // issued turns every wait behind it into a wait for all loads in flight.
+                        const int stage = ks & 1, ahead = min(ks + D - 1, ksteps - 1);
+                        load_a(ahead, ra[(u + D - 1) % D], rs[(u + D - 1) % D]);
+                        load_b(ahead, b[(u + D - 1) % D], sbk[(u + D - 1) % D]);
+                        if constexpr (!FP8) { if (u == 1) load_b_scales(ahead, sb_next); }           // ahead % 4 == 0 (D == 4)
                         if constexpr (!FP8) {
                             if (u == 0 && ks > 0) {
 #pragma unroll
@@ -184,10 +187,11 @@ __global__ void __launch_bounds__(256) tf_gemm(const GemmArgs p) {
                         }
 #pragma unroll
                         for (int f = 0; f < FR; ++f) {
-                            const u4v lo = *reinterpret_cast<const u4v*>(&s_a[stage][((f * 2) * 64 + lane) * 16]);
-                            const u4v hi = *reinterpret_cast<const u4v*>(&s_a[stage][((f * 2 + 1) * 64 + lane) * 16]);
+                            const int tf = 4 * mh + f;             // fragment of the tile
+                            const u4v lo = *reinterpret_cast<const u4v*>(&s_a[stage][((tf * 2) * 64 + lane) * 16]);
+                            const u4v hi = *reinterpret_cast<const u4v*>(&s_a[stage][((tf * 2 + 1) * 64 + lane) * 16]);
                             const v8i av = v8i{(int)lo[0], (int)lo[1], (int)lo[2], (int)lo[3], (int)hi[0], (int)hi[1], (int)hi[2], (int)hi[3]};
-                            const int sa = (int)((s_as[stage][f * 16 + r16] >> (8 * g)) & 0xffu);
+                            const int sa = (int)((s_as[stage][tf * 16 + r16] >> (8 * g)) & 0xffu);
 #pragma unroll
                             for (int j = 0; j < 4; ++j) {
                                 const BFrag<FP8>& bj = b[u][j];
@@ -199,25 +203,29 @@ __global__ void __launch_bounds__(256) tf_gemm(const GemmArgs p) {
                                     acc[f][j] = __builtin_amdgcn_mfma_scale_f32_16x16x128_f8f6f4(av, bv, acc[f][j], 0, 4, 0, sa, 0, (int)(sb[j] >> (8 * u)));
                                 }
                             }
+                            // a use the optimizer cannot move: without it every product of the unrolled k-steps is sunk below the
+                            // barriers, the k-steps' A fragments stay alive until then and spill
+#pragma unroll
+                            for (int j = 0; j < 4; ++j) asm volatile("" :: "v"(acc[f][j]));
                         }
-                        if (ks + 1 < ksteps) store_a(stage ^ 1, ra[(u + 1) % D], rs[(u + 1) % D]);
+                        store_a(stage ^ 1, ra[(u + 1) % D], rs[(u + 1) % D]);
                         __syncthreads();
                     }
                 }
             }
         };
-        if (frags > 6) main_loop(std::integral_constant<int, 8>{});
-        else if (frags > 4) main_loop(std::integral_constant<int, 6>{});
-        else if (frags > 2) main_loop(std::integral_constant<int, 4>{});
-        else main_loop(std::integral_constant<int, 2>{});
+        if (my_frags > 2) main_loop(std::integral_constant<int, 4>{});
+        else if (my_frags > 0) main_loop(std::integral_constant<int, 2>{});
+        else main_loop(std::integral_constant<int, 0>{});
 
         // ---- epilogue --------------------------------------------------------------------------------------------------
+        // lane (g, r16) of fragment f holds rows 64 mh + 16 f + 4 g + i (i < 4) and, per weight tile j, column r16 of the tile
         if constexpr (FC1) {
             const float hi_lim = tf_bf16(tf_to_bf16(p.limit)), lo_lim = tf_bf16(tf_to_bf16(-p.limit));
-            float hv[8][2][4];
-            float amax[8][4];
+            float hv[4][2][4];
+            float amax[4][4];
 #pragma unroll
-            for (int f = 0; f < 8; ++f)
+            for (int f = 0; f < 4; ++f)
 #pragma unroll
                 for (int i = 0; i < 4; ++i) {
                     float m = 0.f;
@@ -226,10 +234,10 @@ __global__ void __launch_bounds__(256) tf_gemm(const GemmArgs p) {
                         float value;
                         if (MODE == TF_GEMM_FC1_SHARED) {
                             const uint16_t gb = tf_to_bf16(acc[f][j][i]), ub = tf_to_bf16(acc[f][2 + j][i]);
-                            if (p.tap != nullptr && f < frags) {
-                                const int row = 16 * f + 4 * g + i;
+                            if (p.tap != nullptr && f < my_frags) {
+                                const int row = 64 * mh + 16 * f + 4 * g + i;
                                 if (row < valid) {
-                                    const size_t at = (size_t)(tile * 128 + row) * 2 * p.inter + ng * 128 + wave * 32 + j * 16 + r16;
+                                    const size_t at = (size_t)(tile * 128 + row) * 2 * p.inter + ng * 128 + nq * 32 + j * 16 + r16;
                                     p.tap[at] = gb;
                                     p.tap[at + p.inter] = ub;
                                 }
@@ -238,8 +246,7 @@ __global__ void __launch_bounds__(256) tf_gemm(const GemmArgs p) {
                             value = __fmul_rn(gv / __fadd_rn(1.0f, tf_exp(-gv)), uv);
                         } else {
                             // routed experts: no bit-level definition of this step exists (the reference's is inside a binary), the
-                            // result is rounded to BF16 next; the many-row path spends as long here as in the matrix instructions
-                            // with the exact sequence, so it takes the hardware exponential and reciprocal
+                            // result is rounded to BF16 next; the many-row path takes the hardware exponential and reciprocal
                             const float gv = fminf(acc[f][2 + j][i], p.limit), uv = fminf(p.limit, fmaxf(-p.limit, acc[f][j][i]));
                             value = __fmul_rn(__fmul_rn(gv, tf_logistic_fast(gv)), uv);
                         }
@@ -249,40 +256,40 @@ __global__ void __launch_bounds__(256) tf_gemm(const GemmArgs p) {
                     }
                     amax[f][i] = tf_row16_max(m);
                 }
-            if (p.act_block == 128) {
+            if (p.act_block == 128) {          // one scale per row and 128 columns: across the four column quarters
 #pragma unroll
-                for (int f = 0; f < 8; ++f)
+                for (int f = 0; f < 4; ++f)
 #pragma unroll
-                    for (int i = 0; i < 4; ++i) if (r16 == 0) s_amax[wave][16 * f + 4 * g + i] = amax[f][i];
+                    for (int i = 0; i < 4; ++i) if (r16 == 0) s_amax[nq][64 * mh + 16 * f + 4 * g + i] = amax[f][i];
                 __syncthreads();
 #pragma unroll
-                for (int f = 0; f < 8; ++f)
+                for (int f = 0; f < 4; ++f)
 #pragma unroll
                     for (int i = 0; i < 4; ++i) {
-                        const int row = 16 * f + 4 * g + i;
+                        const int row = 64 * mh + 16 * f + 4 * g + i;
                         amax[f][i] = fmaxf(fmaxf(s_amax[0][row], s_amax[1][row]), fmaxf(s_amax[2][row], s_amax[3][row]));
                     }
             }
             const float min_amax = MODE == TF_GEMM_FC1_SHARED ? 1e-4f : 0.f;
 #pragma unroll
-            for (int f = 0; f < 8; ++f) {
-                if (f < frags) {
+            for (int f = 0; f < 4; ++f) {
+                if (f < my_frags) {
 #pragma unroll
                     for (int i = 0; i < 4; ++i) {
-                        const int row = 16 * f + 4 * g + i;
+                        const int row = 64 * mh + 16 * f + 4 * g + i;
                         if (row < valid) {
                             const uint32_t exponent = tf_block_exponent(min_amax > 0.f ? fmaxf(amax[f][i], min_amax) : amax[f][i]);
                             const float inv = tf_block_inverse(exponent);
                             const size_t phys = (size_t)tile * 128 + row;
-                            const int col = ng * 128 + wave * 32 + r16;
+                            const int col = ng * 128 + nq * 32 + r16;
 #pragma unroll
                             for (int j = 0; j < 2; ++j) {
                                 p.h_codes[phys * p.inter + col + 16 * j] = (uint8_t)tf_to_e4m3(__fmul_rn(hv[f][j][i], inv));
                                 if (p.h_bf16 != nullptr) p.h_bf16[phys * p.inter + col + 16 * j] = tf_to_bf16(hv[f][j][i]);
                             }
                             if (r16 == 0) {
-                                if (p.act_block == 32) p.h_scales[phys * (p.inter / 32) + ng * 4 + wave] = (uint8_t)exponent;
-                                else if (wave == 0) p.h_scales[phys * (p.inter / 128) + ng] = (uint8_t)exponent;
+                                if (p.act_block == 32) p.h_scales[phys * (p.inter / 32) + ng * 4 + nq] = (uint8_t)exponent;
+                                else if (nq == 0) p.h_scales[phys * (p.inter / 128) + ng] = (uint8_t)exponent;
                             }
                         }
                     }
@@ -290,11 +297,11 @@ __global__ void __launch_bounds__(256) tf_gemm(const GemmArgs p) {
             }
         } else {
 #pragma unroll
-            for (int f = 0; f < 8; ++f) {
-                if (f < frags) {
+            for (int f = 0; f < 4; ++f) {
+                if (f < my_frags) {
 #pragma unroll
                     for (int i = 0; i < 4; ++i) {
-                        const int row = 16 * f + 4 * g + i;
+                        const int row = 64 * mh + 16 * f + 4 * g + i;
                         if (row < valid) {
                             const int phys = tile * 128 + row;
                             size_t out_row = (size_t)phys;
@@ -303,7 +310,7 @@ __global__ void __launch_bounds__(256) tf_gemm(const GemmArgs p) {
 #pragma unroll
                             for (int j = 0; j < 4; ++j) {
                                 const float v = MODE == TF_GEMM_FC2_ROUTED ? __fmul_rn(acc[f][j][i], scale) : acc[f][j][i];
-                                p.out[out_row * p.hidden + ng * 256 + wave * 64 + 16 * j + r16] = tf_to_bf16(v);
+                                p.out[out_row * p.hidden + ng * 256 + nq * 64 + 16 * j + r16] = tf_to_bf16(v);
                             }
                         }
                     }
@@ -320,22 +327,22 @@ inline bool tf_gemm_shape_ok(const GemmArgs& a, bool fc1) {
 }
 inline int tf_launch_fc1_gemm(const GemmArgs& a, int cus, hipStream_t s) {
     if (!tf_gemm_shape_ok(a, true)) return -4;
-    tf_gemm<false, TF_GEMM_FC1_ROUTED><<<tf_gemm_grid(cus), 256, 0, s>>>(a);
+    tf_gemm<false, TF_GEMM_FC1_ROUTED><<<tf_gemm_grid(cus), 512, 0, s>>>(a);
     return (int)hipGetLastError();
 }
 inline int tf_launch_fc2_gemm(const GemmArgs& a, int cus, hipStream_t s) {
     if (!tf_gemm_shape_ok(a, false)) return -4;
-    tf_gemm<false, TF_GEMM_FC2_ROUTED><<<tf_gemm_grid(cus), 256, 0, s>>>(a);
+    tf_gemm<false, TF_GEMM_FC2_ROUTED><<<tf_gemm_grid(cus), 512, 0, s>>>(a);
     return (int)hipGetLastError();
 }
 inline int tf_launch_dense_gemm(const GemmArgs& a, int cus, hipStream_t s) {
     if (!tf_gemm_shape_ok(a, false)) return -4;
-    tf_gemm<true, TF_GEMM_DENSE><<<tf_gemm_grid(cus), 256, 0, s>>>(a);
+    tf_gemm<true, TF_GEMM_DENSE><<<tf_gemm_grid(cus), 512, 0, s>>>(a);
     return (int)hipGetLastError();
 }
 inline int tf_launch_shared_fc1_gemm(const GemmArgs& a, int cus, hipStream_t s) {
     if (!tf_gemm_shape_ok(a, true)) return -4;
-    tf_gemm<true, TF_GEMM_FC1_SHARED><<<tf_gemm_grid(cus), 256, 0, s>>>(a);
+    tf_gemm<true, TF_GEMM_FC1_SHARED><<<tf_gemm_grid(cus), 512, 0, s>>>(a);
     return (int)hipGetLastError();
 }
 
