@@ -45,6 +45,8 @@ MFMA_FP8_PEAK_TFLOPS, MFMA_FP4_PEAK_TFLOPS = 5000.0, 10100.0
 # each counter scaled by its reading for a 256 MiB copy kernel).  The line's `traffic` is this ratio times the algorithmic
 # bytes of this run's launches; None where no counter run exists for the configuration.
 TRAFFIC_OVER_ALGORITHMIC = {"c2": 1.008}
+# Many rows: HBM bytes a launch of the routed FC1 kernel, measured the same way at the same number of rows.
+WIDE_TRAFFIC_BYTES = {"c4": 3.43e9, "c5": 7.53e9}
 
 
 def make_inputs(synth, name, cfg, device, batches=BATCHES):
@@ -213,7 +215,8 @@ def main():
                       "achieved": fc1_flops / (fc1_ms * 1e-3) / 1e12, "peak": MFMA_FP8_PEAK_TFLOPS, "unit": "TFLOP/s",
                       "frac": fc1_flops / (fc1_ms * 1e-3) / 1e12 / MFMA_FP8_PEAK_TFLOPS,
                       "frac_of_fp4_peak": fc1_flops / (fc1_ms * 1e-3) / 1e12 / MFMA_FP4_PEAK_TFLOPS,
-                      "operands": "A = FP8 E4M3 activations, B = FP4 E2M1 weights: issues at the FP8 rate (measured)", "traffic": None,
+                      "operands": "A = FP8 E4M3 activations, B = FP4 E2M1 weights: issues at the FP8 rate (measured)",
+                      "traffic": WIDE_TRAFFIC_BYTES.get(args.config), "traffic_source": "rocprofv3 counters on tf_layer_probe at the same rows (profiles/)",
                       "flops_per_launch": fc1_flops, "avg_launch_ms": fc1_ms, "weight_gbs": fc1_bytes / (fc1_ms * 1e-3) / 1e9} if wide else
                      {"bound": "hbm", "kernel": "tf_phase1_stream (FC1 + SwiGLU of the routed experts and the shared expert in one launch)",
                       "achieved": achieved, "peak": HBM_PEAK_GBS, "unit": "GB/s", "frac": achieved / HBM_PEAK_GBS,
