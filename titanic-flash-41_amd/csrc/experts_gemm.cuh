@@ -1,13 +1,15 @@
 // Many-row (prefill) expert projections: grouped GEMM on v_mfma_scale_f32_16x16x128_f8f6f4.
 //
 // One task = one M tile of 128 physical rows (one expert's rows, gathered through the permutation map) x one column
-// group.  A workgroup of four waves keeps a 128 x 256 accumulator (each wave 128 rows x 64 weight rows, in AGPRs/VGPRs):
-//   FC1: 128 intermediate columns = 128 "up" + 128 "gate" weight rows, so SwiGLU and the FP8 requantization of the
-//        result (one scale a row and `act_block` columns) run in the epilogue, from registers;
+// group.  A workgroup of eight waves (512 threads, two waves a SIMD) keeps a 128 x 256 accumulator: wave (mh, nq) holds
+// rows 64 mh .. of the tile x 64 weight rows (four 16-row fragments x four 16-row weight tiles):
+//   FC1: 128 intermediate columns = 128 "up" + 128 "gate" weight rows (a wave: 32 + 32 of the same 32 columns), so SwiGLU
+//        and the FP8 requantization of the result (one scale a row and `act_block` columns) run in the epilogue, from
+//        registers;
 //   FC2 / dense: 256 output columns; routed rows are scaled by their routing weight and scattered to route order.
 // The E4M3 token tile goes through LDS (double-buffered, stored in matrix-instruction fragment order so every wave reads
 // 1 KiB contiguous, conflict-free, per fragment); the prepared weights go from global memory straight into the B operand
-// (each wave owns its weight rows, 1 KiB contiguous per fragment and k-step) with the next k-step in flight.
+// (1 KiB contiguous per weight tile and k-step) through a ring of register sets, three k-steps ahead of their use.
 // Workgroups are persistent and XCD-aware: workgroup b runs on XCD b % 8 and only ever touches 1/8 of the column groups,
 // so every XCD's L2 holds its own slices of the expert's weights while the expert's tiles pass by; partially filled
 // tiles skip the 16-row fragments past their last valid row.
