@@ -51,6 +51,14 @@ def test_scale_code_and_prepared_layout_report():
     assert info["expert_bytes"] == E * (3 * H * I // 2 + 3 * H * I // 32)
     assert info["scale_code_bytes"] == oracle.scale_code1_layout(E, H, I)[5] * 4
     assert info["coded_rows"] == E * (2 * (I // 128) * (H // 128) + (H // 128) * (I // 128)) * 128 and info["raw_rows"] < info["coded_rows"]
+    # the scratch arena has one size, whoever computes it: the host mirror, the library, the contract writer
+    import ctypes
+    from helpers import configure, native
+    ctx = configure(g)
+    contract = pkg.contracts.scratch_layout(dict(hidden=g.hidden, experts=g.experts, topk=g.topk, intermediate=g.intermediate,
+                                                 act_block=g.act_block), rows)
+    assert info["scratch_bytes"] == native.load().ca_primitives_scratch_bytes(ctx, 0, rows) == contract[1]
+    assert info["max_tiles"] == contract[3] and info["tile_m"] == contract[2]
     layer.close()
 
 

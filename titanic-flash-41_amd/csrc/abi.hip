@@ -14,7 +14,6 @@ namespace {
 ca_geometry g_geometry = {5120, 384, 6, 576, 576, 1, 1.5f, 32, 32, 32, 129264, 10.f};   // src/ffn.rs:65-66, 245-258
 
 bool supported_k(int k) { return k == 512 || k == 1024 || k == 2048 || k == 4096; }
-constexpr size_t kSyncBytes = 16384;   // arrival word + queue / dependency counters of the streaming launch
 int check_geometry(const ca_geometry& g) {
     if (g.hidden <= 0 || g.hidden % 512 || g.experts <= 0 || g.experts > 512 || g.topk <= 0 || g.topk > 8 ||
         g.topk > g.experts || g.intermediate <= 0 || g.intermediate % 512 || g.shared_intermediate <= 0 ||
@@ -32,7 +31,6 @@ struct Context {
     int stream_wgs;    // persistent workgroups of the streaming kernels
     hipEvent_t marks[5];   // profiling aid: see ca_primitives_marks
     bool marking;
-    bool single_launch; // FC1 + FC2 + sum in one launch with in-kernel dependencies (experimental: slower than two launches so far)
 };
 
 // Records mark `i` on the launch stream when the caller asked for marks (never while a stream is captured: the caller's duty).
@@ -99,7 +97,7 @@ void shared_stream_args(const Context& c, const uint64_t* p, int m, StreamArgs& 
 // order, its input codes taken from the front-end's shared-flavour output), folded into the same phase launches.
 // `sum` (may be null, needs `sh`): {routed output, layer output} device pointers and the live row count: the ordered sum and the
 // shared addition run as well (inside the single streaming launch when the shapes allow it).
-struct SumArgs { uint64_t routed_out, output; int live; uint64_t sync; };
+struct SumArgs { uint64_t routed_out, output; int live; };
 int launch_dynamic(const Context& c, bool route, const uint64_t* p, const int32_t* sc, hipStream_t s, int phases = 7, const uint64_t* sh = nullptr,
                    const SumArgs* sum = nullptr) {
     const ca_geometry& g = c.g;
@@ -117,10 +115,6 @@ int launch_dynamic(const Context& c, bool route, const uint64_t* p, const int32_
     if (few ? tile_m != 16 : tile_m != TF_GEMM_TILE_M) return -1;
     if (few && max_tiles > TF_LDS_TILES) return -1;
 
-    // single streaming launch: one unit is 16 loads a lane in both projections
-    const bool mega = c.single_launch && few && sh && sum && sum->sync && phases == 7 && (g.hidden == 1024 || g.hidden == 4096) && g.hidden == 2 * g.intermediate && g.shared_intermediate == g.intermediate;
-    const int counter_words = mega ? 8 + max_tiles + 4 + g.hidden / 64 : 0;
-    uint32_t* counters = mega ? (uint32_t*)sum->sync + 16 : nullptr;
     mark(c, 0, s);
     const uint16_t* x = (const uint16_t*)p[P_A];
     int32_t* ids = (int32_t*)p[P_IDS];
@@ -142,12 +136,12 @@ int launch_dynamic(const Context& c, bool route, const uint64_t* p, const int32_
                 (const float*)p[P_BIAS], (const float*)p[P_BIAS_ALT], (const long long*)p[P_TOKENS], (const int32_t*)p[P_LIVE],
                 (const int32_t*)p[P_PADDING], rows, g.topk, g.experts, g.hidden, groups, tile_m, owner, g.act_block,
                 (uint8_t*)p[P_PACKED_MIN], (uint8_t*)p[P_SCALES_MIN], g.scoring, g.route_scale, (long long)g.alt_token,
-                (const uint16_t*)p[P_GATE_W], (uint32_t*)p[P_SYNC], logit_blocks, counters, counter_words);
+                (const uint16_t*)p[P_GATE_W], (uint32_t*)p[P_SYNC], logit_blocks);
         } else {
             ca_moe_frontend<<<quant_blocks, 512, 0, s>>>(
                 x, ids, weights, (uint8_t*)p[P_PACKED], (uint8_t*)p[P_SCALES], (int32_t*)p[P_TOKEN_MAP], (float*)p[P_TOKEN_WEIGHTS],
                 (int32_t*)p[P_TASK_EXPERT], (int32_t*)p[P_TASK_VALID], (int32_t*)p[P_TILE_BASE], rows, g.topk, g.experts, g.hidden,
-                groups, tile_m, g.act_block, (uint8_t*)p[P_PACKED_MIN], (uint8_t*)p[P_SCALES_MIN], counters, counter_words);
+                groups, tile_m, g.act_block, (uint8_t*)p[P_PACKED_MIN], (uint8_t*)p[P_SCALES_MIN]);
         }
     } else {
         if (route || !p[P_PLAN_SCRATCH]) return -1;   // wide owners route with ca_route_topk first
@@ -196,19 +190,6 @@ int launch_dynamic(const Context& c, bool route, const uint64_t* p, const int32_
         b.w = (const uint8_t*)p[P_W2]; b.ws = (const uint8_t*)p[P_S2];
         b.w_expert_stride = w2_stride; b.ws_expert_stride = s2_stride;
         b.k = g.intermediate; b.out = (uint16_t*)p[P_SCATTER];
-        if (mega) {
-            MegaArgs m{};
-            m.r1 = a; m.s1 = sa; m.r2 = b; m.s2 = sb;
-            m.counters = counters; m.max_tiles = max_tiles;
-            m.routes = (const uint16_t*)p[P_SCATTER]; m.shared_down = (const uint16_t*)sh[H_OUT];
-            m.routed_out = (uint16_t*)sum->routed_out; m.output = (uint16_t*)sum->output;
-            m.rows = rows; m.live = sum->live < rows ? sum->live : rows; m.topk = g.topk;
-            const size_t lds = 16 * (size_t)g.intermediate + 16 * (size_t)(g.intermediate / g.act_block);
-            // one workgroup a CU keeps every operand in registers (the 4096-wide unit does not fit twice); the grid is what is resident
-            if (g.hidden == 1024) tf_moe_stream<2, 1, 2><<<c.cus * 2, 256, lds, s>>>(m);
-            else tf_moe_stream<8, 4, 1><<<c.cus, 256, lds, s>>>(m);
-            return launch_status();
-        }
         if (phases & 2) {
             status = launch_phase1(a, sa, c.stream_wgs, s);
             if (status) return status;
@@ -422,7 +403,6 @@ void* ca_primitives_open(int32_t* status) {
     if (e != hipSuccess) { *status = (int32_t)e; return nullptr; }
     Context* c = new Context{};
     c->g = g_geometry; c->cus = cus; c->stream_wgs = cus * 2;
-    if (const char* v = std::getenv("TITANIC_MOE_SINGLE_LAUNCH")) c->single_launch = v[0] == '1';
     if (const char* v = std::getenv("TITANIC_MOE_STREAM_WGS_PER_CU")) {
         const int n = std::atoi(v);
         if (n >= 1 && n <= 8) c->stream_wgs = cus * n;
@@ -465,7 +445,7 @@ int32_t ca_primitives_launch(void* context, int32_t index, const uint64_t* point
             // + routed output, layer output (both or neither) and the live row count: the sum and the shared addition run too
             const uint64_t routed_out = pointers[P_ROUTE_COUNT + H_COUNT - 2], output = pointers[P_ROUTE_COUNT + H_COUNT - 1];
             if (!routed_out != !output) return -1;
-            const SumArgs sum{routed_out, output, scalars[S_ROUTE_COUNT], pointers[P_SYNC]};
+            const SumArgs sum{routed_out, output, scalars[S_ROUTE_COUNT]};
             return launch_dynamic(c, pointers[P_LOGITS] != 0, pointers, scalars, s, 7, sh, output ? &sum : nullptr);
         }
         default: return -3;
@@ -488,12 +468,15 @@ int64_t ca_primitives_scratch_bytes(void* context, int32_t index, int32_t rows) 
     const long long tiles = (pairs + tile_m - 1) / tile_m - 1 + (g.experts < pairs ? g.experts : pairs), padded = tiles * tile_m;
     long long bytes = 0;
     auto add = [&](long long n) { bytes += (n + 255) / 256 * 256; };
-    add(2ll * rows * g.hidden); add(2ll * rows * g.hidden / g.act_block);              // packed + scales, both flavours
-    add(2ll * rows * g.hidden / g.act_block);
-    add(padded * g.intermediate * 2); add(padded * g.intermediate); add(padded * g.intermediate / g.act_block);
-    add(tiles * 4 * 8); add(tiles * 4 * 8); add((g.experts + 1) * 4ll); add(padded * 4); add(padded * 4);
-    add(pairs * g.hidden * 2);
-    add(((pairs + 63) / 64) * g.experts * 4 + pairs * 4);
+    const long long H = g.hidden, I = g.intermediate, B = g.act_block;
+    // the regions of the runtime contract, in its order, each aligned to 256 bytes: token codes and scales (routed flavour,
+    // shared flavour), intermediate (BF16, codes, scales), tile tables, row maps, route outputs, wide-plan scratch, sync word
+    add(rows * H); add(rows * H / B); add(rows * H); add(rows * H / B);
+    add(padded * I * 2); add(padded * I); add(padded * I / B);
+    add(tiles * 4); add(tiles * 4); add((g.experts + 1) * 4ll); add(padded * 4); add(padded * 4);
+    add(pairs * H * 2);
+    add(((pairs + 63) / 64 * g.experts + pairs) * 4);
+    add(256);
     return bytes;
 }
 

@@ -421,336 +421,3 @@ __global__ void __launch_bounds__(256, 2) tf_phase2_stream(const StreamArgs rout
     if (lo < r_items) tf_fc2_items<false, KSR>(routed, (int)lo, (int)(hi < r_items ? hi : r_items), red, dyn, dyn + 16 * (size_t)kmax, plan);
     if (hi > r_items) tf_fc2_items<true, KSS>(shared, (int)(lo > r_items ? lo - r_items : 0), (int)(hi - r_items), red, dyn, dyn + 16 * (size_t)kmax, plan);
 }
-
-// ---- One persistent launch for FC1 + SwiGLU, FC2 and the ordered sum (few rows) ---------------------------------------------
-// Five lists of units: routed FC1 items, shared FC1 items, routed FC2 items, shared FC2 items, sum units (64 output columns
-// of every row).  A unit only waits for units of earlier lists, and a workgroup never waits inside the FC1 lists, so with
-// every workgroup resident the waits end; they are bounded all the same (a bound that expires raises the error word and the
-// unit proceeds, so the grid always drains).  The weights of the next
-// unit are requested before the current unit's dependency wait and products, which keeps loads in flight across the
-// FC1 -> FC2 boundary.  Requires hidden == 2 * intermediate == 2 * shared intermediate (one unit = 16 loads a lane in both
-// projections).
-struct MegaArgs {
-    StreamArgs r1, s1, r2, s2;       // routed / shared operands of FC1 and FC2 (s1.w == nullptr: no shared expert)
-    uint32_t* counters;              // [0] queue head, [1] error word, [2] finished workgroups, [8 + tile] FC1 items done per routed tile,
-                                     // [8 + max_tiles + m] per shared tile, [8 + max_tiles + 4 + c] FC2 items done per 64-column group
-    int max_tiles;
-    const uint16_t* routes;          // [rows][topk][hidden] (= r2.out)
-    const uint16_t* shared_down;     // [rows][hidden] (= s2.out)
-    uint16_t* routed_out;            // [rows][hidden]
-    uint16_t* output;                // [rows][hidden]
-    int rows, live, topk;
-    const int32_t* live_ptr;         // device live-row count (takes precedence over `live`), may be null
-};
-template <int N>
-struct RawUnit {
-    u4v d[N];
-    uint32_t scale[4];
-};
-template <int TILES, int KS, int N>
-__device__ __forceinline__ void tf_raw_load_fp4(RawUnit<N>& u, const uint8_t* w, const uint8_t* scales, const int (&ntile)[TILES], int k, int ks_first, int lane) {
-    static_assert(TILES * KS == N && TILES * ((KS + 3) / 4) <= 4, "unit shape");
-    constexpr int SW = (KS + 3) / 4;
-#pragma unroll
-    for (int t = 0; t < TILES; ++t) {
-        const u4v* src = reinterpret_cast<const u4v*>(w) + ((size_t)ntile[t] * (k / 128) + ks_first) * 64 + lane;
-#pragma unroll
-        for (int s = 0; s < KS; ++s) u.d[t * KS + s] = tf_stream_load(src + s * 64);
-        const uint32_t* sc = reinterpret_cast<const uint32_t*>(scales) + ((size_t)ntile[t] * (k / 512) + ks_first / 4) * 64 + lane;
-#pragma unroll
-        for (int q = 0; q < SW; ++q) u.scale[t * SW + q] = __builtin_nontemporal_load(sc + q * 64) >> (8 * (ks_first & 3));
-    }
-}
-template <int TILES, int KS, int N>      // TILES weight tiles of two 16-byte planes a k-step
-__device__ __forceinline__ void tf_raw_load_fp8(RawUnit<N>& u, const uint8_t* w, const uint8_t* scales, const int (&ntile)[TILES], int k, int ks_first, int lane,
-                                                int bn, int bk) {
-    static_assert(TILES * KS * 2 == N && TILES * ((KS + 3) / 4) <= 4, "unit shape");
-    constexpr int SW = (KS + 3) / 4;
-    const int g = lane >> 4;
-#pragma unroll
-    for (int t = 0; t < TILES; ++t) {
-        const u4v* src = reinterpret_cast<const u4v*>(w) + (((size_t)ntile[t] * (k / 128) + ks_first) * 2) * 64 + lane;
-#pragma unroll
-        for (int s = 0; s < 2 * KS; ++s) u.d[t * 2 * KS + s] = tf_stream_load(src + s * 64);
-        const uint8_t* sc = scales + (size_t)((ntile[t] * 16 + (lane & 15)) / bn) * (k / bk);
-#pragma unroll
-        for (int q = 0; q < SW; ++q) {
-            uint32_t word = 0x7f7f7f7fu;
-#pragma unroll
-            for (int b = 0; b < 4; ++b)
-                if (4 * q + b < KS) word = (word & ~(0xffu << (8 * b))) | ((uint32_t)sc[((ks_first + 4 * q + b) * 128 + 32 * g) / bk] << (8 * b));
-            u.scale[t * SW + q] = word;
-        }
-    }
-}
-template <bool FP8, int KS, int N, int KSMAX>
-__device__ __forceinline__ v4f tf_raw_dot(const ATile<KSMAX>& a, const RawUnit<N>& u, int t) {
-    constexpr int SW = (KS + 3) / 4;
-    v4f acc = {0.f, 0.f, 0.f, 0.f};
-#pragma unroll
-    for (int s = 0; s < KS; ++s) {
-        const int sa = (int)a.scale[s >> 2], sb = (int)u.scale[t * SW + (s >> 2)];
-        if constexpr (FP8) {
-            const u4v lo = u.d[(t * KS + s) * 2], hi = u.d[(t * KS + s) * 2 + 1];
-            const v8i bv = v8i{(int)lo[0], (int)lo[1], (int)lo[2], (int)lo[3], (int)hi[0], (int)hi[1], (int)hi[2], (int)hi[3]};
-            TF_MFMA4(a.a[s], bv, acc, 0, s, sa, sb)
-        } else {
-            const u4v lo = u.d[t * KS + s];
-            const v8i bv = v8i{(int)lo[0], (int)lo[1], (int)lo[2], (int)lo[3], 0, 0, 0, 0};
-            TF_MFMA4(a.a[s], bv, acc, 4, s, sa, sb)
-        }
-    }
-    return acc;
-}
-
-enum { TF_U_FC1R = 0, TF_U_FC1S = 1, TF_U_FC2R = 2, TF_U_FC2S = 3, TF_U_SUM = 4, TF_U_END = 5 };
-struct PipeUnit { int kind, item, sub; };
-
-template <int KS1, int KS2, int OCC>
-__global__ void __launch_bounds__(256, OCC) tf_moe_stream(const MegaArgs p) {
-    constexpr int N = 2 * KS1;
-    static_assert(N == 4 * KS2, "one unit is 2 KS1 = 4 KS2 loads a lane");
-    __shared__ float red[8][2][4][64];
-    extern __shared__ uint8_t dyn[];
-    uint8_t* s_codes = dyn;
-    uint8_t* s_scales = dyn + 16 * (size_t)p.r2.k;
-    const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
-    const int tiles = tf_tiles(p.r1), mtiles = p.s1.w ? tf_tiles(p.s1) : 0;
-    const int per1r = p.r1.inter / 16, per1s = p.s1.w ? p.s1.inter / 16 : 0, per2r = p.r2.hidden / 64, per2s = p.s2.w ? p.s2.hidden / 32 : 0;
-    const int col_groups = p.output != nullptr ? p.r2.hidden / 64 : 0;
-    uint32_t* tile_done = p.counters + 8;
-    uint32_t* shared_done = tile_done + p.max_tiles;
-    uint32_t* col_done = shared_done + 4;
-
-    // This workgroup's share: a contiguous, cost-balanced range of every list (a shared FC1 item costs two units), visited in
-    // queue order.  All workgroups are resident together (the host sizes the grid to what fits), so a wait on another
-    // workgroup's items ends.
-    const long long G = gridDim.x, b = blockIdx.x;
-    const long long c1 = (long long)tiles * per1r + 2ll * mtiles * per1s, lo1 = c1 * b / G, hi1 = c1 * (b + 1) / G;
-    const long long n1r = (long long)tiles * per1r;
-    const long long c2 = (long long)tiles * per2r + (long long)mtiles * per2s, lo2 = c2 * b / G, hi2 = c2 * (b + 1) / G;
-    const long long n2r = (long long)tiles * per2r;
-    int range_lo[5], range_hi[5];
-    range_lo[0] = (int)(lo1 < n1r ? lo1 : n1r); range_hi[0] = (int)(hi1 < n1r ? hi1 : n1r);
-    range_lo[1] = (int)(((lo1 > n1r ? lo1 - n1r : 0) + 1) / 2); range_hi[1] = (int)(((hi1 > n1r ? hi1 - n1r : 0) + 1) / 2);
-    range_lo[2] = (int)(lo2 < n2r ? lo2 : n2r); range_hi[2] = (int)(hi2 < n2r ? hi2 : n2r);
-    range_lo[3] = (int)(lo2 > n2r ? lo2 - n2r : 0); range_hi[3] = (int)(hi2 > n2r ? hi2 - n2r : 0);
-    range_lo[4] = (int)(col_groups * b / G); range_hi[4] = (int)(col_groups * (b + 1) / G);
-    int list = 0, at = range_lo[0];
-    auto grab = [&]() -> PipeUnit {
-        while (list < 5 && at >= range_hi[list]) { ++list; if (list < 5) at = range_lo[list]; }
-        PipeUnit r;
-        r.sub = 0;
-        r.kind = list;          // TF_U_* follow the list order; 5 = end
-        r.item = list < 5 ? at++ : 0;
-        return r;
-    };
-    auto load_unit = [&](RawUnit<N>& u, const PipeUnit& pu) {
-        if (pu.kind == TF_U_FC1R) {
-            const ItemRef r = tf_item(p.r1, pu.item, per1r);
-            const int nt[2] = {r.j, per1r + r.j};
-            tf_raw_load_fp4<2, KS1, N>(u, p.r1.w + (size_t)r.expert * p.r1.w_expert_stride, p.r1.ws + (size_t)r.expert * p.r1.ws_expert_stride, nt, p.r1.k,
-                                       wave * KS1, lane);
-        } else if (pu.kind == TF_U_FC1S) {
-            const ItemRef r = tf_item(p.s1, pu.item, per1s);
-            const int nt[1] = {pu.sub * per1s + r.j};
-            tf_raw_load_fp8<1, KS1, N>(u, p.s1.w, p.s1.ws, nt, p.s1.k, wave * KS1, lane, p.s1.bn, p.s1.bk);
-        } else if (pu.kind == TF_U_FC2R) {
-            const ItemRef r = tf_item(p.r2, pu.item, per2r);
-            const int nt[4] = {4 * r.j, 4 * r.j + 1, 4 * r.j + 2, 4 * r.j + 3};
-            tf_raw_load_fp4<4, KS2, N>(u, p.r2.w + (size_t)r.expert * p.r2.w_expert_stride, p.r2.ws + (size_t)r.expert * p.r2.ws_expert_stride, nt, p.r2.k,
-                                       wave * KS2, lane);
-        } else if (pu.kind == TF_U_FC2S) {
-            const ItemRef r = tf_item(p.s2, pu.item, per2s);
-            const int nt[2] = {2 * r.j, 2 * r.j + 1};
-            tf_raw_load_fp8<2, KS2, N>(u, p.s2.w, p.s2.ws, nt, p.s2.k, wave * KS2, lane, p.s2.bn, p.s2.bk);
-        }
-    };
-    // Bounded wait until *counter >= target (thread 0 polls; every thread passes an acquire fence afterwards).
-    auto wait_for = [&](const uint32_t* counter, uint32_t target) {
-        if (tid == 0) {
-            int spins = 0;
-            while (__hip_atomic_load(counter, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT) < target) {
-                __builtin_amdgcn_s_sleep(1);
-                if (++spins > (1 << 20)) { atomicOr(p.counters + 1, 1u); break; }
-            }
-        }
-        __syncthreads();
-    };
-
-    PipeUnit cur = grab();
-    RawUnit<N> bcur, bnext;
-    load_unit(bcur, cur);
-    ATile<KS1> a;                    // FC2 units use its first KS2 k-steps (a workgroup never returns from FC2 to FC1 units)
-    int a_kind = -1, a_tile = -1;
-    v4f first_acc = {0.f, 0.f, 0.f, 0.f};
-    int parity = 0;
-    while (cur.kind != TF_U_END) {
-        PipeUnit nxt;
-        if (cur.kind == TF_U_FC1S && cur.sub == 0) { nxt = cur; nxt.sub = 1; }
-        else nxt = grab();
-        load_unit(bnext, nxt);
-        if (cur.kind == TF_U_FC1R || cur.kind == TF_U_FC1S) {
-            const bool shared = cur.kind == TF_U_FC1S;
-            const StreamArgs& q = shared ? p.s1 : p.r1;
-            const ItemRef r = tf_item(q, cur.item, shared ? per1s : per1r);
-            if (a_kind != cur.kind || a_tile != r.tile) {
-                long long row = -1;
-                if ((lane & 15) < r.valid) row = shared ? r.tile * 16 + (lane & 15) : q.token_map[r.tile * 16 + (lane & 15)] / q.topk;
-                tf_load_a<KS1>(a, q.a_codes, q.a_scales, row, q.k, q.act_block, wave * KS1, lane);
-                a_kind = cur.kind; a_tile = r.tile;
-            }
-            v4f c0, c1;
-            bool finish = true;
-            if (shared) {
-                const v4f c = tf_raw_dot<true, KS1, N>(a, bcur, 0);
-                if (cur.sub == 0) { first_acc = c; finish = false; }
-                c0 = first_acc; c1 = c;
-            } else {
-                c0 = tf_raw_dot<false, KS1, N>(a, bcur, 0);
-                c1 = tf_raw_dot<false, KS1, N>(a, bcur, 1);
-            }
-            if (finish) {
-                float (*slot)[2][4][64] = red + parity * 4;
-                parity ^= 1;
-#pragma unroll
-                for (int i = 0; i < 4; ++i) { slot[wave][0][i][lane] = c0[i]; slot[wave][1][i][lane] = c1[i]; }
-                __syncthreads();
-                if (wave == 0) {
-#pragma unroll
-                    for (int i = 0; i < 4; ++i) {
-                        const int m = 4 * (lane >> 4) + i;
-                        uint16_t h_bits = 0;
-                        if (m < r.valid) {
-                            float first = slot[0][0][i][lane], second = slot[0][1][i][lane];
-#pragma unroll
-                            for (int w2 = 1; w2 < 4; ++w2) {
-                                first = __fadd_rn(first, slot[w2][0][i][lane]);
-                                second = __fadd_rn(second, slot[w2][1][i][lane]);
-                            }
-                            float value;
-                            const size_t row = (size_t)(r.tile * 16 + m);
-                            if (shared) {
-                                const uint16_t gb = tf_to_bf16(first), ub = tf_to_bf16(second);
-                                if (q.tap != nullptr) {
-                                    q.tap[row * 2 * q.inter + 16 * r.j + (lane & 15)] = gb;
-                                    q.tap[row * 2 * q.inter + q.inter + 16 * r.j + (lane & 15)] = ub;
-                                }
-                                const float hi = tf_bf16(tf_to_bf16(q.limit)), lo = tf_bf16(tf_to_bf16(-q.limit));
-                                const float gv = fminf(tf_bf16(gb), hi), uv = fminf(fmaxf(tf_bf16(ub), lo), hi);
-                                value = __fmul_rn(gv / __fadd_rn(1.0f, tf_exp(-gv)), uv);
-                            } else {
-                                const float gv = fminf(second, q.limit), uv = fminf(q.limit, fmaxf(-q.limit, first));
-                                value = __fmul_rn(__fmul_rn(gv, tf_logistic(gv)), uv);
-                            }
-                            h_bits = tf_to_bf16(value);
-                        }
-                        tf_publish_bf16_pair(q.out, (size_t)(r.tile * 16 + m) * q.inter + 16 * r.j + (lane & 15), h_bits, m < r.valid, lane);
-                    }
-                    tf_stores_done();
-                    if (lane == 0) atomicAdd((shared ? shared_done : tile_done) + r.tile, 1u);
-                }
-            }
-        } else if (cur.kind == TF_U_FC2R || cur.kind == TF_U_FC2S) {
-            const bool shared = cur.kind == TF_U_FC2S;
-            const StreamArgs& q = shared ? p.s2 : p.r2;
-            const ItemRef r = tf_item(q, cur.item, shared ? per2s : per2r);
-            if (a_kind != cur.kind || a_tile != r.tile) {
-                wait_for((shared ? shared_done : tile_done) + r.tile, (uint32_t)(shared ? per1s : per1r));
-                const int per_row = q.k >> 3, group_lanes = q.act_block >> 3;
-                for (int e = tid; e < r.valid * per_row; e += blockDim.x) {
-                    const int m = e / per_row, c8 = e - m * per_row;
-                    const u4v wv = tf_acquire_u4v(reinterpret_cast<const u4v*>(q.a_bf16 + (size_t)(r.tile * 16 + m) * q.k) + c8);
-                    float v[8];
-#pragma unroll
-                    for (int i = 0; i < 4; ++i) { v[2 * i] = tf_bf16_lo(wv[i]); v[2 * i + 1] = tf_bf16_hi(wv[i]); }
-                    const float amax = tf_group_amax(v, group_lanes);
-                    const Quant8 c = tf_quant8(v, amax, q.min_amax);
-                    reinterpret_cast<u2v*>(s_codes + (size_t)m * q.k)[c8] = u2v{c.lo, c.hi};
-                    if ((c8 & (group_lanes - 1)) == 0) s_scales[m * (q.k / q.act_block) + c8 / group_lanes] = (uint8_t)c.exponent;
-                    if (q.q_codes != nullptr && r.j == 0) {
-                        reinterpret_cast<u2v*>(q.q_codes + (size_t)(r.tile * 16 + m) * q.k)[c8] = u2v{c.lo, c.hi};
-                        if ((c8 & (group_lanes - 1)) == 0)
-                            q.q_scales[(size_t)(r.tile * 16 + m) * (q.k / q.act_block) + c8 / group_lanes] = (uint8_t)c.exponent;
-                    }
-                }
-                __syncthreads();
-                tf_load_a<KS2, KS1>(a, s_codes, s_scales, (lane & 15) < r.valid ? (lane & 15) : -1, q.k, q.act_block, wave * KS2, lane);
-                a_kind = cur.kind; a_tile = r.tile;
-                __syncthreads();     // the staging area may be rewritten by the next tile only after every wave holds its A operand
-            }
-            const int nt_count = shared ? 2 : 4;
-#pragma unroll
-            for (int t = 0; t < 4; ++t) {
-                if (t < nt_count) {
-                    const v4f c = shared ? tf_raw_dot<true, KS2, N>(a, bcur, t) : tf_raw_dot<false, KS2, N>(a, bcur, t);
-#pragma unroll
-                    for (int i = 0; i < 4; ++i) red[(t >> 1) * 4 + wave][t & 1][i][lane] = c[i];
-                }
-            }
-            __syncthreads();
-            if (wave < nt_count) {
-                float (*slot)[2][4][64] = red + (wave >> 1) * 4;
-                const int which = wave & 1;
-#pragma unroll
-                for (int i = 0; i < 4; ++i) {
-                    const int m = 4 * (lane >> 4) + i;
-                    uint16_t bits = 0;
-                    size_t at = 0;
-                    if (m < r.valid) {
-                        float acc = slot[0][which][i][lane];
-#pragma unroll
-                        for (int w2 = 1; w2 < 4; ++w2) acc = __fadd_rn(acc, slot[w2][which][i][lane]);
-                        const int col = (shared ? 32 : 64) * r.j + 16 * wave + (lane & 15);
-                        if (!shared) {
-                            const int phys = r.tile * 16 + m;
-                            at = (size_t)q.token_map[phys] * q.hidden + col;
-                            bits = tf_to_bf16(__fmul_rn(acc, q.token_weights[phys]));
-                        } else {
-                            at = (size_t)(r.tile * 16 + m) * q.hidden + col;
-                            bits = tf_to_bf16(acc);
-                        }
-                    }
-                    tf_publish_bf16_pair(q.out, at, bits, m < r.valid, lane);
-                }
-                tf_stores_done();
-            }
-            __syncthreads();
-            if (tid == 0 && col_groups) atomicAdd(col_done + (shared ? r.j / 2 : r.j), 1u);
-        } else {   // TF_U_SUM: 64 columns of every row: ordered route sum, BF16, + shared (flush-to-zero add), BF16
-            const int c0 = cur.item * 64, hidden = p.r2.hidden;
-            wait_for(col_done + cur.item, (uint32_t)(tiles + 2 * mtiles));
-            const int live = p.live_ptr != nullptr ? min(p.rows, p.live_ptr[0]) : p.live;
-            for (int e = tid; e < p.rows * 8; e += blockDim.x) {
-                const int row = e >> 3, c8 = (c0 >> 3) + (e & 7);
-                const size_t at = (size_t)row * (hidden >> 3) + c8;
-                u4v routed = reinterpret_cast<const u4v*>(p.routed_out)[at];
-                if (row < live) {
-                    float sum[8];
-#pragma unroll
-                    for (int k = 0; k < 8; ++k) sum[k] = 0.f;
-                    for (int slot = 0; slot < p.topk; ++slot) {
-                        const u4v v = tf_acquire_u4v(reinterpret_cast<const u4v*>(p.routes + ((size_t)row * p.topk + slot) * hidden) + c8);
-#pragma unroll
-                        for (int j = 0; j < 4; ++j) {
-                            sum[2 * j] = __fadd_rn(sum[2 * j], tf_bf16_lo(v[j]));
-                            sum[2 * j + 1] = __fadd_rn(sum[2 * j + 1], tf_bf16_hi(v[j]));
-                        }
-                    }
-#pragma unroll
-                    for (int j = 0; j < 4; ++j) routed[j] = tf_pack_bf16(sum[2 * j], sum[2 * j + 1]);
-                    reinterpret_cast<u4v*>(p.routed_out)[at] = routed;
-                }
-                const u4v y = tf_acquire_u4v(reinterpret_cast<const u4v*>(p.shared_down) + at);
-                u4v o;
-#pragma unroll
-                for (int j = 0; j < 4; ++j)
-                    o[j] = tf_pack_bf16(tf_ftz(__fadd_rn(tf_ftz(tf_bf16_lo(routed[j])), tf_ftz(tf_bf16_lo(y[j])))),
-                                        tf_ftz(__fadd_rn(tf_ftz(tf_bf16_hi(routed[j])), tf_ftz(tf_bf16_hi(y[j])))));
-                reinterpret_cast<u4v*>(p.output)[at] = o;
-            }
-        }
-        bcur = bnext;
-        cur = nxt;
-    }
-}

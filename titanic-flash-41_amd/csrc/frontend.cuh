@@ -133,9 +133,7 @@ extern "C" __global__ void __launch_bounds__(512) ca_moe_frontend(
     const uint16_t* input, const int32_t* ids, const float* weights, uint8_t* packed, uint8_t* scales,
     int32_t* token_map, float* token_weights, int32_t* task_expert, int32_t* task_valid_rows,
     int32_t* expert_tile_base, int32_t rows, int32_t topk, int32_t experts, int32_t cols, int32_t groups,
-    int32_t tile_m, int32_t act_block, uint8_t* packed_min, uint8_t* scales_min, uint32_t* counters, int32_t counter_words) {
-    if (blockIdx.x == 0 && counters != nullptr)      // the queue and dependency counters of the streaming launch that follows
-        for (int i = threadIdx.x; i < counter_words; i += blockDim.x) counters[i] = 0u;
+    int32_t tile_m, int32_t act_block, uint8_t* packed_min, uint8_t* scales_min) {
     tf_frontend_run(input, ids, weights, packed, scales, packed_min, scales_min, token_map, token_weights, task_expert,
                     task_valid_rows, expert_tile_base, rows, topk, experts, cols, groups, tile_m, act_block, 0);
 }
@@ -150,11 +148,8 @@ extern "C" __global__ void __launch_bounds__(512) ca_moe_route_frontend(
     float* logits, const float* bias, const float* bias_alt, const long long* tokens, const int32_t* live,
     const int32_t* padding, int32_t rows, int32_t topk, int32_t experts, int32_t cols, int32_t groups, int32_t tile_m,
     int32_t owner_rows, int32_t act_block, uint8_t* packed_min, uint8_t* scales_min, int32_t scoring,
-    float route_scale, long long alt_token, const uint16_t* gate_w, uint32_t* sync, int32_t logit_blocks, uint32_t* counters,
-    int32_t counter_words) {
+    float route_scale, long long alt_token, const uint16_t* gate_w, uint32_t* sync, int32_t logit_blocks) {
     __shared__ int32_t s_ids[1024];
-    if (blockIdx.x == 0 && counters != nullptr)      // the queue and dependency counters of the streaming launch that follows
-        for (int i = threadIdx.x; i < counter_words; i += blockDim.x) counters[i] = 0u;
     __shared__ float s_weights[1024];
     const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6, waves = blockDim.x >> 6;
     const int first_logit_block = (int)gridDim.x - logit_blocks;

