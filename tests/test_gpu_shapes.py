@@ -1,0 +1,56 @@
+"""GPU parity over the shapes between and around the benchmark configurations, through the C++ host mirror: one row (the
+reference's 1-row micro plan), the 64 / 65-row boundary between the streaming and the grouped-GEMM paths, every supported
+contraction length, top-1 and top-8, the reference's expert count, live prefixes and padding rows on the many-row path.
+Same checks as the benchmark shapes (bit-exact routing, plan, codes; staged tolerance behind the matrix cores)."""
+import numpy as np
+import pytest
+
+from helpers import geometry, pkg, synth
+from test_gpu_layer import check_layer
+
+pytestmark = pytest.mark.gpu
+host = pkg.host
+
+
+def run_case(rows, hidden, experts, topk, inter, shared, mode, live=None, padding=None, tokens=None, **options):
+    g = geometry(hidden, experts, topk, inter, shared, mode)
+    name = "shape-%d-%d-%d-%d-%d-%d" % (rows, hidden, experts, topk, inter, shared)
+    ops = synth.LayerOperands(g, name, device="cuda")
+    x = synth.activations(name, rows, hidden)
+    layer = host.Layer(g, ops, rows, **options)
+    layer.set_tokens(tokens, live=live, padding=padding)
+    layer.run(x.cuda())
+    taps = layer.taps()
+    # gate products of more than 16 rows run on the matrix cores (another summation order than the oracle's)
+    stats = check_layer(g, ops, x, taps, tokens=tokens, live=live, padding=None if padding is None else np.array(padding, np.int32),
+                        exact_logits=rows <= 16, max_rel=2e-2)
+    layer.close()
+    return taps, stats
+
+
+@pytest.mark.parametrize("rows,hidden,experts,topk,inter,shared,mode", [
+    (1, 512, 8, 2, 512, 512, "reference"),          # one row, the smallest contraction
+    (1, 4096, 256, 6, 2048, 2048, "benchmark"),     # one row at the benchmark geometry
+    (3, 4096, 16, 1, 2048, 2048, "benchmark"),      # top-1
+    (16, 2048, 64, 8, 1024, 512, "benchmark"),      # top-8, H 2048 / I 1024, another shared width
+    (6, 1024, 384, 6, 512, 1024, "reference"),      # the reference's expert count and row count
+    (64, 1024, 32, 4, 512, 512, "reference"),       # the last row count of the streaming path
+    (65, 1024, 32, 4, 512, 512, "benchmark"),       # the first of the grouped-GEMM path
+    (130, 2048, 16, 2, 1024, 1024, "reference"),    # a second, partly filled row tile; K 1024 in FC2
+])
+def test_shape(rows, hidden, experts, topk, inter, shared, mode):
+    run_case(rows, hidden, experts, topk, inter, shared, mode)
+
+
+def test_one_live_row_of_a_wider_owner():
+    taps, _ = run_case(8, 1024, 16, 2, 512, 512, "reference", live=1)
+    assert (taps["ids"][1:] == -1).all() and not taps["weights"][1:].any()
+
+
+def test_many_rows_with_a_live_prefix_and_padding_rows():
+    rows = 200
+    padding = [-1] * rows
+    padding[150], padding[151] = 3, 7           # two padding rows repeat live rows' experts with zero weights
+    taps, _ = run_case(rows, 1024, 16, 2, 512, 512, "benchmark", live=152, padding=padding, route_front=False)
+    assert np.array_equal(taps["ids"][150], taps["ids"][3]) and np.array_equal(taps["ids"][151], taps["ids"][7])
+    assert not taps["weights"][150:152].any() and (taps["ids"][152:] == -1).all()
