@@ -106,7 +106,7 @@ class GpuLayer:
         self.live = z((1,), torch.int32)
         self.tokens = z((rows,), torch.int64)
         self.padding = torch.full((rows,), -1, dtype=torch.int32, device=d)
-        self.sync = z((64,), torch.int32)
+        self.sync = z((256,), torch.int32)
 
     def _compact(self, src, kernel, n, k, unit_bytes, unit_elems, extra=None):
         src = src.contiguous()
@@ -133,7 +133,7 @@ class GpuLayer:
         torch.cuda.synchronize()
         sp = ctypes.c_void_p(stream)
         fuse = rows * K <= 1024 if fuse_route is None else fuse_route
-        fuse_gate = fuse_gate and fuse and rows <= 16
+        fuse_gate = fuse_gate and fuse and rows <= STREAM_MAX_ROWS
         for off in range(0, rows, 16):
             if fuse_gate or (rows > 16 and rows > STREAM_MAX_ROWS):
                 break

@@ -139,8 +139,8 @@ extern "C" __global__ void __launch_bounds__(512) ca_moe_frontend(
 }
 // The front-end with the router's top-k inside: block 0 first routes every owner row from the gate's logits (and
 // applies padding routes), then plans; the other blocks quantize meanwhile (launch one block more).
-// With `gate_w` the gate product runs here too: `logit_blocks` further blocks (one wave per expert) compute the logits,
-// publish them and count themselves in at `sync`; block 0 waits for that count, bounded: if the count does not arrive it
+// With `gate_w` the gate product runs here too: `logit_blocks` further blocks (one wave per expert and four rows) compute the logits,
+// publish them and count themselves in at `sync` (eight words, 128 bytes apart: 1 KiB); block 0 waits for the counts, bounded: if the count does not arrive it
 // computes the logits itself, so the kernel always ends.  All blocks of this small grid are resident together.
 extern "C" __global__ void __launch_bounds__(512) ca_moe_route_frontend(
     const uint16_t* input, int32_t* ids, float* weights, uint8_t* packed, uint8_t* scales, int32_t* token_map,
@@ -154,24 +154,33 @@ extern "C" __global__ void __launch_bounds__(512) ca_moe_route_frontend(
     const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6, waves = blockDim.x >> 6;
     const int first_logit_block = (int)gridDim.x - logit_blocks;
     if (gate_w != nullptr && (int)blockIdx.x >= first_logit_block) {
-        const int e = ((int)blockIdx.x - first_logit_block) * waves + wave;
-        if (e < experts) tf_logits_expert(input, gate_w, logits, owner_rows, cols, experts, e, lane);
+        // one wave per (expert, group of four rows): every product of the launch runs in parallel
+        const int groups = (owner_rows + 3) >> 2, task = ((int)blockIdx.x - first_logit_block) * waves + wave;
+        const int e = task / groups, first_row = 4 * (task - e * groups);
+        if (e < experts)
+            tf_logits_expert(input + (size_t)first_row * cols, gate_w, logits + (size_t)first_row * experts, min(4, owner_rows - first_row), cols,
+                             experts, e, lane);
         tf_stores_done();
         __syncthreads();
-        if (threadIdx.x == 0) atomicAdd(sync, 1u);
+        // arrivals are spread over eight words, one cache line apart: atomics on one address serialize
+        const int lb = (int)blockIdx.x - first_logit_block;
+        if (threadIdx.x == 0) atomicAdd(sync + 32 * (lb & 7), 1u);
         return;
     }
     if (blockIdx.x == 0) {
         if (gate_w != nullptr) {
             __shared__ int arrived;
-            if (threadIdx.x == 0) {
+            if (threadIdx.x < 64) {      // lanes 0 .. 7 of the first wave watch one arrival word each
+                const int word = lane & 7;
+                const uint32_t expected = (uint32_t)((logit_blocks - word + 7) >> 3);        // logit blocks lb with lb % 8 == word
                 int ok = 0;
                 for (int spin = 0; spin < (1 << 18); ++spin) {
-                    if (__hip_atomic_load(sync, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT) >= (uint32_t)logit_blocks) { ok = 1; break; }
+                    const bool here = __hip_atomic_load(sync + 32 * word, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT) >= expected;
+                    if (__all(here)) { ok = 1; break; }
                     __builtin_amdgcn_s_sleep(2);
                 }
-                __hip_atomic_store(sync, 0u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
-                arrived = ok;
+                if (lane < 8) __hip_atomic_store(sync + 32 * word, 0u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+                if (lane == 0) arrived = ok;
             }
             __syncthreads();
             if (!arrived)

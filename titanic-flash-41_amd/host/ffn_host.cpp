@@ -255,7 +255,7 @@ std::optional<RouteOperands> Router::run_routed(uint64_t input, size_t input_len
     ensure(!stream_set_ || stream_ == stream.raw(), "router needs one ordered stream");                        // :340-345
     stream_ = stream.raw(); stream_set_ = true;
     const uint64_t gate = weights_->ptr("ffn.gate.weight");
-    const bool gate_in_front = fused && gate_front && rows_ <= 16;
+    const bool gate_in_front = fused && gate_front && rows_ <= 64;
     if (gate_in_front) {
     } else if (rows_ <= 64) {
         for (size_t offset = 0; offset < rows_; offset += 16)                                                  // :351-364
@@ -314,7 +314,7 @@ Workspace::Workspace(std::shared_ptr<const Native> native, size_t rows) : native
     add("token_map_ptr", padded * 4); add("token_weights_ptr", padded * 4);
     add("scatter_ptr", pairs * H * 2);
     add("plan_scratch_ptr", ((pairs + 63) / 64 * g.experts + pairs) * 4);
-    add("sync_ptr", 256);
+    add("sync_ptr", 1024);
     scratch_ = Buffer<uint8_t>(at);
     scratch_.zero();                                                                                          // scratch_initializer "zero", src/moe.rs:440
     output_ = Buffer<uint16_t>(rows * H);

@@ -131,7 +131,7 @@ private:
 };
 
 // Operands a router hands to the experts' front-end when its top-k runs there (src/moe.rs:181-200 RouteOperands).
-// gate_w != 0: the gate product is left to the front-end too (owners of at most 16 rows).
+// gate_w != 0: the gate product is left to the front-end too (owners of at most 64 rows).
 struct RouteOperands { uint64_t logits, bias, bias_alt, tokens, live, padding, ids, weights; size_t owner_rows; uint64_t gate_w; };
 // Operands of the shared expert when it is folded into the routed experts' launches (entry "ffn.experts_with_shared"):
 // prepared w13 / scales / w2 / scales, activation (BF16), its codes and scales, the up-projection tap, the output.
@@ -207,7 +207,7 @@ public:
         bool overlap = true;        // FFN_OVERLAP: shared expert on an auxiliary stream beside the routed experts (:518-522)
         bool sum_shared = true;     // FFN_SUM_SHARED: fused route sum + shared addition (:1037-1046)
         bool route_front = true;    // MOE_ROUTE_FRONT: the router's top-k inside the experts' front-end (:986-990)
-        bool gate_front = true;     // the gate product inside the front-end launch as well (owners of at most 16 rows)
+        bool gate_front = true;     // the gate product inside the front-end launch as well (owners of at most 64 rows)
         bool fold_shared = true;    // few rows: the shared expert's weights stream inside the routed experts' two launches
                                     // (one queue, no cross-stream join); takes precedence over `overlap`
     };
