@@ -106,3 +106,18 @@ def check_rows(g, ops, x, sub, taps, sample):
     rel, mean = error_stats(sub["out"], want["out"])
     assert rel <= 1e-2 and mean <= 1e-3, (rel, mean)
     return rel, mean
+
+
+def test_the_bf16_intermediate_is_only_a_tap_on_the_many_row_path():
+    from helpers import pkg
+    g, ops, x = small_wide("benchmark", 300)
+    layer = pkg.host.Layer(g, ops, 300)
+    layer.set_tokens()
+    layer.run(x.cuda())
+    with_tap = layer.taps()
+    layer.keep_intermediate(False)
+    layer.run(x.cuda())
+    without = layer.taps()
+    for name in ["hq", "hs", "route_out", "out"]:
+        assert np.array_equal(with_tap[name], without[name]), name
+    layer.close()

@@ -103,8 +103,11 @@ int launch_dynamic(const Context& c, bool route, const uint64_t* p, const int32_
     const ca_geometry& g = c.g;
     const int rows = sc[S_TOKENS], tile_m = sc[S_TILE_M], groups = sc[S_GROUPS], max_tiles = sc[S_MAX_TILES];
     if (rows < 1 || rows > sc[S_MAX_ROWS] || groups < 1 || max_tiles < 1 || sc[S_ROWS_PADDED] != max_tiles * tile_m) return -1;
+    // many rows: the BF16 copy of the intermediate is a tap (FC2 reads the codes); few rows: it is what FC2 reads
     for (int i = 0; i < P_DYN_COUNT; ++i)
-        if (!p[i] && i != P_PACKED_MIN && i != P_SCALES_MIN && i != P_INTER_CODES && i != P_INTER_SCALES && i != P_PLAN_SCRATCH) return -1;
+        if (!p[i] && i != P_PACKED_MIN && i != P_SCALES_MIN && i != P_INTER_CODES && i != P_INTER_SCALES && i != P_PLAN_SCRATCH &&
+            !(i == P_INTER && rows > TF_STREAM_MAX_ROWS))
+            return -1;
     if (!supported_k(g.hidden) || !supported_k(g.intermediate)) return -4;
     const long long pairs = (long long)rows * g.topk;
     // capacity of the reference's contracts (max_phys_tiles): A = min(E, pairs) experts open a tile each and the other routes fill

@@ -90,6 +90,12 @@ class Layer:
         self._check(self.lib.tfh_layer_set_tokens(self.h, ids.ctypes.data, self.rows if live is None else live,
                                                   None if pad is None else pad.ctypes.data, self._err, 512))
 
+    def keep_intermediate(self, on):
+        """Many rows: whether FC1 also stores the BF16 intermediate (a tap; FC2 reads the FP8 codes)."""
+        self.lib.tfh_layer_keep_intermediate.argtypes = [ctypes.c_void_p, ctypes.c_int]
+        self.lib.tfh_layer_keep_intermediate.restype = None
+        self.lib.tfh_layer_keep_intermediate(self.h, int(on))
+
     def run(self, x):
         assert x.is_cuda and x.is_contiguous() and x.numel() == self.rows * self.g.hidden
         self._check(self.lib.tfh_layer_run(self.h, x.data_ptr(), self._err, 512))

@@ -57,6 +57,8 @@ void* tfh_layer_create(const char* kernel_library, const ca_geometry* geometry, 
     return h;
 }
 void tfh_layer_destroy(void* handle) { delete (Handle*)handle; }
+// Many rows: drop (0) or keep (1) the BF16 tap of the routed intermediate.
+void tfh_layer_keep_intermediate(void* handle, int on) { ((Handle*)handle)->workspace->keep_intermediate(on != 0); }
 
 int tfh_layer_set_tokens(void* handle, const int64_t* ids, int live, const int32_t* padding, char* error, size_t error_len) {
     Handle* h = (Handle*)handle;

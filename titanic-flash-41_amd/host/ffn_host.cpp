@@ -341,6 +341,7 @@ void Workspace::pointers(const Expert& expert, uint64_t input, const Buffer<int3
     p[0] = input; p[1] = ids.ptr(); p[2] = routing_weights.ptr();
     for (int i = 0; i < 12; ++i) p[3 + i] = at(scratch_names[i]);
     if (!emit_shared_input_) p[5] = p[6] = 0;
+    if (!keep_intermediate_ && rows_ > 64) p[7] = 0;
     p[15] = expert.region("w13").first; p[16] = expert.region("s13").first; p[17] = expert.region("w2").first; p[18] = expert.region("s2").first;
     p[19] = at("scatter_ptr"); p[20] = at("plan_scratch_ptr");
 }

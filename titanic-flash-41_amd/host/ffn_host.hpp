@@ -187,8 +187,10 @@ public:
     size_t bytes_of(const std::string& name) const;
     size_t scratch_bytes() const { return scratch_.bytes(); }
     void emit_shared_input(bool on) { emit_shared_input_ = on; }
+    // many rows: whether FC1 also stores the BF16 intermediate (a tap: FC2 reads the codes).  Few rows always keep it.
+    void keep_intermediate(bool on) { keep_intermediate_ = on; }
 private:
-    bool emit_shared_input_ = true;
+    bool emit_shared_input_ = true, keep_intermediate_ = true;
     void pointers(const Expert& expert, uint64_t input, const Buffer<int32_t>& ids, const Buffer<float>& routing_weights, uint64_t* p) const;
     void guard_stream(const Stream& stream);
     std::shared_ptr<const Native> native_;
