@@ -74,6 +74,26 @@ class Layer:
             raise HostError(self._err.value.decode())
         self.h = ctypes.c_void_p(self.h)
 
+    @classmethod
+    def from_checkpoint(cls, geometry, root, prefix, rows, overlap=True, sum_shared=True, route_front=True, code_scales=False, fold_shared=True,
+                        gate_front=True):
+        """The layer with its operands read from a safetensors checkpoint directory by the host mirror's own scanner."""
+        self = cls.__new__(cls)
+        self.lib = load()
+        native.load()
+        self.g, self.rows = geometry, rows
+        self._err = ctypes.create_string_buffer(512)
+        self.lib.tfh_layer_create_from_checkpoint.restype = ctypes.c_void_p
+        self.lib.tfh_layer_create_from_checkpoint.argtypes = [ctypes.c_char_p, ctypes.c_void_p, ctypes.c_int, ctypes.c_char_p, ctypes.c_char_p] + \
+            [ctypes.c_int] * 6 + [ctypes.c_char_p, ctypes.c_size_t]
+        self.h = self.lib.tfh_layer_create_from_checkpoint(native.KERNEL_LIB.encode(), ctypes.byref(geometry), rows, root.encode(), prefix.encode(),
+                                                           int(overlap), int(sum_shared), int(route_front), int(code_scales), int(fold_shared),
+                                                           int(gate_front), self._err, 512)
+        if not self.h:
+            raise HostError(self._err.value.decode())
+        self.h = ctypes.c_void_p(self.h)
+        return self
+
     def _check(self, status):
         if status < 0:
             raise HostError(self._err.value.decode())
@@ -169,3 +189,25 @@ class Layer:
         v = (ctypes.c_longlong * 8)()
         self.lib.tfh_layer_info(self.h, v)
         return dict(zip(["tile_m", "max_tiles", "scratch_bytes", "atlas_bytes", "expert_bytes", "scale_code_bytes", "raw_rows", "coded_rows"], v))
+
+
+def checkpoint_layer(geometry, root, prefix):
+    """Scans a safetensors checkpoint directory and assembles one layer's operands on the host (no device involved).
+    Returns (dict of numpy arrays in the canonical layout, tensors in the checkpoint, shards)."""
+    lib = load()
+    g = geometry
+    H, E, I, S = g.hidden, g.experts, g.intermediate, g.shared_intermediate
+    shapes = [("gate_w", np.uint16, (E, H)), ("bias", np.float32, (E,)), ("bias_alt", np.float32, (E,)),
+              ("w13", np.uint8, (E, 2 * I, H // 2)), ("s13", np.uint8, (E, 2 * I, H // 32)), ("w2", np.uint8, (E, H, I // 2)),
+              ("s2", np.uint8, (E, H, I // 32)), ("sh_w13", np.uint8, (2 * S, H)), ("sh_s13", np.uint8, (2 * S // g.shared_bn, H // g.shared_bk)),
+              ("sh_w2", np.uint8, (H, S)), ("sh_s2", np.uint8, (H // g.shared_bn, S // g.shared_bk))]
+    arrays = {n: np.empty(shape, dtype) for n, dtype, shape in shapes}
+    outs = (ctypes.c_void_p * 11)(*[arrays[n].ctypes.data for n, _, _ in shapes])
+    sizes = (ctypes.c_size_t * 11)(*[arrays[n].nbytes for n, _, _ in shapes])
+    counts = (ctypes.c_size_t * 2)()
+    err = ctypes.create_string_buffer(512)
+    lib.tfh_checkpoint_layer.argtypes = [ctypes.c_char_p, ctypes.c_char_p, ctypes.c_void_p, ctypes.c_void_p, ctypes.c_void_p, ctypes.c_void_p,
+                                         ctypes.c_char_p, ctypes.c_size_t]
+    if lib.tfh_checkpoint_layer(root.encode(), prefix.encode(), ctypes.byref(geometry), outs, sizes, counts, err, 512) != 0:
+        raise HostError(err.value.decode())
+    return arrays, counts[0], counts[1]

@@ -1,6 +1,7 @@
 // Flat C interface of the host mirror for the python tests and the benchmark (ctypes): one handle per layer instance.
 // Every function returns 0 on success and -1 on failure with the message in the caller's buffer.
 #include "ffn_host.hpp"
+#include "checkpoint.hpp"
 #include <cstdio>
 #include <cstring>
 
@@ -31,30 +32,72 @@ int guarded(char* error, size_t error_len, F&& body) {
 
 extern "C" {
 
+namespace {
+void build_layer(Handle* h, const char* kernel_library, const ca_geometry* geometry, int rows, const tf::Weights::Host& src, bool on_device,
+                 int overlap, int sum_shared, int route_front, int code_scales, int fold_shared, int gate_front) {
+    h->native = std::make_shared<tf::Native>(kernel_library, *geometry);
+    h->weights = on_device ? std::make_shared<tf::Weights>(*geometry, src, true) : std::make_shared<tf::Weights>(*geometry, src);
+    h->prepared = tf::prepare_layer(*h->native, *h->weights, 0);
+    if (code_scales) h->scale_code = tf::code_layer_scales(*h->native, *h->weights, h->prepared);
+    tf::LayerFfn::Options options;
+    options.overlap = overlap != 0; options.sum_shared = sum_shared != 0; options.route_front = route_front != 0; options.fold_shared = fold_shared != 0; options.gate_front = gate_front != 0;
+    h->options = options;
+    h->layer = std::make_unique<tf::LayerFfn>(h->native, h->weights, h->prepared, (size_t)rows, options);
+    h->workspace = std::make_unique<tf::Workspace>(h->native, (size_t)rows);
+    std::vector<int64_t> ids((size_t)rows, 0);
+    h->tokens = std::make_unique<tf::TokenRows>(ids.data(), (size_t)rows, (size_t)rows);
+    h->stream = std::make_unique<tf::Stream>();
+    h->rows = (size_t)rows;
+}
+tf::Weights::Host host_view(const tf::LayerOperandsHost& o) {
+    return tf::Weights::Host{o.gate_w.data(), o.bias.data(), o.bias_alt.data(), o.w13.data(), o.s13.data(), o.w2.data(), o.s2.data(),
+                             o.sh_w13.data(), o.sh_s13.data(), o.sh_w2.data(), o.sh_s2.data()};
+}
+}  // namespace
+
 // operands: gate_w, bias, bias_alt, w13, s13, w2, s2, sh_w13, sh_s13, sh_w2, sh_s2 (canonical checkpoint layout).
 void* tfh_layer_create(const char* kernel_library, const ca_geometry* geometry, int rows, const void* const* operands, int operands_on_device,
                        int overlap, int sum_shared, int route_front, int code_scales, int fold_shared, int gate_front, char* error, size_t error_len) {
     Handle* h = new Handle;
     const int status = guarded(error, error_len, [&] {
-        h->native = std::make_shared<tf::Native>(kernel_library, *geometry);
         tf::Weights::Host src{(const uint16_t*)operands[0], (const float*)operands[1], (const float*)operands[2], (const uint8_t*)operands[3],
                               (const uint8_t*)operands[4], (const uint8_t*)operands[5], (const uint8_t*)operands[6], (const uint8_t*)operands[7],
                               (const uint8_t*)operands[8], (const uint8_t*)operands[9], (const uint8_t*)operands[10]};
-        h->weights = operands_on_device ? std::make_shared<tf::Weights>(*geometry, src, true) : std::make_shared<tf::Weights>(*geometry, src);
-        h->prepared = tf::prepare_layer(*h->native, *h->weights, 0);
-        if (code_scales) h->scale_code = tf::code_layer_scales(*h->native, *h->weights, h->prepared);
-        tf::LayerFfn::Options options;
-        options.overlap = overlap != 0; options.sum_shared = sum_shared != 0; options.route_front = route_front != 0; options.fold_shared = fold_shared != 0; options.gate_front = gate_front != 0;
-        h->options = options;
-        h->layer = std::make_unique<tf::LayerFfn>(h->native, h->weights, h->prepared, (size_t)rows, options);
-        h->workspace = std::make_unique<tf::Workspace>(h->native, (size_t)rows);
-        std::vector<int64_t> ids((size_t)rows, 0);
-        h->tokens = std::make_unique<tf::TokenRows>(ids.data(), (size_t)rows, (size_t)rows);
-        h->stream = std::make_unique<tf::Stream>();
-        h->rows = (size_t)rows;
+        build_layer(h, kernel_library, geometry, rows, src, operands_on_device != 0, overlap, sum_shared, route_front, code_scales, fold_shared, gate_front);
     });
     if (status != 0) { delete h; return nullptr; }
     return h;
+}
+// The same layer with its operands read from a safetensors checkpoint directory (index + shards), layer prefix e.g. "layers.3".
+void* tfh_layer_create_from_checkpoint(const char* kernel_library, const ca_geometry* geometry, int rows, const char* root, const char* prefix,
+                                       int overlap, int sum_shared, int route_front, int code_scales, int fold_shared, int gate_front, char* error,
+                                       size_t error_len) {
+    Handle* h = new Handle;
+    const int status = guarded(error, error_len, [&] {
+        const tf::Checkpoint checkpoint = tf::Checkpoint::scan(root);
+        const tf::LayerOperandsHost operands = tf::load_ffn_layer(checkpoint, prefix, *geometry);
+        build_layer(h, kernel_library, geometry, rows, host_view(operands), false, overlap, sum_shared, route_front, code_scales, fold_shared, gate_front);
+    });
+    if (status != 0) { delete h; return nullptr; }
+    return h;
+}
+// Checkpoint scan and operand assembly alone (no device): fills the caller's eleven host buffers (sizes in bytes, checked) in
+// the order of tfh_layer_create's operands; counts[0] = tensors in the checkpoint, counts[1] = shards.
+int tfh_checkpoint_layer(const char* root, const char* prefix, const ca_geometry* geometry, void* const* out, const size_t* sizes, size_t* counts,
+                         char* error, size_t error_len) {
+    return guarded(error, error_len, [&] {
+        const tf::Checkpoint checkpoint = tf::Checkpoint::scan(root);
+        const tf::LayerOperandsHost o = tf::load_ffn_layer(checkpoint, prefix, *geometry);
+        const void* src[11] = {o.gate_w.data(), o.bias.data(), o.bias_alt.data(), o.w13.data(), o.s13.data(), o.w2.data(), o.s2.data(),
+                               o.sh_w13.data(), o.sh_s13.data(), o.sh_w2.data(), o.sh_s2.data()};
+        const size_t bytes[11] = {o.gate_w.size() * 2, o.bias.size() * 4, o.bias_alt.size() * 4, o.w13.size(), o.s13.size(), o.w2.size(), o.s2.size(),
+                                  o.sh_w13.size(), o.sh_s13.size(), o.sh_w2.size(), o.sh_s2.size()};
+        for (int i = 0; i < 11; ++i) {
+            tf::ensure(sizes[i] == bytes[i], "operand buffer size");
+            std::memcpy(out[i], src[i], bytes[i]);
+        }
+        counts[0] = checkpoint.tensors(); counts[1] = checkpoint.shards();
+    });
 }
 void tfh_layer_destroy(void* handle) { delete (Handle*)handle; }
 // Many rows: drop (0) or keep (1) the BF16 tap of the routed intermediate.

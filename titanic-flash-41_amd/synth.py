@@ -138,3 +138,53 @@ def zipf_bias(experts, s=1.1, strength=1.0, device="cpu"):
 
 def activations(config_name, rows, hidden, device="cpu", step=0, seed=BASE_SEED):
     return to_bf16_bits(normal("%s/x.%d" % (config_name, step), (rows, hidden), device=device, seed=seed))
+
+
+def write_checkpoint(ops, root, prefix="layers.0", shards=2):
+    """Writes one layer's canonical operands as a safetensors checkpoint directory with the reference's tensor names, dtypes
+    and shapes (src/layout.rs:247-275): per expert w1 (gate) / w3 (up) / w2 packed FP4 (I8 [n][k/2]) with F8_E8M0 scales
+    [n][k/32]; shared expert w1 / w3 / w2 F8_E4M3 with F8_E8M0 block scales; gate weight BF16, bias and bias_vl F32.
+    Plain file writing (8-byte little-endian header length, JSON header, tensor bytes): nothing of the format needs a library."""
+    import json
+    import os
+    import numpy as np
+    g = ops.geometry
+    I, S = g.intermediate, g.shared_intermediate
+    def raw(t):
+        return t.detach().cpu().contiguous().view(-1).view(dtype=torch.uint8).numpy().tobytes()
+    tensors = []
+    for e in range(g.experts):
+        x = "%s.ffn.experts.%d." % (prefix, e)
+        tensors += [(x + "w1.weight", "I8", ops.w13[e, I:]), (x + "w1.scale", "F8_E8M0", ops.s13[e, I:]),
+                    (x + "w3.weight", "I8", ops.w13[e, :I]), (x + "w3.scale", "F8_E8M0", ops.s13[e, :I]),
+                    (x + "w2.weight", "I8", ops.w2[e]), (x + "w2.scale", "F8_E8M0", ops.s2[e])]
+    sh = prefix + ".ffn.shared_experts."
+    rows13 = ops.sh_s13.shape[0] // 2
+    tensors += [(sh + "w1.weight", "F8_E4M3", ops.sh_w13[:S]), (sh + "w1.scale", "F8_E8M0", ops.sh_s13[:rows13]),
+                (sh + "w3.weight", "F8_E4M3", ops.sh_w13[S:]), (sh + "w3.scale", "F8_E8M0", ops.sh_s13[rows13:]),
+                (sh + "w2.weight", "F8_E4M3", ops.sh_w2), (sh + "w2.scale", "F8_E8M0", ops.sh_s2),
+                (prefix + ".ffn.gate.weight", "BF16", ops.gate_w), (prefix + ".ffn.gate.bias", "F32", ops.bias),
+                (prefix + ".ffn.gate.bias_vl", "F32", ops.bias_alt)]
+    os.makedirs(root, exist_ok=True)
+    weight_map = {}
+    per = -(-len(tensors) // shards)
+    for k in range(shards):
+        part = tensors[k * per:(k + 1) * per]
+        if not part:
+            continue
+        name = "model-%05d-of-%05d.safetensors" % (k + 1, shards)
+        header, at, blobs = {"__metadata__": {"format": "pt"}}, 0, []
+        for key, dtype, t in part:
+            b = raw(t)
+            header[key] = {"dtype": dtype, "shape": list(t.shape), "data_offsets": [at, at + len(b)]}
+            at += len(b)
+            blobs.append(b)
+            weight_map[key] = name
+        text = json.dumps(header).encode()
+        with open(os.path.join(root, name), "wb") as f:
+            f.write(len(text).to_bytes(8, "little"))
+            f.write(text)
+            for b in blobs:
+                f.write(b)
+    with open(os.path.join(root, "model.safetensors.index.json"), "w") as f:
+        json.dump({"metadata": {}, "weight_map": weight_map}, f)
