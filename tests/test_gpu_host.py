@@ -1,6 +1,8 @@
 """GPU parity of the C++ host mirror (LayerFfn / Router / Workspace / prepare_layer over the C ABI) against the CPU oracle,
 in every schedule the reference has (dual-stream shared branch, fused or separate sum, top-k inside or before the
 front-end), eager and as a replayed graph."""
+import ctypes
+
 import numpy as np
 import pytest
 import torch
@@ -101,4 +103,24 @@ def test_paired_owners_pool_into_one_launch():
     assert rel <= 2e-2 and mean <= 1e-3, (rel, mean)
     with pytest.raises(host.HostError, match="paired FFN needs two live prefixes"):
         layer.pair_run(xa_d, tokens_a, 0, xb_d, tokens_b, live_b)
+    layer.close()
+
+
+@pytest.mark.parametrize("overlap", [False, True])
+def test_prequantized_shared_input(overlap):
+    # LayerFfn::run_quantized_input (src/ffn.rs:974-1047, 1053-1065): the boundary hands over the rows' codes in the shared
+    # expert's quantizer flavour; the result is the one the layer computes when it quantizes the rows itself
+    g, ops, x, rows = make("c1", "reference", "cpu")
+    layer = host.Layer(g, ops, rows, overlap=overlap)
+    layer.set_tokens()
+    layer.run(x.cuda())
+    want = layer.taps()
+    codes, scales = oracle.quantize_rows(x.numpy().view(np.uint16), g.act_block, 1e-4)
+    layer.run_quantized(x.cuda(), torch.from_numpy(codes).cuda(), torch.from_numpy(scales).cuda())
+    got = layer.taps()
+    for name in ["shared_up", "shared_act", "shared_down", "route_out", "out"]:
+        assert np.array_equal(got[name], want[name]), name
+    with pytest.raises(host.HostError, match="prequantized normalized shared input requires both operands"):
+        layer.lib.tfh_layer_run_quantized.argtypes = None
+        layer._check(layer.lib.tfh_layer_run_quantized(layer.h, ctypes.c_uint64(x.cuda().data_ptr()), ctypes.c_uint64(0), ctypes.c_uint64(0), layer._err, 512))
     layer.close()

@@ -120,6 +120,11 @@ class Layer:
         assert x.is_cuda and x.is_contiguous() and x.numel() == self.rows * self.g.hidden
         self._check(self.lib.tfh_layer_run(self.h, x.data_ptr(), self._err, 512))
 
+    def run_quantized(self, x, codes, scales):
+        """One pass with the shared expert fed from the caller's pre-quantized rows (E4M3 codes, UE8M0 scales; device tensors)."""
+        self.lib.tfh_layer_run_quantized.argtypes = [ctypes.c_void_p, ctypes.c_uint64, ctypes.c_uint64, ctypes.c_uint64, ctypes.c_char_p, ctypes.c_size_t]
+        self._check(self.lib.tfh_layer_run_quantized(self.h, x.data_ptr(), codes.data_ptr(), scales.data_ptr(), self._err, 512))
+
     def capture(self, xs):
         """Captures one pass over each tensor of `xs` (or the single tensor `xs`), in order, into one graph."""
         xs = [xs] if not isinstance(xs, (list, tuple)) else list(xs)

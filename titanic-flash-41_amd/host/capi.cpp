@@ -118,6 +118,16 @@ int tfh_layer_run(void* handle, uint64_t input, char* error, size_t error_len) {
         h->stream->synchronize();
     });
 }
+// One eager pass with the shared expert fed from pre-quantized input (LayerFfn::run_quantized_input): `codes` / `scales` are
+// device addresses of the rows' E4M3 codes and UE8M0 scales in the shared expert's quantizer flavour.
+int tfh_layer_run_quantized(void* handle, uint64_t input, uint64_t codes, uint64_t scales, char* error, size_t error_len) {
+    Handle* h = (Handle*)handle;
+    return guarded(error, error_len, [&] {
+        const tf::LayerFfn::QuantizedInput q{codes, scales};
+        h->layer->run_quantized_input(*h->workspace, input, h->rows * (size_t)h->native->geometry().hidden, &q, *h->tokens, *h->stream);
+        h->stream->synchronize();
+    });
+}
 // Captures one pass over each of `count` inputs, in order, into one graph (the reference captures its whole forward, forty
 // layers' passes, into one graph and replays it: src/probe.rs:1527-1542, src/cuda.rs:2068-2153); returns the graph's index.
 int tfh_layer_capture(void* handle, const uint64_t* inputs, int count, char* error, size_t error_len) {

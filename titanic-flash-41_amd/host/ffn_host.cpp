@@ -439,24 +439,28 @@ void LayerFfn::run_shared(const Workspace& workspace, uint64_t input, const Stre
         const int32_t qs[3] = {(int32_t)rows_, native_->geometry().hidden, 0};
         native_->primitive(3, q, 5, qs, 3, stream.raw(), "gemm.mxfp8_quant_cute");
     }
-    const uint64_t p[11] = {workspace.at("shared_a_storage_ptr"), workspace.at("shared_scale_storage_ptr"), shared_w13_.values, shared_w13_.scales,
-                            shared_w2_.values, shared_w2_.scales, activation_.ptr(), activation_codes_.ptr(), activation_scales_.ptr(),
-                            shared_up_.ptr(), shared_down_.ptr()};
+    run_shared_quantized(workspace.at("shared_a_storage_ptr"), workspace.at("shared_scale_storage_ptr"), stream);
+}
+void LayerFfn::run_shared_quantized(uint64_t codes, uint64_t scales, const Stream& stream) {
+    ensure(codes && scales, "prequantized normalized shared input requires both operands");
+    const uint64_t p[11] = {codes, scales, shared_w13_.values, shared_w13_.scales, shared_w2_.values, shared_w2_.scales, activation_.ptr(),
+                            activation_codes_.ptr(), activation_scales_.ptr(), shared_up_.ptr(), shared_down_.ptr()};
     const int32_t s[1] = {(int32_t)rows_};
     native_->primitive(5, p, 11, s, 1, stream.raw(), "ffn.shared_expert");
 }
 void LayerFfn::add_shared(const Workspace& workspace, const Stream& stream) {                                  // :1066-1084
     native_->ffn_add((int)rows_, workspace.output().ptr(), shared_down_.ptr(), output_.ptr(), stream.raw());
 }
-void LayerFfn::run(Workspace& workspace, uint64_t input, size_t input_len, const TokenRows& tokens, const Stream& stream) {   // :974-1047
+void LayerFfn::run_quantized_input(Workspace& workspace, uint64_t input, size_t input_len, const QuantizedInput* quantized, const TokenRows& tokens,
+                                   const Stream& stream) {                                                      // :974-1047
     const ca_geometry& g = native_->geometry();
     ensure(workspace.rows() == rows_, "MoE workspace context mismatch");
     const bool fused = options_.route_front && rows_ * g.topk <= 1024;                                          // :988-990
     // Dual-stream schedule (:1007-1010, :1028-1036): the shared branch forks before routing, quantizes the input itself
     // and joins before the sum.  Without the branch the front-end emits the shared-flavour codes beside the routed ones.
-    const bool fold = options_.fold_shared && rows_ <= 64;
+    const bool fold = options_.fold_shared && rows_ <= 64 && !quantized;      // given codes: the shared expert runs from them, beside the routed launches
     const bool branch = branch_stream_ && !fold;
-    workspace.emit_shared_input(!branch);
+    workspace.emit_shared_input(!branch && !quantized);
     if (fold) {
         const SharedOperands shared{shared_w13_.values, shared_w13_.scales, shared_w2_.values, shared_w2_.scales, activation_.ptr(),
                                     activation_codes_.ptr(), activation_scales_.ptr(), shared_up_.ptr(), shared_down_.ptr(),
@@ -472,13 +476,15 @@ void LayerFfn::run(Workspace& workspace, uint64_t input, size_t input_len, const
     if (branch) {
         input_ready_->record(stream.raw());
         input_ready_->wait(branch_stream_->raw());
-        run_shared(workspace, input, *branch_stream_);
+        if (quantized) run_shared_quantized(quantized->codes, quantized->scales, *branch_stream_);              // :1058-1064
+        else run_shared(workspace, input, *branch_stream_);
         output_ready_->record(branch_stream_->raw());
     }
     const std::optional<RouteOperands> route = router_.run_routed(input, input_len, tokens, fused, stream, options_.gate_front);
     const auto deferred = workspace.run_live_for_ffn(expert_, input, input_len, router_.ids(), router_.routing(), tokens.active_rows(),
                                                      options_.sum_shared, route, stream);
     if (branch) output_ready_->wait(stream.raw());
+    else if (quantized) run_shared_quantized(quantized->codes, quantized->scales, stream);
     else run_shared(workspace, 0, stream);
     if (deferred) sum_shared(workspace, deferred->second, stream);
     else add_shared(workspace, stream);

@@ -214,7 +214,15 @@ public:
                                     // (one queue, no cross-stream join); takes precedence over `overlap`
     };
     LayerFfn(std::shared_ptr<const Native> native, std::shared_ptr<Weights> weights, Prepared layout, size_t rows, Options options);
-    void run(Workspace& workspace, uint64_t input, size_t input_len, const TokenRows& tokens, const Stream& stream);
+    void run(Workspace& workspace, uint64_t input, size_t input_len, const TokenRows& tokens, const Stream& stream) {
+        run_quantized_input(workspace, input, input_len, nullptr, tokens, stream);                             // src/ffn.rs:965-973
+    }
+    // run_quantized_input (:974-1047): `quantized` (may be null) = E4M3 codes and UE8M0 scales of the same rows in the shared
+    // expert's quantizer flavour (amax floored at 1e-4), produced upstream with the normalized input; the shared expert then
+    // consumes them instead of quantizing the BF16 rows again.
+    struct QuantizedInput { uint64_t codes, scales; };
+    void run_quantized_input(Workspace& workspace, uint64_t input, size_t input_len, const QuantizedInput* quantized, const TokenRows& tokens,
+                             const Stream& stream);
     const Buffer<uint16_t>& output() const { return output_; }
     Router& router() { return router_; }
     const Buffer<uint16_t>& shared_up() const { return shared_up_; }
@@ -227,6 +235,8 @@ public:
     size_t rows() const { return rows_; }
     // input != 0: quantize it first (the branch's own quantizer); 0: use the codes the front-end left in the workspace.
     void run_shared(const Workspace& workspace, uint64_t input, const Stream& stream);
+    // the shared expert from given codes / scales (Linear::run_quantized, src/fp8_linear.rs:792-806)
+    void run_shared_quantized(uint64_t codes, uint64_t scales, const Stream& stream);
     void sum_shared(const Workspace& workspace, size_t live_rows, const Stream& stream);
 private:
     void add_shared(const Workspace& workspace, const Stream& stream);
