@@ -12,8 +12,10 @@ pytestmark = pytest.mark.gpu
 host = pkg.host
 
 
-def run_case(rows, hidden, experts, topk, inter, shared, mode, live=None, padding=None, tokens=None, **options):
+def run_case(rows, hidden, experts, topk, inter, shared, mode, live=None, padding=None, tokens=None, alt_token=None, **options):
     g = geometry(hidden, experts, topk, inter, shared, mode)
+    if alt_token is not None:
+        g.alt_token = alt_token
     name = "shape-%d-%d-%d-%d-%d-%d" % (rows, hidden, experts, topk, inter, shared)
     ops = synth.LayerOperands(g, name, device="cuda")
     x = synth.activations(name, rows, hidden)
@@ -54,3 +56,12 @@ def test_many_rows_with_a_live_prefix_and_padding_rows():
     taps, _ = run_case(rows, 1024, 16, 2, 512, 512, "benchmark", live=152, padding=padding, route_front=False)
     assert np.array_equal(taps["ids"][150], taps["ids"][3]) and np.array_equal(taps["ids"][151], taps["ids"][7])
     assert not taps["weights"][150:152].any() and (taps["ids"][152:] == -1).all()
+
+
+def test_drafter_parameter_set():
+    # the reference's drafter layers: 128 experts, top-3, no image-token bias (src/layer_id.rs:39-47): a row whose token id is
+    # the main model's image token must be routed with the ordinary bias
+    tokens = [129264, 1, 2, 3, 4, 5]
+    taps, _ = run_case(6, 1024, 128, 3, 512, 512, "reference", tokens=tokens, alt_token=-1)
+    again, _ = run_case(6, 1024, 128, 3, 512, 512, "reference", tokens=[7, 1, 2, 3, 4, 5], alt_token=-1)
+    assert np.array_equal(taps["ids"], again["ids"]) and np.array_equal(taps["out"], again["out"])
