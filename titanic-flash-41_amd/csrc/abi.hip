@@ -132,7 +132,7 @@ int launch_dynamic(const Context& c, bool route, const uint64_t* p, const int32_
             // with the gate weight (and a zeroed sync word) the gate product runs inside this launch too (owner rows <= 64)
             const bool gate = p[P_GATE_W] != 0;
             if (gate && (!p[P_SYNC] || owner > TF_STREAM_MAX_ROWS || g.hidden > 8192)) return -1;
-            const int logit_blocks = gate ? (g.experts * ((owner + 3) / 4) + 7) / 8 : 0;       // eight waves a block, one (expert, four rows) a wave
+            const int logit_blocks = gate ? ((owner + 3) / 4) * ((g.experts + 7) / 8) : 0;     // per group of four rows: eight waves a block, one expert a wave
             ca_moe_route_frontend<<<quant_blocks + 1 + logit_blocks, 512, 0, s>>>(
                 x, ids, weights, (uint8_t*)p[P_PACKED], (uint8_t*)p[P_SCALES], (int32_t*)p[P_TOKEN_MAP], (float*)p[P_TOKEN_WEIGHTS],
                 (int32_t*)p[P_TASK_EXPERT], (int32_t*)p[P_TASK_VALID], (int32_t*)p[P_TILE_BASE], (float*)p[P_LOGITS],
@@ -479,7 +479,7 @@ int64_t ca_primitives_scratch_bytes(void* context, int32_t index, int32_t rows) 
     add(tiles * 4); add(tiles * 4); add((g.experts + 1) * 4ll); add(padded * 4); add(padded * 4);
     add(pairs * H * 2);
     add(((pairs + 63) / 64 * g.experts + pairs) * 4);
-    add(1024);
+    add(4096);
     return bytes;
 }
 

@@ -140,8 +140,9 @@ extern "C" __global__ void __launch_bounds__(512) ca_moe_frontend(
 // The front-end with the router's top-k inside: block 0 first routes every owner row from the gate's logits (and
 // applies padding routes), then plans; the other blocks quantize meanwhile (launch one block more).
 // With `gate_w` the gate product runs here too: `logit_blocks` further blocks (one wave per expert and four rows) compute the logits,
-// publish them and count themselves in at `sync` (eight words, 128 bytes apart: 1 KiB); block 0 waits for the counts, bounded: if the count does not arrive it
-// computes the logits itself, so the kernel always ends.  All blocks of this small grid are resident together.
+// publish them and count themselves in at `sync` (seventeen words, 128 bytes apart, zero before the first launch); block 0
+// waits for the counts, bounded: if they do not arrive it computes the logits itself, so the kernel always ends.  All blocks
+// of this small grid are resident together.
 extern "C" __global__ void __launch_bounds__(512) ca_moe_route_frontend(
     const uint16_t* input, int32_t* ids, float* weights, uint8_t* packed, uint8_t* scales, int32_t* token_map,
     float* token_weights, int32_t* task_expert, int32_t* task_valid_rows, int32_t* expert_tile_base,
@@ -153,44 +154,82 @@ extern "C" __global__ void __launch_bounds__(512) ca_moe_route_frontend(
     __shared__ float s_weights[1024];
     const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6, waves = blockDim.x >> 6;
     const int first_logit_block = (int)gridDim.x - logit_blocks;
+    const RouteParams p{experts, topk, scoring, route_scale, alt_token};
+    // Logit blocks are group-major: block lb works on row group lb / per_group (four rows), experts 8 (lb % per_group) ..
+    // More than two row groups: the last block of a group to finish routes the group's rows itself (one routing round for
+    // the whole owner instead of one per eight rows in block 0) and block 0 only collects, applies padding and plans.
+    const int row_groups = (owner_rows + 3) >> 2, per_group = (experts + waves - 1) / waves;
+    const bool distributed = gate_w != nullptr && row_groups > 2;
+    uint32_t* routed_groups = sync + 32 * 16;            // arrival words: 128 bytes apart; [0, 16) per row group or per lb % 8, [16] routed groups
     if (gate_w != nullptr && (int)blockIdx.x >= first_logit_block) {
-        // one wave per (expert, group of four rows): every product of the launch runs in parallel
-        const int groups = (owner_rows + 3) >> 2, task = ((int)blockIdx.x - first_logit_block) * waves + wave;
-        const int e = task / groups, first_row = 4 * (task - e * groups);
-        if (e < experts)
+        const int lb = (int)blockIdx.x - first_logit_block, group = lb / per_group, e = (lb - group * per_group) * waves + wave;
+        const int first_row = 4 * group;
+        if (e < experts && first_row < owner_rows)
             tf_logits_expert(input + (size_t)first_row * cols, gate_w, logits + (size_t)first_row * experts, min(4, owner_rows - first_row), cols,
                              experts, e, lane);
         tf_stores_done();
         __syncthreads();
-        // arrivals are spread over eight words, one cache line apart: atomics on one address serialize
-        const int lb = (int)blockIdx.x - first_logit_block;
-        if (threadIdx.x == 0) atomicAdd(sync + 32 * (lb & 7), 1u);
+        if (!distributed) {
+            // arrivals are spread over eight words: atomics on one address serialize
+            if (threadIdx.x == 0) atomicAdd(sync + 32 * (lb & 7), 1u);
+            return;
+        }
+        __shared__ int last;
+        if (threadIdx.x == 0) {
+            last = atomicAdd(sync + 32 * group, 1u) == (uint32_t)(per_group - 1);
+            if (last) __hip_atomic_store(sync + 32 * group, 0u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);     // for the next launch
+        }
+        __syncthreads();
+        if (!last) return;
+        tf_route_block(logits, bias, bias_alt, tokens, live, nullptr, ids, weights, min(owner_rows, first_row + 4), p, first_row, waves, false,
+                       nullptr, nullptr, true);
+        tf_stores_done();
+        __syncthreads();
+        if (threadIdx.x == 0) atomicAdd(routed_groups, 1u);
         return;
     }
     if (blockIdx.x == 0) {
+        bool routed = false;
         if (gate_w != nullptr) {
             __shared__ int arrived;
-            if (threadIdx.x < 64) {      // lanes 0 .. 7 of the first wave watch one arrival word each
-                const int word = lane & 7;
-                const uint32_t expected = (uint32_t)((logit_blocks - word + 7) >> 3);        // logit blocks lb with lb % 8 == word
+            if (threadIdx.x < 64) {
                 int ok = 0;
-                for (int spin = 0; spin < (1 << 18); ++spin) {
-                    const bool here = __hip_atomic_load(sync + 32 * word, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT) >= expected;
-                    if (__all(here)) { ok = 1; break; }
-                    __builtin_amdgcn_s_sleep(2);
+                if (distributed) {
+                    for (int spin = 0; spin < (1 << 18); ++spin) {
+                        if (__hip_atomic_load(routed_groups, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT) >= (uint32_t)row_groups) { ok = 1; break; }
+                        __builtin_amdgcn_s_sleep(2);
+                    }
+                    if (lane == 0) __hip_atomic_store(routed_groups, 0u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+                } else {                 // lanes 0 .. 7 of the first wave watch one arrival word each
+                    const int word = lane & 7;
+                    const uint32_t expected = (uint32_t)((logit_blocks - word + 7) >> 3);        // logit blocks lb with lb % 8 == word
+                    for (int spin = 0; spin < (1 << 18); ++spin) {
+                        const bool here = __hip_atomic_load(sync + 32 * word, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT) >= expected;
+                        if (__all(here)) { ok = 1; break; }
+                        __builtin_amdgcn_s_sleep(2);
+                    }
+                    if (lane < 8) __hip_atomic_store(sync + 32 * word, 0u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
                 }
-                if (lane < 8) __hip_atomic_store(sync + 32 * word, 0u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
                 if (lane == 0) arrived = ok;
             }
             __syncthreads();
-            if (!arrived)
+            if (!arrived)                // the bound expired: this block forms the logits (and routes) itself, so the kernel always ends
                 for (int e = wave; e < experts; e += waves) tf_logits_expert(input, gate_w, logits, owner_rows, cols, experts, e, lane);
             tf_stores_done();
             __syncthreads();
+            if (arrived && distributed) {
+                // collect the groups' routes (written by other workgroups of this launch), then padding rows
+                for (int i = threadIdx.x; i < owner_rows * topk; i += blockDim.x) {
+                    s_ids[i] = (int32_t)__hip_atomic_load(reinterpret_cast<const uint32_t*>(ids) + i, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+                    s_weights[i] = tf_acquire_f32(weights + i);
+                }
+                __syncthreads();
+                tf_apply_padding(padding, ids, weights, owner_rows, topk, s_ids, s_weights);
+                routed = true;
+            }
         }
-        const RouteParams p{experts, topk, scoring, route_scale, alt_token};
-        tf_route_block(logits, bias, bias_alt, tokens, live, padding, ids, weights, owner_rows, p, 0,
-                       blockDim.x >> 6, true, s_ids, s_weights);
+        if (!routed)
+            tf_route_block(logits, bias, bias_alt, tokens, live, padding, ids, weights, owner_rows, p, 0, waves, true, s_ids, s_weights);
     }
     if ((int)blockIdx.x >= first_logit_block) return;
     // quantizer blocks are blocks [1, first_logit_block)

@@ -112,13 +112,30 @@ __device__ __forceinline__ void tf_route_row(const float* logits, const float* b
     for (int k = 0; k < 8; ++k) if (k < p.topk) out_weights[k] = __fmul_rn(w[k] / total, p.route_scale);
 }
 
+// Padding rows of a batched step take their source row's experts with zero weights; by one block, after the rows' routes
+// are complete (in `ids` / `weights`, and in the LDS copy when there is one).  Ends with a block barrier.
+__device__ __forceinline__ void tf_apply_padding(const int32_t* padding, int32_t* ids, float* weights, int rows, int topk, int32_t* s_ids,
+                                                 float* s_weights) {
+    if (padding != nullptr)
+        for (int i = threadIdx.x; i < rows * topk; i += blockDim.x) {
+            const int r = i / topk, s = padding[r];
+            if (s >= 0) {
+                const int32_t from = s_ids != nullptr ? s_ids[s * topk + (i - r * topk)] : ids[s * topk + (i - r * topk)];
+                ids[i] = from;
+                weights[i] = 0.f;
+                if (s_ids != nullptr) { s_ids[i] = from; s_weights[i] = 0.f; }
+            }
+        }
+    __syncthreads();
+}
+
 // Routes rows [first_row, first_row + waves of this block) of `rows`; rows at or past min(rows, live[0]) get ids -1 and
 // weights 0.  `padding` (may be null) is applied only by a single-block launch, after a block barrier.
 __device__ __forceinline__ void tf_route_block(const float* logits, const float* bias, const float* bias_alt,
                                                const long long* tokens, const int32_t* live, const int32_t* padding,
                                                int32_t* ids, float* weights, int rows, const RouteParams& p,
                                                int first_row, int row_stride, bool apply_padding, int32_t* s_ids = nullptr,
-                                               float* s_weights = nullptr) {
+                                               float* s_weights = nullptr, bool publish = false) {
     const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
     const int n_live = min(rows, live[0]);
     for (int row = first_row + wave; row < rows; row += row_stride) {
@@ -132,8 +149,13 @@ __device__ __forceinline__ void tf_route_block(const float* logits, const float*
 #pragma unroll
         for (int k = 0; k < 8; ++k)
             if (k < p.topk && lane == k) {
-                ids[row * p.topk + k] = is_live ? chosen[k] : -1;
-                weights[row * p.topk + k] = is_live ? share[k] : 0.f;
+                if (publish) {      // read next by another workgroup of the same launch
+                    tf_publish_u32(reinterpret_cast<uint32_t*>(ids) + row * p.topk + k, (uint32_t)(is_live ? chosen[k] : -1));
+                    tf_publish_f32(weights + row * p.topk + k, is_live ? share[k] : 0.f);
+                } else {
+                    ids[row * p.topk + k] = is_live ? chosen[k] : -1;
+                    weights[row * p.topk + k] = is_live ? share[k] : 0.f;
+                }
                 if (s_ids != nullptr) {      // a copy in LDS for the plan that follows in the same block
                     s_ids[row * p.topk + k] = is_live ? chosen[k] : -1;
                     s_weights[row * p.topk + k] = is_live ? share[k] : 0.f;
@@ -143,17 +165,7 @@ __device__ __forceinline__ void tf_route_block(const float* logits, const float*
     if (apply_padding) {
         __threadfence_block();
         __syncthreads();
-        if (padding != nullptr)
-            for (int i = threadIdx.x; i < rows * p.topk; i += blockDim.x) {
-                const int r = i / p.topk, s = padding[r];
-                if (s >= 0) {
-                    const int32_t from = s_ids != nullptr ? s_ids[s * p.topk + (i - r * p.topk)] : ids[s * p.topk + (i - r * p.topk)];
-                    ids[i] = from;
-                    weights[i] = 0.f;
-                    if (s_ids != nullptr) { s_ids[i] = from; s_weights[i] = 0.f; }
-                }
-            }
-        __syncthreads();
+        tf_apply_padding(padding, ids, weights, rows, p.topk, s_ids, s_weights);
     }
 }
 
