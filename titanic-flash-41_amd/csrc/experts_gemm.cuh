@@ -8,7 +8,7 @@
 //        registers;
 //   FC2 / dense: 256 output columns; routed rows are scaled by their routing weight and scattered to route order.
 // The E4M3 token tile goes through LDS (double-buffered, stored in matrix-instruction fragment order so every wave reads
-// 1 KiB contiguous, conflict-free, per fragment); the prepared weights go from global memory straight into the B operand
+// 1 KiB contiguous, conflict-free, per fragment; its scales are staged once a tile); the prepared weights go from global memory straight into the B operand
 // (1 KiB contiguous per weight tile and k-step) through a ring of register sets, three k-steps ahead of their use.
 // Workgroups are persistent and XCD-aware: workgroup b runs on XCD b % 8 and only ever touches 1/8 of the column groups,
 // so every XCD's L2 holds its own slices of the expert's weights while the expert's tiles pass by; partially filled
@@ -23,6 +23,8 @@
 
 #define TF_STREAM_MAX_ROWS 64
 #define TF_GEMM_TILE_M 128
+#define TF_GEMM_MAX_SCALES_ROW 128                 // activation scales a row the tile table holds: k / act_block
+#define TF_GEMM_SCALE_WORDS 8                       // words of that table a thread moves: 128 rows x 128 bytes / 512 threads / 4
 
 struct GemmArgs {
     const uint8_t* a_codes;          // E4M3 [rows][k]: token rows (FC1), physical rows (routed FC2), dense rows
@@ -58,12 +60,15 @@ __global__ void __launch_bounds__(512) tf_gemm(const GemmArgs p) {
     constexpr bool ROUTED = MODE == TF_GEMM_FC1_ROUTED || MODE == TF_GEMM_FC2_ROUTED;
     constexpr int GROUP_COLS = FC1 ? 128 : 256;          // output columns a task covers
     __shared__ __attribute__((aligned(16))) uint8_t s_a[2][16384];     // [stage][m-frag 8][half 2][lane 64][16 B]
-    __shared__ uint32_t s_as[2][128];                                   // [stage][row]: scale bytes of the row's four K32 blocks
+    __shared__ __attribute__((aligned(16))) uint8_t s_scale[128 * (TF_GEMM_MAX_SCALES_ROW + 4)];    // [row][k-block]: the tile's activation scales; the row stride is an odd number of words
     __shared__ float s_amax[4][128];
     __shared__ long long s_row[128];                                    // source row of each tile row
     // eight waves: row half mh (64 rows = four 16-row fragments) x column quarter nq (64 weight rows = four 16-row tiles)
-    const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6, mh = wave >> 2, nq = wave & 3, g = lane >> 4, r16 = lane & 15;
+    // the wave's index as a scalar: everything derived from it (weight tile addresses, LDS fragment offsets) stays out of the vector registers
+    const int tid = threadIdx.x, lane = tid & 63, wave = __builtin_amdgcn_readfirstlane(tid >> 6), mh = wave >> 2, nq = wave & 3, g = lane >> 4, r16 = lane & 15;
     const int ksteps = p.k / 128;
+    const int scales_row = p.k / p.act_block, scale_words_row = scales_row / 4, scale_stride = scales_row + 4;
+    const int act_shift = p.act_block == 32 ? 5 : 7;
     const int n_cols = FC1 ? p.inter : p.hidden, groups = n_cols / GROUP_COLS;
     const int tiles = ROUTED ? p.expert_tile_base[p.experts] : (p.dense_rows + 127) / 128;
     const int xcd = blockIdx.x & 7, local = blockIdx.x >> 3, local_count = gridDim.x >> 3;
@@ -103,7 +108,6 @@ __global__ void __launch_bounds__(512) tf_gemm(const GemmArgs p) {
             a_src[i] = p.a_codes + s_row[row] * p.k + piece * 16;
             a_dst[i] = c * 16;
         }
-        const uint8_t* as_src = p.a_scales + s_row[tid & 127] * (p.k / p.act_block);
         // weight row tiles of this wave: FC1 routed: two "up" tiles then two "gate" tiles of the same 32 intermediate columns;
         // FC1 shared: gate tiles then up tiles; FC2 / dense: four tiles of 64 output columns
         int ntile[4];
@@ -112,17 +116,30 @@ __global__ void __launch_bounds__(512) tf_gemm(const GemmArgs p) {
             if (FC1) ntile[j] = (j >> 1) * (p.inter / 16) + (ng * 128 + nq * 32) / 16 + (j & 1);
             else ntile[j] = (ng * 256 + nq * 64) / 16 + j;
         }
-        auto load_a = [&](int ks, u4v (&ra)[2], uint32_t& rs) {
+        auto load_a = [&](int ks, u4v (&ra)[2]) {
 #pragma unroll
             for (int i = 0; i < 2; ++i) ra[i] = *reinterpret_cast<const u4v*>(a_src[i] + (size_t)ks * 128);
-            // the raw scale bytes only: arithmetic on a value just requested would make this a wait for every load in flight
-            if (p.act_block == 32) rs = *reinterpret_cast<const uint32_t*>(as_src + ks * 4);
-            else rs = as_src[ks];
         };
-        auto store_a = [&](int stage, const u4v (&ra)[2], uint32_t rs) {
+        auto store_a = [&](int stage, const u4v (&ra)[2]) {
 #pragma unroll
             for (int i = 0; i < 2; ++i) *reinterpret_cast<u4v*>(&s_a[stage][a_dst[i]]) = ra[i];
-            if (tid < 128) s_as[stage][tid] = p.act_block == 32 ? rs : 0x01010101u * rs;      // one byte per K32 block of the k-step
+        };
+        // The rows' activation scales of every k-step go to LDS once a tile (a byte a row and k-step fetched inside the main
+        // loop costs a cache line request per row: as many requests as the tile's codes need).  Requested first, stored after
+        // the main loop's first operand requests are out.
+        uint32_t scale_regs[TF_GEMM_SCALE_WORDS];
+#pragma unroll
+        for (int i = 0; i < TF_GEMM_SCALE_WORDS; ++i) {
+            const int c = min(tid + 512 * i, 128 * scale_words_row - 1);            // word c % per_row of row c / per_row
+            scale_regs[i] = *reinterpret_cast<const uint32_t*>(p.a_scales + s_row[c / scale_words_row] * scales_row + (c % scale_words_row) * 4);
+        }
+        auto store_scales = [&]() {
+#pragma unroll
+            for (int i = 0; i < TF_GEMM_SCALE_WORDS; ++i) {
+                const int c = tid + 512 * i;
+                if (c < 128 * scale_words_row)
+                    *reinterpret_cast<uint32_t*>(&s_scale[(c / scale_words_row) * scale_stride + (c % scale_words_row) * 4]) = scale_regs[i];
+            }
         };
         // B operand of one k-step: plain loads (an expert's weight slice is re-read by the expert's other tiles from this
         // XCD's L2).  FP8: with the lane's block scale of the k-step; FP4: scales come a word per four k-steps (load_b_scales).
@@ -160,14 +177,14 @@ __global__ void __launch_bounds__(512) tf_gemm(const GemmArgs p) {
             constexpr int FR = decltype(fr_constant)::value;
             constexpr int D = FP8 ? 2 : 4;         // ksteps % 4 == 0
             u4v ra[D][2];
-            uint32_t rs[D];
             BFrag<FP8> b[D][4];
             uint32_t sbk[D][4];                  // FP8: the slot's scale bytes
             uint32_t sb[4] = {0, 0, 0, 0}, sb_next[4] = {0, 0, 0, 0};   // FP4: scale words of the current / next four k-steps
 #pragma unroll
-            for (int d = 0; d < D - 1; ++d) { load_a(d, ra[d], rs[d]); load_b(d, b[d], sbk[d]); }
+            for (int d = 0; d < D - 1; ++d) { load_a(d, ra[d]); load_b(d, b[d], sbk[d]); }
             if constexpr (!FP8) load_b_scales(0, sb);
-            store_a(0, ra[0], rs[0]);
+            store_scales();
+            store_a(0, ra[0]);
             __syncthreads();
             for (int ks0 = 0; ks0 < ksteps; ks0 += D) {
 #pragma unroll
@@ -178,7 +195,7 @@ __global__ void __launch_bounds__(512) tf_gemm(const GemmArgs p) {
                         // nothing): the compiler counts outstanding loads statically, and a load that may or may not have been
                         // issued turns every wait behind it into a wait for all loads in flight.
                         const int stage = ks & 1, ahead = min(ks + D - 1, ksteps - 1);
-                        load_a(ahead, ra[(u + D - 1) % D], rs[(u + D - 1) % D]);
+                        load_a(ahead, ra[(u + D - 1) % D]);
                         load_b(ahead, b[(u + D - 1) % D], sbk[(u + D - 1) % D]);
                         if constexpr (!FP8) { if (u == 1) load_b_scales(ahead, sb_next); }           // ahead % 4 == 0 (D == 4)
                         if constexpr (!FP8) {
@@ -187,22 +204,31 @@ __global__ void __launch_bounds__(512) tf_gemm(const GemmArgs p) {
                                 for (int j = 0; j < 4; ++j) sb[j] = sb_next[j];
                             }
                         }
+                        // the next fragment's rows leave LDS while the current fragment's products run: two register sets
+                        v8i av[2];
+                        int sa[FR > 0 ? FR : 1];
 #pragma unroll
-                        for (int f = 0; f < FR; ++f) {
+                        for (int f = 0; f < FR; ++f) sa[f] = s_scale[((4 * mh + f) * 16 + r16) * scale_stride + ((ks * 128 + 32 * g) >> act_shift)];
+                        auto read_frag = [&](int f, v8i& a) {
                             const int tf = 4 * mh + f;             // fragment of the tile
                             const u4v lo = *reinterpret_cast<const u4v*>(&s_a[stage][((tf * 2) * 64 + lane) * 16]);
                             const u4v hi = *reinterpret_cast<const u4v*>(&s_a[stage][((tf * 2 + 1) * 64 + lane) * 16]);
-                            const v8i av = v8i{(int)lo[0], (int)lo[1], (int)lo[2], (int)lo[3], (int)hi[0], (int)hi[1], (int)hi[2], (int)hi[3]};
-                            const int sa = (int)((s_as[stage][tf * 16 + r16] >> (8 * g)) & 0xffu);
+                            a = v8i{(int)lo[0], (int)lo[1], (int)lo[2], (int)lo[3], (int)hi[0], (int)hi[1], (int)hi[2], (int)hi[3]};
+                        };
+                        if constexpr (FR > 0) read_frag(0, av[0]);
+#pragma unroll
+                        for (int f = 0; f < FR; ++f) {
+                            if (f + 1 < FR) read_frag(f + 1, av[(f + 1) & 1]);
+                            const v8i a_now = av[f & 1];
 #pragma unroll
                             for (int j = 0; j < 4; ++j) {
                                 const BFrag<FP8>& bj = b[u][j];
                                 if constexpr (FP8) {
                                     const v8i bv = v8i{(int)bj.lo[0], (int)bj.lo[1], (int)bj.lo[2], (int)bj.lo[3], (int)bj.hi[0], (int)bj.hi[1], (int)bj.hi[2], (int)bj.hi[3]};
-                                    acc[f][j] = __builtin_amdgcn_mfma_scale_f32_16x16x128_f8f6f4(av, bv, acc[f][j], 0, 0, 0, sa, 0, (int)sbk[u][j]);
+                                    acc[f][j] = __builtin_amdgcn_mfma_scale_f32_16x16x128_f8f6f4(a_now, bv, acc[f][j], 0, 0, 0, sa[f], 0, (int)sbk[u][j]);
                                 } else {
                                     const v8i bv = v8i{(int)bj.lo[0], (int)bj.lo[1], (int)bj.lo[2], (int)bj.lo[3], 0, 0, 0, 0};
-                                    acc[f][j] = __builtin_amdgcn_mfma_scale_f32_16x16x128_f8f6f4(av, bv, acc[f][j], 0, 4, 0, sa, 0, (int)(sb[j] >> (8 * u)));
+                                    acc[f][j] = __builtin_amdgcn_mfma_scale_f32_16x16x128_f8f6f4(a_now, bv, acc[f][j], 0, 4, 0, sa[f], 0, (int)(sb[j] >> (8 * u)));
                                 }
                             }
                             // a use the optimizer cannot move: without it every product of the unrolled k-steps is sunk below the
@@ -210,7 +236,16 @@ __global__ void __launch_bounds__(512) tf_gemm(const GemmArgs p) {
 #pragma unroll
                             for (int j = 0; j < 4; ++j) asm volatile("" :: "v"(acc[f][j]));
                         }
-                        store_a(stage ^ 1, ra[(u + 1) % D], rs[(u + 1) % D]);
+                        // issue order of the k-step: fragment f + 1's LDS reads go out before fragment f's four products
+                        if constexpr (FR > 0) {
+                            __builtin_amdgcn_sched_group_barrier(0x100, FR + 2, 0);
+#pragma unroll
+                            for (int f = 0; f < FR; ++f) {
+                                if (f + 1 < FR) __builtin_amdgcn_sched_group_barrier(0x100, 2, 0);
+                                __builtin_amdgcn_sched_group_barrier(0x008, 4, 0);
+                            }
+                        }
+                        store_a(stage ^ 1, ra[(u + 1) % D]);
                         __syncthreads();
                     }
                 }
@@ -324,7 +359,7 @@ __global__ void __launch_bounds__(512) tf_gemm(const GemmArgs p) {
 
 inline int tf_gemm_grid(int cus) { return cus >= 8 ? cus / 8 * 8 : 8; }
 inline bool tf_gemm_shape_ok(const GemmArgs& a, bool fc1) {
-    return a.k >= 512 && a.k % 512 == 0 && (a.act_block == 32 || a.act_block == 128) &&
+    return a.k >= 512 && a.k % 512 == 0 && (a.act_block == 32 || a.act_block == 128) && a.k / a.act_block <= TF_GEMM_MAX_SCALES_ROW &&
            (fc1 ? (a.inter >= 128 && a.inter % 128 == 0) : (a.hidden >= 256 && a.hidden % 256 == 0));
 }
 inline int tf_launch_fc1_gemm(const GemmArgs& a, int cus, hipStream_t s) {
