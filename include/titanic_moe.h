@@ -60,6 +60,20 @@ const char* ca_kernel_name(int index);
 /* kernels/moe_nibble_layout_probe.cu:17-21 */
 int ca_moe_nibble_permute(void* data, uint64_t bytes, int inverse, void* stream);
 
+/* ---- libcanada_moe_input_codec.so surface: the wire row "dual_quant_rows_v1" of the sequence-parallel prefill ------
+ * (runtime/kernels/moe-input-codec-coalesced-v1/moe-dual-quant-codec-fast.cu).  A row of k values is k routed E4M3 codes,
+ * k / 32 UE8M0 scale bytes and k / 32 32-bit correction words: k * 37 / 32 bytes.  All pointers are device pointers, every
+ * call only enqueues on `stream`; 0, -1 for an argument out of range (the reference's own checks), or a hipError_t. */
+/* :81-87.  routed[rows][k], scales[rows][k/32] (routed quantizer), shared[rows][k] (shared quantizer's codes) -> packed. */
+int ca_encode(const uint8_t* routed, const uint8_t* scales, const uint8_t* shared, uint8_t* packed, int rows, int k, void* stream);
+/* :88-94.  packed -> shared[rows][k], row_scales[rows][k/32] and the same scale bytes at the reference's matrix-instruction
+ * offsets in mma_scales (rows * k / 32 bytes; additive: may be null).  rows % 128 == 0. */
+int ca_decode(const uint8_t* packed, uint8_t* shared, uint8_t* row_scales, uint8_t* mma_scales, int rows, int k, void* stream);
+/* :99-105.  *local = min(rows, max(0, *global - rank * rows)), rank 0..3. */
+int ca_local_live(const int* global, int* local, int rows, int rank, void* stream);
+/* :138-144.  input[rows][k] (bf16) -> packed: both quantizers and the encoder in one pass. */
+int ca_pack_bf16(const void* input, uint8_t* packed, int rows, int k, void* stream);
+
 /* ---- operator ABI (src/primitives.rs:45-60, 91-182; bridge.cc) ------------------------------------------------- */
 int32_t ca_primitives_abi(void);                /* returns 1 */
 void* ca_primitives_open(int32_t* status);      /* host handle; snapshots the process geometry and the device's CU count */

@@ -349,3 +349,39 @@ def scale_codes4_decode(coded, matrices, n, columns):
     out = np.zeros(matrices * n * columns, np.uint8)
     lib().orc_scale_codes4_decode(_p(coded), _p(out), _i32(matrices), _i32(n), _i32(columns))
     return out
+
+
+def codec_row_bytes(k):
+    return k + (k // 32) * 5
+
+
+def codec_encode(routed, routed_scales, shared):
+    routed, routed_scales, shared = _c(routed, np.uint8), _c(routed_scales, np.uint8), _c(shared, np.uint8)
+    rows, k = routed.shape
+    packed = np.zeros((rows, codec_row_bytes(k)), np.uint8)
+    lib().orc_codec_encode(_p(routed), _p(routed_scales), _p(shared), _p(packed), _i32(rows), _i32(k))
+    return packed
+
+
+def codec_decode(packed, k, mma=False):
+    packed = _c(packed, np.uint8)
+    rows = packed.shape[0]
+    shared = np.empty((rows, k), np.uint8)
+    row_scales = np.empty((rows, k // 32), np.uint8)
+    mma_scales = np.zeros(rows * (k // 32), np.uint8) if mma else None
+    lib().orc_codec_decode(_p(packed), _p(shared), _p(row_scales), _p(mma_scales), _i32(rows), _i32(k))
+    return (shared, row_scales, mma_scales) if mma else (shared, row_scales)
+
+
+def codec_pack_bf16(x):
+    x = _c(x, np.uint16)
+    rows, k = x.shape
+    packed = np.zeros((rows, codec_row_bytes(k)), np.uint8)
+    lib().orc_codec_pack_bf16(_p(x), _p(packed), _i32(rows), _i32(k))
+    return packed
+
+
+def codec_local_live(global_live, rows, rank):
+    f = lib().orc_codec_local_live
+    f.restype = ctypes.c_int32
+    return int(f(_i32(global_live), _i32(rows), _i32(rank)))

@@ -74,6 +74,12 @@ void orc_quantize_rows(const uint16_t* x, int32_t rows, int32_t cols, int32_t bl
                        uint8_t* codes, uint8_t* scales);
 
 /* ---- shared expert ------------------------------------------------------------------------- */
+void orc_codec_encode(const uint8_t* routed, const uint8_t* routed_scales, const uint8_t* shared, uint8_t* packed,
+                      int32_t rows, int32_t k);
+void orc_codec_decode(const uint8_t* packed, uint8_t* shared, uint8_t* row_scales, uint8_t* mma_scales, int32_t rows,
+                      int32_t k);
+void orc_codec_pack_bf16(const uint16_t* input, uint8_t* packed, int32_t rows, int32_t k);
+int32_t orc_codec_local_live(int32_t global, int32_t rows, int32_t rank);
 void orc_shared_swiglu(const uint16_t* in, uint16_t* act, int32_t rows, int32_t inter, float limit);
 void orc_shared_swiglu_quant(const uint16_t* in, uint16_t* act, uint8_t* codes, uint8_t* scales, int32_t rows,
                              int32_t inter, int32_t block, float limit);

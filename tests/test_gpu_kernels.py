@@ -88,7 +88,8 @@ def test_wide_plan_bit_exact(rows, experts, topk, tile_m):
     tmap = torch.full((max_tiles * tile_m,), -1, dtype=torch.int32, device="cuda")
     tw = torch.zeros(max_tiles * tile_m, dtype=torch.float32, device="cuda")
     native.launch("ca_plan_wave_counts", (waves + 3) // 4, 256, [d_ids, pairs, experts, wave_counts, local_rank])
-    native.launch("ca_plan_scan", 1, 512, [wave_counts, waves, experts, 1, tile_m, base, te, tv])
+    native.launch("ca_plan_scan", experts, 256, [wave_counts, waves, experts, base])
+    native.launch("ca_plan_tiles", 1, 512, [experts, 1, tile_m, base, te, tv])
     native.launch("ca_plan_scatter", (pairs + 255) // 256, 256, [d_ids, d_w, wave_counts, local_rank, base, pairs, experts, tile_m, tmap, tw])
     torch.cuda.synchronize()
     want = oracle.plan(ids, weights, experts, 1, tile_m, capacity_tiles=max_tiles)

@@ -36,6 +36,8 @@ ENTRIES = [
     ("kernel_007", "moe.w4a8.phase2", DYN_POINTERS, DYN_SCALARS),
     ("kernel_008", "moe.front_end", DYN_POINTERS, DYN_SCALARS),
     ("kernel_009", "ffn.experts_with_shared", DYN_POINTERS + ROUTE_POINTERS + SHARED_POINTERS, DYN_SCALARS + ["owner_rows"]),
+    # entry 0 with a_ptr holding wire rows "dual_quant_rows_v1" (the reference's packed contract: src/moe.rs:512-583)
+    ("kernel_010", "integration.tp_moe.dynamic", DYN_POINTERS, DYN_SCALARS),
 ]
 
 ROLE = {"a_ptr": "input", "topk_ids_ptr": "ids", "topk_weights_ptr": "routing_weights", "b_w13": "w13", "sfb_w13_ptr": "s13",

@@ -1,6 +1,7 @@
 // C ABI of libtitanic_moe_hip.so: the entry points the reference's Rust FFN operators bind (see include/titanic_moe.h).
 // Nothing here allocates, frees or synchronizes; every entry point only enqueues kernels on the caller's stream.
 #include "../../include/titanic_moe.h"
+#include "codec.cuh"
 #include "combine.cuh"
 #include "experts_gemm.cuh"
 #include "experts_stream.cuh"
@@ -98,8 +99,13 @@ void shared_stream_args(const Context& c, const uint64_t* p, int m, StreamArgs& 
 // `sum` (may be null, needs `sh`): {routed output, layer output} device pointers and the live row count: the ordered sum and the
 // shared addition run as well (inside the single streaming launch when the shapes allow it).
 struct SumArgs { uint64_t routed_out, output; int live; };
+int codec_blocks(const Context& c, long long rows, int k) {
+    const long long blocks = (rows * (k >> 3) + 255) / 256;
+    return (int)(blocks < (long long)c.cus * 16 ? blocks : (long long)c.cus * 16);
+}
+// `packed_input`: p[P_A] holds wire rows "dual_quant_rows_v1" (src/moe.rs:512-583) instead of BF16 rows.
 int launch_dynamic(const Context& c, bool route, const uint64_t* p, const int32_t* sc, hipStream_t s, int phases = 7, const uint64_t* sh = nullptr,
-                   const SumArgs* sum = nullptr) {
+                   const SumArgs* sum = nullptr, bool packed_input = false) {
     const ca_geometry& g = c.g;
     const int rows = sc[S_TOKENS], tile_m = sc[S_TILE_M], groups = sc[S_GROUPS], max_tiles = sc[S_MAX_TILES];
     if (rows < 1 || rows > sc[S_MAX_ROWS] || groups < 1 || max_tiles < 1 || sc[S_ROWS_PADDED] != max_tiles * tile_m) return -1;
@@ -109,6 +115,7 @@ int launch_dynamic(const Context& c, bool route, const uint64_t* p, const int32_
             !(i == P_INTER && rows > TF_STREAM_MAX_ROWS))
             return -1;
     if (!supported_k(g.hidden) || !supported_k(g.intermediate)) return -4;
+    if (packed_input && g.act_block != 32) return -4;      // the wire row carries 32-wide blocks
     const long long pairs = (long long)rows * g.topk;
     // capacity of the reference's contracts (max_phys_tiles): A = min(E, pairs) experts open a tile each and the other routes fill
     // at most floor((pairs - A) / tile_m) <= ceil(pairs / tile_m) - 1 more
@@ -123,7 +130,7 @@ int launch_dynamic(const Context& c, bool route, const uint64_t* p, const int32_
     int32_t* ids = (int32_t*)p[P_IDS];
     float* weights = (float*)p[P_WEIGHTS];
     if (!(phases & 1)) {
-    } else if (pairs <= 1024 && g.experts < 1024) {
+    } else if (pairs <= 1024 && g.experts < 1024 && !packed_input) {
         const int quant_blocks = (int)((((long long)rows * (g.hidden >> 3)) + 1023) / 1024);
         if (route) {
             const int owner = sc[S_OWNER_ROWS];
@@ -152,16 +159,17 @@ int launch_dynamic(const Context& c, bool route, const uint64_t* p, const int32_
         int32_t* wave_counts = (int32_t*)p[P_PLAN_SCRATCH];
         int32_t* local_rank = wave_counts + (size_t)waves * g.experts;
         ca_plan_wave_counts<<<(waves + 3) / 4, 256, 0, s>>>(ids, (int)pairs, g.experts, wave_counts, local_rank);
-        ca_plan_scan<<<1, 512, 0, s>>>(wave_counts, waves, g.experts, groups, tile_m, (int32_t*)p[P_TILE_BASE],
-                                       (int32_t*)p[P_TASK_EXPERT], (int32_t*)p[P_TASK_VALID]);
+        ca_plan_scan<<<g.experts, 256, 0, s>>>(wave_counts, waves, g.experts, (int32_t*)p[P_TILE_BASE]);
+        ca_plan_tiles<<<1, 512, 0, s>>>(g.experts, groups, tile_m, (int32_t*)p[P_TILE_BASE], (int32_t*)p[P_TASK_EXPERT], (int32_t*)p[P_TASK_VALID]);
         ca_plan_scatter<<<(int)((pairs + 255) / 256), 256, 0, s>>>(ids, weights, wave_counts, local_rank, (int32_t*)p[P_TILE_BASE],
                                                                     (int)pairs, g.experts, tile_m, (int32_t*)p[P_TOKEN_MAP],
                                                                     (float*)p[P_TOKEN_WEIGHTS]);
-        const long long items = (long long)rows * (g.hidden >> 3);
-        int blocks = (int)((items + 255) / 256);
-        if (blocks > c.cus * 16) blocks = c.cus * 16;
-        ca_quantize_rows<<<blocks, 256, 0, s>>>(x, (uint8_t*)p[P_PACKED], (uint8_t*)p[P_SCALES], (uint8_t*)p[P_PACKED_MIN],
-                                                (uint8_t*)p[P_SCALES_MIN], rows, g.hidden, g.act_block);
+        const int blocks = codec_blocks(c, rows, g.hidden);
+        if (packed_input)
+            ca_codec_unpack_routed<<<blocks, 256, 0, s>>>((const uint8_t*)p[P_A], (uint8_t*)p[P_PACKED], (uint8_t*)p[P_SCALES], rows, g.hidden);
+        else
+            ca_quantize_rows<<<blocks, 256, 0, s>>>(x, (uint8_t*)p[P_PACKED], (uint8_t*)p[P_SCALES], (uint8_t*)p[P_PACKED_MIN],
+                                                    (uint8_t*)p[P_SCALES_MIN], rows, g.hidden, g.act_block);
     }
     int status = launch_status();
     if (status) return status;
@@ -314,6 +322,7 @@ const EntryShape kEntries[] = {
     {"moe.w4a8.phase2", P_DYN_COUNT, S_DYN_COUNT},
     {"moe.front_end", P_DYN_COUNT, S_DYN_COUNT},
     {"ffn.experts_with_shared", P_ROUTE_COUNT + H_COUNT - 2 + 2, S_ROUTE_COUNT + 1},
+    {"integration.tp_moe.dynamic", P_DYN_COUNT, S_DYN_COUNT},      // input_format dual_quant_rows_v1
 };
 constexpr int kEntryCount = sizeof(kEntries) / sizeof(kEntries[0]);
 
@@ -322,12 +331,13 @@ struct KernelName { const char* name; const void* function; };
 const KernelName kKernels[] = {
     TF_KERNEL(ca_router_logits_rows), TF_KERNEL(ca_route_topk), TF_KERNEL(ca_route_padding_rows), TF_KERNEL(ca_route_census),
     TF_KERNEL(ca_moe_frontend), TF_KERNEL(ca_moe_route_frontend), TF_KERNEL(ca_quantize_rows), TF_KERNEL(ca_plan_wave_counts),
-    TF_KERNEL(ca_plan_scan), TF_KERNEL(ca_plan_scatter), TF_KERNEL(ca_shared_swiglu_rows), TF_KERNEL(ca_shared_swiglu_quant),
+    TF_KERNEL(ca_plan_scan), TF_KERNEL(ca_plan_tiles), TF_KERNEL(ca_plan_scatter), TF_KERNEL(ca_shared_swiglu_rows), TF_KERNEL(ca_shared_swiglu_quant),
     TF_KERNEL(ca_ffn_add_rows), TF_KERNEL(ca_moe_topk_sum), TF_KERNEL(ca_ffn_sum_shared), TF_KERNEL(ca_moe_group_sum_rows),
     TF_KERNEL(ca_expert_compact_words), TF_KERNEL(ca_expert_expand_words), TF_KERNEL(ca_expert_compact_scales),
     TF_KERNEL(ca_expert_expand_scales), TF_KERNEL(ca_dense_compact_fp8), TF_KERNEL(ca_moe_nibble_permute_words),
     TF_KERNEL(ca_expert_scale_code1), TF_KERNEL(ca_expert_scale_code1_check), TF_KERNEL(ca_expert_scale_code1_census),
-    TF_KERNEL(ca_expert_scale_codes4), TF_KERNEL(ca_router_logits_mfma),
+    TF_KERNEL(ca_expert_scale_codes4), TF_KERNEL(ca_router_logits_mfma), TF_KERNEL(ca_codec_encode), TF_KERNEL(ca_codec_decode),
+    TF_KERNEL(ca_codec_pack_bf16), TF_KERNEL(ca_codec_unpack_routed), TF_KERNEL(ca_codec_local_live),
 };
 constexpr int kKernelCount = sizeof(kKernels) / sizeof(kKernels[0]);
 
@@ -357,8 +367,9 @@ int ca_router_logits(int rows, const void* x, const void* w, void* out, void* st
 int ca_router_logits_wide(int rows, const void* x, const void* w, void* out, void* stream) {
     if (rows < 1 || !x || !w || !out) return -1;
     if (rows <= 16) return ca_router_logits(rows, x, w, out, stream);
-    const dim3 grid((rows + 63) / 64, (g_geometry.experts + 31) / 32);
-    ca_router_logits_mfma<<<grid, 256, 0, (hipStream_t)stream>>>((const uint16_t*)x, (const uint16_t*)w, (float*)out, rows,
+    if (g_geometry.hidden % 64) return -4;
+    const dim3 grid((rows + 127) / 128, (g_geometry.experts + 255) / 256);
+    ca_router_logits_mfma<<<grid, 512, 0, (hipStream_t)stream>>>((const uint16_t*)x, (const uint16_t*)w, (float*)out, rows,
                                                                  g_geometry.hidden, g_geometry.experts);
     return launch_status();
 }
@@ -379,6 +390,29 @@ int ca_ffn_add(int rows, const void* routed, const void* shared, void* out, void
 int ca_moe_nibble_permute(void* data, uint64_t bytes, int inverse, void* stream) {
     if (!data || bytes % 4 || (inverse != 0 && inverse != 1)) return -1;
     ca_moe_nibble_permute_words<<<256, 256, 0, (hipStream_t)stream>>>((uint32_t*)data, bytes / 4, inverse);
+    return launch_status();
+}
+
+// ---- row codec (runtime/kernels/moe-input-codec-coalesced-v1/moe-dual-quant-codec-fast.cu:81-94, 99-105, 138-144) ----
+namespace { int codec_grid(long long rows, int k) { const long long b = (rows * (k >> 3) + 255) / 256; return (int)(b < 4096 ? b : 4096); } }
+int ca_encode(const uint8_t* routed, const uint8_t* scales, const uint8_t* shared, uint8_t* packed, int rows, int k, void* stream) {
+    if (!routed || !scales || !shared || !packed || rows <= 0 || k <= 0 || k % 128) return -1;
+    ca_codec_encode<<<codec_grid(rows, k), 256, 0, (hipStream_t)stream>>>(routed, scales, shared, packed, rows, k);
+    return launch_status();
+}
+int ca_decode(const uint8_t* packed, uint8_t* shared, uint8_t* row_scales, uint8_t* mma_scales, int rows, int k, void* stream) {
+    if (!packed || !shared || !row_scales || rows <= 0 || rows % 128 || k <= 0 || k % 128) return -1;
+    ca_codec_decode<<<codec_grid(rows, k), 256, 0, (hipStream_t)stream>>>(packed, shared, row_scales, mma_scales, rows, k);
+    return launch_status();
+}
+int ca_local_live(const int* global, int* local, int rows, int rank, void* stream) {
+    if (!global || !local || rows <= 0 || rank < 0 || rank >= 4) return -1;
+    ca_codec_local_live<<<1, 64, 0, (hipStream_t)stream>>>(global, local, rows, rank);
+    return launch_status();
+}
+int ca_pack_bf16(const void* input, uint8_t* packed, int rows, int k, void* stream) {
+    if (!input || !packed || rows <= 0 || k <= 0 || k % 128) return -1;
+    ca_codec_pack_bf16<<<codec_grid(rows, k), 256, 0, (hipStream_t)stream>>>((const uint16_t*)input, packed, rows, k);
     return launch_status();
 }
 
@@ -451,6 +485,7 @@ int32_t ca_primitives_launch(void* context, int32_t index, const uint64_t* point
             const SumArgs sum{routed_out, output, scalars[S_ROUTE_COUNT]};
             return launch_dynamic(c, pointers[P_LOGITS] != 0, pointers, scalars, s, 7, sh, output ? &sum : nullptr);
         }
+        case 10: return launch_dynamic(c, false, pointers, scalars, s, 7, nullptr, nullptr, true);
         default: return -3;
     }
 }

@@ -384,38 +384,85 @@ inline int tf_launch_shared_fc1_gemm(const GemmArgs& a, int cus, hipStream_t s) 
 }
 
 // Gate product for many rows: logits[rows][experts] = x . w^T, BF16 inputs, FP32 accumulate on the matrix cores
-// (v_mfma_f32_32x32x16_bf16).  grid (ceil(rows / 64), ceil(experts / 32)), block 256: wave w takes row half w & 1 of the
-// block's 64 rows and half w >> 1 of K; the two K halves of a tile are added through LDS (first half + second half).
+// (v_mfma_f32_32x32x16_bf16).  grid (ceil(rows / 128), ceil(experts / 256)), block 512: a workgroup keeps a 128 x 256 tile
+// of logits (wave (mr, nq): rows 64 mr .., experts 64 nq ..: 2 x 2 accumulators of 32 x 32), so the rows are read from HBM
+// once and the gate weight (2 MB) from L2 once per 128 rows.  Both operands go through LDS, 64 columns of K a step, double
+// buffered, loaded as whole 128-byte row pieces (eight lanes a row) and stored in matrix-instruction fragment order: the
+// 16-byte piece kc of row r of a 32-row tile sits in block (tile, kc / 2), half kc % 2, slot (r + 2 kc) % 32; the rotation
+// by 2 kc keeps both the stores (two rows x eight pieces a phase) and the fragment reads free of bank conflicts.
 typedef __bf16 bf16x8 __attribute__((ext_vector_type(8)));
 typedef float v16f __attribute__((ext_vector_type(16)));
-extern "C" __global__ void __launch_bounds__(256) ca_router_logits_mfma(const uint16_t* x, const uint16_t* w, float* out, int rows,
+extern "C" __global__ void __launch_bounds__(512) ca_router_logits_mfma(const uint16_t* x, const uint16_t* w, float* out, int rows,
                                                                         int hidden, int experts) {
-    __shared__ float s_part[2][32 * 32];
-    const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6, half = wave & 1, kpart = wave >> 1;
-    const int row = blockIdx.x * 64 + half * 32 + (lane & 31), e = blockIdx.y * 32 + (lane & 31);
-    const int kg = lane >> 5;                                 // lane group: k = 8 kg .. 8 kg + 7 of each 16-wide step
-    v16f acc;
+    constexpr int X_TILES = 4, W_TILES = 8, STAGE = (X_TILES + W_TILES) * 4 * 1024;      // 32-row tiles; 4 KiB a tile and step
+    __shared__ __attribute__((aligned(16))) uint8_t s_ops[2][STAGE];
+    const int tid = threadIdx.x, lane = tid & 63, wave = __builtin_amdgcn_readfirstlane(tid >> 6), mr = wave >> 2, nq = wave & 3;
+    const int r32 = lane & 31, kg = lane >> 5;
+    const int row0 = blockIdx.x * 128, e0 = blockIdx.y * 256;
+    // this thread's pieces of a step: x: 128 rows x 8 pieces = 1,024 (2 a thread); w: 256 rows x 8 = 2,048 (4 a thread)
+    const uint16_t* src[6];
+    int dst[6];
 #pragma unroll
-    for (int i = 0; i < 16; ++i) acc[i] = 0.f;
-    const int k_begin = kpart * (hidden / 2), k_end = k_begin + hidden / 2;
-    const bool row_ok = row < rows;
-    for (int k = k_begin; k < k_end; k += 16) {
-        u4v av = {0, 0, 0, 0};
-        if (row_ok) av = *reinterpret_cast<const u4v*>(x + (size_t)row * hidden + k + 8 * kg);
-        const u4v bv = *reinterpret_cast<const u4v*>(w + (size_t)min(e, experts - 1) * hidden + k + 8 * kg);
-        acc = __builtin_amdgcn_mfma_f32_32x32x16_bf16(__builtin_bit_cast(bf16x8, av), __builtin_bit_cast(bf16x8, bv), acc, 0, 0, 0);
+    for (int i = 0; i < 6; ++i) {
+        const int c = tid + 512 * i, is_w = i >= 2, local = is_w ? c - 1024 : c, r = local >> 3, kc = local & 7;
+        const int tile = (is_w ? X_TILES : 0) + (r >> 5);
+        const long long source_row = is_w ? min(e0 + r, experts - 1) : min(row0 + r, rows - 1);
+        src[i] = (is_w ? w : x) + source_row * hidden + kc * 8;
+        dst[i] = ((tile * 4 + (kc >> 1)) * 64 + (kc & 1) * 32 + ((r + 2 * kc) & 31)) * 16;
     }
-    if (kpart == 1) {
+    v16f acc[2][2];
 #pragma unroll
-        for (int i = 0; i < 16; ++i) s_part[half][i * 64 + lane] = acc[i];
-    }
+    for (int a = 0; a < 2; ++a)
+#pragma unroll
+        for (int b = 0; b < 2; ++b)
+#pragma unroll
+            for (int i = 0; i < 16; ++i) acc[a][b][i] = 0.f;
+    // operands of step s + 3 are requested while step s is multiplied: a ring of three register sets (indexed statically by
+    // unrolling four steps; hidden % 512 == 0), one LDS stage ahead of the products
+    constexpr int D = 4;
+    u4v regs[D][6];
+    const int steps = hidden / 64;
+#pragma unroll
+    for (int d = 0; d < D - 1; ++d)
+#pragma unroll
+        for (int i = 0; i < 6; ++i) regs[d][i] = *reinterpret_cast<const u4v*>(src[i] + (size_t)min(d, steps - 1) * 64);
+#pragma unroll
+    for (int i = 0; i < 6; ++i) *reinterpret_cast<u4v*>(&s_ops[0][dst[i]]) = regs[0][i];
     __syncthreads();
-    if (kpart == 0) {
+    for (int step0 = 0; step0 < steps; step0 += D) {
 #pragma unroll
-        for (int i = 0; i < 16; ++i) {
-            const int m = 8 * (i >> 2) + 4 * (lane >> 5) + (i & 3);          // D[m][n = lane % 32]
-            const int out_row = blockIdx.x * 64 + half * 32 + m;
-            if (out_row < rows && e < experts) out[(size_t)out_row * experts + e] = __fadd_rn(acc[i], s_part[half][i * 64 + lane]);
+        for (int u = 0; u < D; ++u) {
+            const int step = step0 + u, stage = step & 1, ahead = min(step + D - 1, steps - 1);
+#pragma unroll
+            for (int i = 0; i < 6; ++i) regs[(u + D - 1) % D][i] = *reinterpret_cast<const u4v*>(src[i] + (size_t)ahead * 64);
+#pragma unroll
+            for (int sub = 0; sub < 4; ++sub) {
+                const int slot = (r32 + 4 * sub + 2 * kg) & 31;                 // (r + 2 kc) % 32 with kc = 2 sub + kg
+                u4v av[2], bv[2];
+#pragma unroll
+                for (int a = 0; a < 2; ++a) av[a] = *reinterpret_cast<const u4v*>(&s_ops[stage][(((2 * mr + a) * 4 + sub) * 64 + kg * 32 + slot) * 16]);
+#pragma unroll
+                for (int b = 0; b < 2; ++b) bv[b] = *reinterpret_cast<const u4v*>(&s_ops[stage][(((X_TILES + 2 * nq + b) * 4 + sub) * 64 + kg * 32 + slot) * 16]);
+#pragma unroll
+                for (int a = 0; a < 2; ++a)
+#pragma unroll
+                    for (int b = 0; b < 2; ++b)
+                        acc[a][b] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(__builtin_bit_cast(bf16x8, av[a]), __builtin_bit_cast(bf16x8, bv[b]), acc[a][b], 0, 0, 0);
+            }
+#pragma unroll
+            for (int i = 0; i < 6; ++i) *reinterpret_cast<u4v*>(&s_ops[stage ^ 1][dst[i]]) = regs[(u + 1) % D][i];
+            __syncthreads();
         }
     }
+#pragma unroll
+    for (int a = 0; a < 2; ++a)
+#pragma unroll
+        for (int b = 0; b < 2; ++b) {
+            const int e = e0 + (2 * nq + b) * 32 + r32;
+#pragma unroll
+            for (int i = 0; i < 16; ++i) {
+                const int row = row0 + (2 * mr + a) * 32 + 8 * (i >> 2) + 4 * kg + (i & 3);      // D[m][n = lane % 32]
+                if (row < rows && e < experts) out[(size_t)row * experts + e] = acc[a][b][i];
+            }
+        }
 }

@@ -251,7 +251,7 @@ extern "C" __global__ void __launch_bounds__(256) ca_quantize_rows(
                      (long long)blockIdx.x * blockDim.x + threadIdx.x, (long long)gridDim.x * blockDim.x);
 }
 
-// ---- Wide plan (any number of routes): three kernels, no atomics, same tables as the one-block plan. ----------------
+// ---- Wide plan (any number of routes): four kernels, no atomics, same tables as the one-block plan. -----------------
 // 1. One wave per 64 consecutive routes: each route's rank among the wave's earlier routes of its expert, and the wave's
 //    per-expert counts.
 extern "C" __global__ void __launch_bounds__(256) ca_plan_wave_counts(
@@ -277,19 +277,39 @@ extern "C" __global__ void __launch_bounds__(256) ca_plan_wave_counts(
     __builtin_amdgcn_wave_barrier();
     for (int e = lane; e < experts; e += 64) wave_counts[(size_t)wave * experts + e] = s_count[w][e];
 }
-// 2. One block, one thread per expert: exclusive prefix of the wave counts (in place), tiles, tile bases, task tables.
-extern "C" __global__ void __launch_bounds__(512) ca_plan_scan(
-    int32_t* wave_counts, int32_t waves, int32_t experts, int32_t groups, int32_t tile_m, int32_t* expert_tile_base,
-    int32_t* task_expert, int32_t* task_valid_rows) {
+// 2a. One block per expert: exclusive prefix of the expert's wave counts (in place); the expert's route count goes to
+//     expert_tile_base[expert] for step 2b.
+extern "C" __global__ void __launch_bounds__(256) ca_plan_scan(int32_t* wave_counts, int32_t waves, int32_t experts, int32_t* expert_tile_base) {
+    __shared__ int32_t s_wave[4];
+    const int t = threadIdx.x, lane = t & 63, wave = t >> 6, e = blockIdx.x;
+    if (e >= experts) return;
+    const int per = (waves + 255) >> 8, first = t * per, last = min(first + per, waves);
+    int sum = 0;
+    for (int w = first; w < last; ++w) sum += wave_counts[(size_t)w * experts + e];
+    int prefix = sum;
+#pragma unroll
+    for (int o = 1; o < 64; o <<= 1) {
+        const int below = __shfl_up(prefix, o);
+        if (lane >= o) prefix += below;
+    }
+    if (lane == 63) s_wave[wave] = prefix;
+    __syncthreads();
+    int run = prefix - sum;
+    for (int w = 0; w < wave; ++w) run += s_wave[w];
+    for (int w = first; w < last; ++w) {
+        const int c = wave_counts[(size_t)w * experts + e];
+        wave_counts[(size_t)w * experts + e] = run;
+        run += c;
+    }
+    if (t == 255) expert_tile_base[e] = run;
+}
+// 2b. One block, one thread per expert: tiles from the counts step 2a left in expert_tile_base, tile bases, task tables.
+extern "C" __global__ void __launch_bounds__(512) ca_plan_tiles(int32_t experts, int32_t groups, int32_t tile_m, int32_t* expert_tile_base,
+                                                                int32_t* task_expert, int32_t* task_valid_rows) {
     __shared__ int32_t s_wave[8];
     const int t = threadIdx.x, lane = t & 63, wave = t >> 6;
-    int count = 0;
-    if (t < experts)
-        for (int w = 0; w < waves; ++w) {
-            const int c = wave_counts[(size_t)w * experts + t];
-            wave_counts[(size_t)w * experts + t] = count;
-            count += c;
-        }
+    const int count = t < experts ? expert_tile_base[t] : 0;
+    __syncthreads();
     const int tiles = (count + tile_m - 1) / tile_m;
     int prefix = tiles;
 #pragma unroll

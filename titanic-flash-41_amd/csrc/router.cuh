@@ -58,7 +58,9 @@ struct RouteParams {
 };
 
 // One wave routes one row.  Lane l holds experts l, l + 64, ... (at most 8 per lane: experts <= 512).  Every lane
-// returns the same ids / weights in registers [k]; topk <= 8.
+// returns the same ids / weights in registers [k]; topk <= 8.  COHERENT: the logits were written by other workgroups of this
+// launch (device-scope loads); otherwise by an earlier launch (plain loads).
+template <bool COHERENT>
 __device__ __forceinline__ void tf_route_row(const float* logits, const float* bias, int lane, const RouteParams& p,
                                              int32_t* out_ids, float* out_weights) {
     float score[8], biased[8];
@@ -68,7 +70,7 @@ __device__ __forceinline__ void tf_route_row(const float* logits, const float* b
         score[i] = 0.f;
         biased[i] = -INFINITY;
         if (e < p.experts) {
-            const float x = tf_acquire_f32(logits + e);
+            const float x = COHERENT ? tf_acquire_f32(logits + e) : logits[e];
             float s;
             if (p.scoring == 1) s = __builtin_sqrtf(x > 20.f ? x : tf_log1p_pos(tf_exp(x)));
             else s = tf_logistic(x);
@@ -131,6 +133,7 @@ __device__ __forceinline__ void tf_apply_padding(const int32_t* padding, int32_t
 
 // Routes rows [first_row, first_row + waves of this block) of `rows`; rows at or past min(rows, live[0]) get ids -1 and
 // weights 0.  `padding` (may be null) is applied only by a single-block launch, after a block barrier.
+template <bool COHERENT = true>
 __device__ __forceinline__ void tf_route_block(const float* logits, const float* bias, const float* bias_alt,
                                                const long long* tokens, const int32_t* live, const int32_t* padding,
                                                int32_t* ids, float* weights, int rows, const RouteParams& p,
@@ -144,7 +147,7 @@ __device__ __forceinline__ void tf_route_block(const float* logits, const float*
         float share[8];
         if (is_live) {
             const bool alt = bias_alt != nullptr && tokens != nullptr && p.alt_token >= 0 && tokens[row] == p.alt_token;
-            tf_route_row(logits + (size_t)row * p.experts, alt ? bias_alt : bias, lane, p, chosen, share);
+            tf_route_row<COHERENT>(logits + (size_t)row * p.experts, alt ? bias_alt : bias, lane, p, chosen, share);
         }
 #pragma unroll
         for (int k = 0; k < 8; ++k)
@@ -177,7 +180,7 @@ extern "C" __global__ void ca_route_topk(const float* logits, const float* bias,
                                          int32_t scoring, float route_scale, long long alt_token) {
     const RouteParams p{experts, topk, scoring, route_scale, alt_token};
     const int waves = blockDim.x >> 6;
-    tf_route_block(logits, bias, bias_alt, tokens, live, padding, ids, weights, rows, p, blockIdx.x * waves,
+    tf_route_block<false>(logits, bias, bias_alt, tokens, live, padding, ids, weights, rows, p, blockIdx.x * waves,
                    gridDim.x * waves, gridDim.x == 1);
 }
 

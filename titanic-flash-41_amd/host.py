@@ -125,6 +125,13 @@ class Layer:
         self.lib.tfh_layer_run_quantized.argtypes = [ctypes.c_void_p, ctypes.c_uint64, ctypes.c_uint64, ctypes.c_uint64, ctypes.c_char_p, ctypes.c_size_t]
         self._check(self.lib.tfh_layer_run_quantized(self.h, x.data_ptr(), codes.data_ptr(), scales.data_ptr(), self._err, 512))
 
+    def run_row_transport(self, x, packed_out=None):
+        """One pass through the one-rank row transport: pack to wire rows, routed experts from the packed rows, shared expert from
+        the decoded codes.  `packed_out`: optional uint8 device tensor [rows, hidden * 37 // 32] that receives the packed rows."""
+        self.lib.tfh_layer_run_row_transport.argtypes = [ctypes.c_void_p, ctypes.c_uint64, ctypes.c_uint64, ctypes.c_char_p, ctypes.c_size_t]
+        assert x.is_cuda and x.is_contiguous() and x.numel() == self.rows * self.g.hidden
+        self._check(self.lib.tfh_layer_run_row_transport(self.h, x.data_ptr(), packed_out.data_ptr() if packed_out is not None else 0, self._err, 512))
+
     def capture(self, xs):
         """Captures one pass over each tensor of `xs` (or the single tensor `xs`), in order, into one graph."""
         xs = [xs] if not isinstance(xs, (list, tuple)) else list(xs)

@@ -128,6 +128,20 @@ int tfh_layer_run_quantized(void* handle, uint64_t input, uint64_t codes, uint64
         h->stream->synchronize();
     });
 }
+// One eager pass through the row transport of the sequence-parallel prefill on one rank (LayerFfn::run_row_transport): the rows
+// are packed into wire rows "dual_quant_rows_v1", the routed experts run from the packed rows, the shared expert from the codes
+// decoded out of them.  `packed_out` (may be 0): device address that receives a copy of the packed rows (rows x hidden x 37 / 32).
+int tfh_layer_run_row_transport(void* handle, uint64_t input, uint64_t packed_out, char* error, size_t error_len) {
+    Handle* h = (Handle*)handle;
+    return guarded(error, error_len, [&] {
+        if (!h->layer->row_transport_active()) h->layer->enable_row_transport();
+        h->layer->run_row_transport(*h->workspace, input, h->rows * (size_t)h->native->geometry().hidden, *h->tokens, *h->stream);
+        if (packed_out)
+            tf::check(hipMemcpyAsync((void*)packed_out, (const void*)h->layer->packed_rows().ptr(), h->layer->packed_rows().len(), hipMemcpyDeviceToDevice,
+                                     h->stream->raw()), "copy packed rows");
+        h->stream->synchronize();
+    });
+}
 // Captures one pass over each of `count` inputs, in order, into one graph (the reference captures its whole forward, forty
 // layers' passes, into one graph and replays it: src/probe.rs:1527-1542, src/cuda.rs:2068-2153); returns the graph's index.
 int tfh_layer_capture(void* handle, const uint64_t* inputs, int count, char* error, size_t error_len) {

@@ -32,6 +32,10 @@ Native::Native(const std::string& library, const ca_geometry& geometry) : g_(geo
     launch_ = symbol<decltype(launch_)>(lib_, "ca_primitives_launch");
     scratch_bytes_ = symbol<decltype(scratch_bytes_)>(lib_, "ca_primitives_scratch_bytes");
     marks_ = symbol<decltype(marks_)>(lib_, "ca_primitives_marks");
+    encode_ = symbol<decltype(encode_)>(lib_, "ca_encode");                                              // src/ffn.rs:808-811
+    decode_ = symbol<decltype(decode_)>(lib_, "ca_decode");
+    local_live_ = symbol<decltype(local_live_)>(lib_, "ca_local_live");
+    pack_bf16_ = symbol<decltype(pack_bf16_)>(lib_, "ca_pack_bf16");
     int32_t status = 0;
     ctx_ = symbol<void* (*)(int32_t*)>(lib_, "ca_primitives_open")(&status);
     if (status != 0 || !ctx_) throw Error("initialize primitive library: " + std::to_string(status));   // src/primitives.rs:116-119
@@ -42,6 +46,18 @@ Native::~Native() {
 }
 void Native::marks(hipEvent_t* events) const {
     ensure(marks_(ctx_, (void* const*)events, events ? 5 : 0) == 0, "profiling marks rejected");
+}
+void Native::codec_encode(uint64_t routed, uint64_t scales, uint64_t shared, uint64_t packed, int rows, int k, hipStream_t s) const {
+    ensure(encode_((const uint8_t*)routed, (const uint8_t*)scales, (const uint8_t*)shared, (uint8_t*)packed, rows, k, s) == 0, "packed MoE encode launch");   // src/ffn.rs:856-858
+}
+void Native::codec_decode(uint64_t packed, uint64_t shared, uint64_t row_scales, uint64_t mma_scales, int rows, int k, hipStream_t s) const {
+    ensure(decode_((const uint8_t*)packed, (uint8_t*)shared, (uint8_t*)row_scales, (uint8_t*)mma_scales, rows, k, s) == 0, "packed MoE shared decode launch");   // :872-874
+}
+void Native::codec_local_live(uint64_t global, uint64_t local, int rows, int rank, hipStream_t s) const {
+    ensure(local_live_((const int*)global, (int*)local, rows, rank, s) == 0, "packed MoE local metadata launch");                   // :845-846
+}
+void Native::codec_pack_bf16(uint64_t input, uint64_t packed, int rows, int k, hipStream_t s) const {
+    ensure(pack_bf16_((const void*)input, (uint8_t*)packed, rows, k, s) == 0, "fused packed MoE producer launch");                  // :849-850
 }
 void Native::router_logits(int rows, uint64_t x, uint64_t w, uint64_t out, hipStream_t s) const {
     ensure(router_logits_(rows, (const void*)x, (const void*)w, (void*)out, s) == 0, "tiny router GPU launch failed");   // src/ffn.rs:352-363
@@ -406,6 +422,20 @@ void Workspace::run_live(const Expert& expert, uint64_t input, size_t input_len,
     const int32_t ss[3] = {(int32_t)live, 0, 0};
     native_->primitive(2, sp, 3, ss, 3, stream.raw(), "moe.w4a16.topk_sum");
 }
+void Workspace::run_packed(const Expert& expert, uint64_t packed, size_t packed_len, const Buffer<int32_t>& ids, const Buffer<float>& routing_weights,
+                           const Stream& stream) {                                                             // src/moe.rs:571-577
+    const ca_geometry& g = native_->geometry();
+    guard_stream(stream);
+    ensure(g.act_block == 32 && packed && packed_len == rows_ * (size_t)g.hidden * 37 / 32, "packed MoE operand");
+    ensure(ids.len() == rows_ * g.topk && routing_weights.len() == rows_ * g.topk, "MoE input shape mismatch");
+    uint64_t p[21];
+    pointers(expert, packed, ids, routing_weights, p);
+    const int32_t scalars[6] = {(int32_t)rows_, (int32_t)rows_, (int32_t)(max_tiles_ * tile_m_), (int32_t)max_tiles_, (int32_t)tile_m_, 1};
+    native_->primitive(10, p, 21, scalars, 6, stream.raw(), "integration.tp_moe.dynamic (dual_quant_rows_v1)");
+    const uint64_t sp[3] = {at("scatter_ptr"), output_.ptr(), 0};
+    const int32_t ss[3] = {(int32_t)rows_, 0, 0};
+    native_->primitive(2, sp, 3, ss, 3, stream.raw(), "moe.w4a16.topk_sum");
+}
 void Workspace::run_phase(int entry, const Expert& expert, uint64_t input, const Buffer<int32_t>& ids, const Buffer<float>& routing_weights,
                           const Stream& stream) {
     ensure(entry == 6 || entry == 7 || entry == 8, "phase entry");
@@ -488,6 +518,37 @@ void LayerFfn::run_quantized_input(Workspace& workspace, uint64_t input, size_t 
     else run_shared(workspace, 0, stream);
     if (deferred) sum_shared(workspace, deferred->second, stream);
     else add_shared(workspace, stream);
+}
+void LayerFfn::enable_row_transport() {                                                                        // src/ffn.rs:789-822
+    const ca_geometry& g = native_->geometry();
+    ensure(g.act_block == 32 && rows_ % 128 == 0 && !row_transport_active(), "packed MoE transport requires the wide sequential profile");
+    packed_ = Buffer<uint8_t>(rows_ * (size_t)g.hidden * 37 / 32);
+    decoded_codes_ = Buffer<uint8_t>(rows_ * (size_t)g.hidden);
+    decoded_scales_ = Buffer<uint8_t>(rows_ * (size_t)g.hidden / 32);
+    local_live_ = Buffer<int32_t>(1);
+}
+void LayerFfn::run_row_transport(Workspace& workspace, uint64_t input, size_t input_len, const TokenRows& tokens, const Stream& stream) {   // :827-878
+    const ca_geometry& g = native_->geometry();
+    ensure(row_transport_active() && tokens.rows() == rows_ && input && input_len == rows_ * (size_t)g.hidden && workspace.rows() == rows_,
+           "packed MoE transport input geometry/context");
+    // one rank: its share is every row, its live count the batch's
+    native_->codec_local_live(tokens.live().ptr(), local_live_.ptr(), (int)rows_, 0, stream.raw());
+    router_.run(input, input_len, tokens, stream);
+    native_->codec_pack_bf16(input, packed_.ptr(), (int)rows_, g.hidden, stream.raw());
+    // (all-gather of packed rows, ids and routing weights over the ranks goes here)
+    native_->codec_decode(packed_.ptr(), decoded_codes_.ptr(), decoded_scales_.ptr(), 0, (int)rows_, g.hidden, stream.raw());
+    if (branch_stream_) {                                                                                      // :566-584 run_packed_and_shared
+        input_ready_->record(stream.raw());
+        workspace.run_packed(expert_, packed_.ptr(), packed_.len(), router_.ids(), router_.routing(), stream);
+        input_ready_->wait(branch_stream_->raw());
+        run_shared_quantized(decoded_codes_.ptr(), decoded_scales_.ptr(), *branch_stream_);
+        output_ready_->record(branch_stream_->raw());
+        output_ready_->wait(stream.raw());
+    } else {
+        workspace.run_packed(expert_, packed_.ptr(), packed_.len(), router_.ids(), router_.routing(), stream);
+        run_shared_quantized(decoded_codes_.ptr(), decoded_scales_.ptr(), stream);
+    }
+    add_shared(workspace, stream);
 }
 void LayerFfn::sum_shared(const Workspace& workspace, size_t live_rows, const Stream& stream) {               // :1037-1046 ca_ffn_sum_shared
     const ca_geometry& g = native_->geometry();

@@ -40,6 +40,11 @@ public:
     int64_t scratch_bytes(int index, int rows) const;
     // five events recorded around the launches of the dynamic entries (null: off)
     void marks(hipEvent_t* events) const;
+    // the wire row "dual_quant_rows_v1" (src/ffn.rs:805-811 RowTransport's functions)
+    void codec_encode(uint64_t routed, uint64_t scales, uint64_t shared, uint64_t packed, int rows, int k, hipStream_t s) const;
+    void codec_decode(uint64_t packed, uint64_t shared, uint64_t row_scales, uint64_t mma_scales, int rows, int k, hipStream_t s) const;
+    void codec_local_live(uint64_t global, uint64_t local, int rows, int rank, hipStream_t s) const;
+    void codec_pack_bf16(uint64_t input, uint64_t packed, int rows, int k, hipStream_t s) const;
 private:
     void* lib_ = nullptr;
     void* ctx_ = nullptr;
@@ -53,6 +58,10 @@ private:
     int32_t (*launch_)(void*, int32_t, const uint64_t*, size_t, const int32_t*, size_t, void*) = nullptr;
     int64_t (*scratch_bytes_)(void*, int32_t, int32_t) = nullptr;
     int32_t (*marks_)(void*, void* const*, size_t) = nullptr;
+    int (*encode_)(const uint8_t*, const uint8_t*, const uint8_t*, uint8_t*, int, int, void*) = nullptr;
+    int (*decode_)(const uint8_t*, uint8_t*, uint8_t*, uint8_t*, int, int, void*) = nullptr;
+    int (*local_live_)(const int*, int*, int, int, void*) = nullptr;
+    int (*pack_bf16_)(const void*, uint8_t*, int, int, void*) = nullptr;
 };
 
 // ---- device atlas (src/weights.rs:276-417: contiguous expert groups, 256-byte aligned views) --------------------------
@@ -180,6 +189,10 @@ public:
     // run_live (:1011-1043): only the first `live` rows are launched (ids / weights given); output() holds their reduced rows.
     void run_live(const Expert& expert, uint64_t input, size_t input_len, const Buffer<int32_t>& ids, const Buffer<float>& routing_weights,
                   size_t live, const Stream& stream);
+    // run_packed (src/moe.rs:571-577): the routed experts from wire rows "dual_quant_rows_v1" (rows x hidden x 37 / 32 bytes,
+    // 32-wide activation blocks) instead of BF16 rows; every row is launched.
+    void run_packed(const Expert& expert, uint64_t packed, size_t packed_len, const Buffer<int32_t>& ids, const Buffer<float>& routing_weights,
+                    const Stream& stream);
     // Phase nodes alone (for per-kernel timing): 8 = front-end (plan + quantize), 6 = FC1 + SwiGLU, 7 = FC2.
     void run_phase(int entry, const Expert& expert, uint64_t input, const Buffer<int32_t>& ids, const Buffer<float>& routing_weights, const Stream& stream);
     // scratch regions by role name (the runtime contract's pointer table)
@@ -238,8 +251,17 @@ public:
     // the shared expert from given codes / scales (Linear::run_quantized, src/fp8_linear.rs:792-806)
     void run_shared_quantized(uint64_t codes, uint64_t scales, const Stream& stream);
     void sum_shared(const Workspace& workspace, size_t live_rows, const Stream& stream);
+    // Row transport of the sequence-parallel prefill on one rank (src/ffn.rs:789-878): the rows are routed, packed into wire rows
+    // by the fused producer, (gathered: with one rank the rows are already all here), the shared quantizer's codes are decoded
+    // from them, the routed experts run from the packed rows and the shared expert from the decoded codes.
+    void enable_row_transport();
+    bool row_transport_active() const { return packed_.len() != 0; }
+    void run_row_transport(Workspace& workspace, uint64_t input, size_t input_len, const TokenRows& tokens, const Stream& stream);
+    const Buffer<uint8_t>& packed_rows() const { return packed_; }
 private:
     void add_shared(const Workspace& workspace, const Stream& stream);
+    Buffer<uint8_t> packed_, decoded_codes_, decoded_scales_;
+    Buffer<int32_t> local_live_;
     std::shared_ptr<const Native> native_;
     Router router_;
     Expert expert_;

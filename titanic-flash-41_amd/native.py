@@ -12,7 +12,8 @@ CODE_OBJECT = os.path.join(HERE, "titanic_moe_gfx950.hsaco")
 EXPORTS = ["ca_ffn_abi", "ca_ffn_configure", "ca_ffn_geometry", "ca_router_logits", "ca_shared_swiglu", "ca_ffn_add",
            "ca_router_logits_wide", "ca_kernel_launch", "ca_kernel_count", "ca_kernel_name", "ca_moe_nibble_permute",
            "ca_primitives_abi", "ca_primitives_open", "ca_primitives_close", "ca_primitives_launch", "ca_primitives_launch2",
-           "ca_primitives_entries", "ca_primitives_scratch_bytes", "ca_primitives_marks"]
+           "ca_primitives_entries", "ca_primitives_scratch_bytes", "ca_primitives_marks", "ca_encode", "ca_decode", "ca_local_live",
+           "ca_pack_bf16"]
 
 
 class Geometry(ctypes.Structure):
@@ -58,6 +59,10 @@ def load():
     lib.ca_primitives_entries.restype = i32
     lib.ca_primitives_scratch_bytes.restype = ctypes.c_int64
     lib.ca_primitives_scratch_bytes.argtypes = [vp, i32, i32]
+    lib.ca_encode.argtypes = [vp, vp, vp, vp, ctypes.c_int, ctypes.c_int, vp]
+    lib.ca_decode.argtypes = [vp, vp, vp, vp, ctypes.c_int, ctypes.c_int, vp]
+    lib.ca_local_live.argtypes = [vp, vp, ctypes.c_int, ctypes.c_int, vp]
+    lib.ca_pack_bf16.argtypes = [vp, vp, ctypes.c_int, ctypes.c_int, vp]
     lib.ca_primitives_marks.restype = i32
     lib.ca_primitives_marks.argtypes = [vp, ctypes.POINTER(vp), ctypes.c_size_t]
     _lib = lib
