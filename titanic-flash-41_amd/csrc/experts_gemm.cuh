@@ -63,6 +63,8 @@ __global__ void __launch_bounds__(512) tf_gemm(const GemmArgs p) {
     __shared__ __attribute__((aligned(16))) uint8_t s_scale[128 * (TF_GEMM_MAX_SCALES_ROW + 4)];    // [row][k-block]: the tile's activation scales; the row stride is an odd number of words
     __shared__ float s_amax[4][128];
     __shared__ long long s_row[128];                                    // source row of each tile row
+    __shared__ int32_t s_route[128];                                    // routed FC2: route (output row) of each tile row
+    __shared__ float s_weight[128];                                     // routed FC2: routing weight of each tile row
     // eight waves: row half mh (64 rows = four 16-row fragments) x column quarter nq (64 weight rows = four 16-row tiles)
     // the wave's index as a scalar: everything derived from it (weight tile addresses, LDS fragment offsets) stays out of the vector registers
     const int tid = threadIdx.x, lane = tid & 63, wave = __builtin_amdgcn_readfirstlane(tid >> 6), mh = wave >> 2, nq = wave & 3, g = lane >> 4, r16 = lane & 15;
@@ -76,26 +78,40 @@ __global__ void __launch_bounds__(512) tf_gemm(const GemmArgs p) {
     const int gpx = split ? groups / 8 : 0;
     const long long my_tasks = split ? (long long)tiles * gpx : ((long long)tiles * groups - xcd + 7) / 8;
 
+    // What a tile needs from the plan tables is requested a whole tile ahead (with the previous tile's first operand loads), so
+    // that no tile starts with a chain of dependent round trips: the tile's expert and row count, and per tile row its source
+    // row (routed FC1: through the permutation map) or its route and routing weight (routed FC2).  The last tile requests
+    // itself again: no load is conditional.
+    struct TileRef { int tile, ng, expert, valid; long long src; int32_t route; float weight; };
+    auto fetch = [&](long long q) {
+        TileRef r;
+        if (split) { r.tile = (int)(q / gpx); r.ng = xcd * gpx + (int)(q % gpx); }
+        else { const long long id = q * 8 + xcd; r.tile = (int)(id / groups); r.ng = (int)(id % groups); }
+        r.expert = 0;
+        if (ROUTED) { r.expert = p.task_expert[r.tile * p.groups]; r.valid = p.task_valid_rows[r.tile * p.groups]; }
+        else r.valid = min(128, p.dense_rows - r.tile * 128);
+        const int at = r.tile * 128 + (tid & 127);
+        r.src = at; r.route = 0; r.weight = 0.f;
+        if (MODE == TF_GEMM_FC1_ROUTED) r.src = p.token_map[at];          // route index; rows past the valid ones: never looked up
+        if (MODE == TF_GEMM_FC2_ROUTED) { r.route = p.token_map[at]; r.weight = p.token_weights[at]; }
+        return r;
+    };
+    if (local >= my_tasks) return;
+    TileRef next = fetch(local);
     for (long long q = local; q < my_tasks; q += local_count) {
-        int tile, ng;
-        if (split) { tile = (int)(q / gpx); ng = xcd * gpx + (int)(q % gpx); }
-        else { const long long id = q * 8 + xcd; tile = (int)(id / groups); ng = (int)(id % groups); }
-        int expert = 0, valid;
-        if (ROUTED) { expert = p.task_expert[tile * p.groups]; valid = p.task_valid_rows[tile * p.groups]; }
-        else valid = min(128, p.dense_rows - tile * 128);
+        const TileRef cur = next;
+        const int tile = cur.tile, ng = cur.ng, expert = cur.expert, valid = cur.valid;
         const uint8_t* w = p.w + (size_t)expert * p.w_expert_stride;
         const uint8_t* ws = p.ws + (size_t)expert * p.ws_expert_stride;
         __syncthreads();
         if (tid < 128) {
-            // rows past the last valid one re-read the last valid row (no load of the main loop is conditional); their products
-            // are never stored
-            const int t = min(tid, valid - 1);
-            long long src;
-            if (MODE == TF_GEMM_FC1_ROUTED) src = p.token_map[tile * 128 + t] / p.topk;
-            else src = (long long)tile * 128 + t;
-            s_row[tid] = src;
+            s_row[tid] = MODE == TF_GEMM_FC1_ROUTED ? cur.src / p.topk : cur.src;
+            if (MODE == TF_GEMM_FC2_ROUTED) { s_route[tid] = cur.route; s_weight[tid] = cur.weight; }
         }
         __syncthreads();
+        next = fetch(min(q + local_count, my_tasks - 1));
+        // rows past the last valid one re-read the last valid row (no load of the main loop is conditional); their products are
+        // never stored
         // this thread's two 16-byte chunks of every k-step's A tile: chunk id c = tid + 512 i is LDS slot c (a wave fills one
         // 1 KiB fragment block with consecutive 16-byte slots: no bank conflicts), i.e. fragment c / 128, K half (c / 64) % 2,
         // row c % 16 of the fragment, 16-byte piece (c % 64) / 16 of the half
@@ -105,7 +121,7 @@ __global__ void __launch_bounds__(512) tf_gemm(const GemmArgs p) {
         for (int i = 0; i < 2; ++i) {
             const int c = tid + 512 * i, block = c >> 6, slot = c & 63;
             const int row = (block >> 1) * 16 + (slot & 15), piece = (block & 1) * 4 + (slot >> 4);
-            a_src[i] = p.a_codes + s_row[row] * p.k + piece * 16;
+            a_src[i] = p.a_codes + s_row[min(row, valid - 1)] * p.k + piece * 16;
             a_dst[i] = c * 16;
         }
         // weight row tiles of this wave: FC1 routed: two "up" tiles then two "gate" tiles of the same 32 intermediate columns;
@@ -131,7 +147,7 @@ __global__ void __launch_bounds__(512) tf_gemm(const GemmArgs p) {
 #pragma unroll
         for (int i = 0; i < TF_GEMM_SCALE_WORDS; ++i) {
             const int c = min(tid + 512 * i, 128 * scale_words_row - 1);            // word c % per_row of row c / per_row
-            scale_regs[i] = *reinterpret_cast<const uint32_t*>(p.a_scales + s_row[c / scale_words_row] * scales_row + (c % scale_words_row) * 4);
+            scale_regs[i] = *reinterpret_cast<const uint32_t*>(p.a_scales + s_row[min(c / scale_words_row, valid - 1)] * scales_row + (c % scale_words_row) * 4);
         }
         auto store_scales = [&]() {
 #pragma unroll
@@ -340,10 +356,9 @@ __global__ void __launch_bounds__(512) tf_gemm(const GemmArgs p) {
                     for (int i = 0; i < 4; ++i) {
                         const int row = 64 * mh + 16 * f + 4 * g + i;
                         if (row < valid) {
-                            const int phys = tile * 128 + row;
-                            size_t out_row = (size_t)phys;
+                            size_t out_row = (size_t)tile * 128 + row;
                             float scale = 1.f;
-                            if (MODE == TF_GEMM_FC2_ROUTED) { out_row = (size_t)p.token_map[phys]; scale = p.token_weights[phys]; }
+                            if (MODE == TF_GEMM_FC2_ROUTED) { out_row = (size_t)s_route[row]; scale = s_weight[row]; }
 #pragma unroll
                             for (int j = 0; j < 4; ++j) {
                                 const float v = MODE == TF_GEMM_FC2_ROUTED ? __fmul_rn(acc[f][j][i], scale) : acc[f][j][i];
