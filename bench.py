@@ -1,7 +1,7 @@
 #!/usr/bin/env python3
 """Benchmark of the MoE FFN layer on one MI355X.
 
-    python bench.py [--gpus 1] [--steps K] [--warmup W] [--config c2|c3]
+    python bench.py [--gpus 1] [--steps K] [--warmup W] [--config c2|c3|c4|c5] [--numerics benchmark|reference]
 
 A step is one pass of the whole layer (gate product, top-k + plan + token quantization, routed FC1 + SwiGLU, FC2, shared
 expert, ordered sum + shared addition) over one batch of synthetic token rows that is already resident in HBM, replayed
@@ -119,6 +119,9 @@ def main():
     ap.add_argument("--steps", type=int, default=2000)
     ap.add_argument("--warmup", type=int, default=200)
     ap.add_argument("--config", default="c2", choices=sorted(CONFIGS))
+    ap.add_argument("--numerics", default="benchmark", choices=["benchmark", "reference"],
+                    help="benchmark: sigmoid scores, renormalised, 128-wide activation blocks, 128 x 128 shared weight blocks (the headline); "
+                         "reference: the reference's own numerics (sqrt-softplus x 1.5, 32-wide blocks, 32 x 32, image-token bias)")
     ap.add_argument("--no-cpu-baseline", action="store_true")
     ap.add_argument("--copy-probe", action="store_true", help="append four 256 MiB device copies (counter calibration)")
     ap.add_argument("--profile-steps", type=int, default=64, help="eager passes with per-kernel HIP events for the roofline")
@@ -132,7 +135,11 @@ def main():
     pkg = importlib.import_module("titanic-flash-41_amd")
     native, synth, host = pkg.native, pkg.synth, pkg.host
     cfg = CONFIGS[args.config]
-    g = native.Geometry(cfg["hidden"], cfg["experts"], cfg["topk"], cfg["inter"], cfg["shared"], 0, 1.0, 128, 128, 128, -1, 10.0)
+    if args.numerics == "benchmark":
+        g = native.Geometry(cfg["hidden"], cfg["experts"], cfg["topk"], cfg["inter"], cfg["shared"], 0, 1.0, 128, 128, 128, -1, 10.0)
+    else:
+        g = native.Geometry(cfg["hidden"], cfg["experts"], cfg["topk"], cfg["inter"], cfg["shared"], 1, 1.5, 32, 32, 32, 129264, 10.0)
+    B, BN, BK = g.act_block, g.shared_bn, g.shared_bk
     torch.cuda.set_device(0)
     t0 = time.time()
     wide = cfg["rows"] > 64
@@ -178,14 +185,14 @@ def main():
     distinct = float(np.mean([len(set(ids.ravel().tolist())) for ids in ids_per_batch]))
     tiles = float(np.mean(tiles_per_batch))
     # algorithmic bytes: every streamed tile of FC1 reads one expert's up + gate weights and scales once
-    fc1_bytes = tiles * (2 * I * H // 2 + 2 * I * H // 32) + rows * (H + H // 128) + rows * K * I * 2
+    fc1_bytes = tiles * (2 * I * H // 2 + 2 * I * H // 32) + rows * (H + H // B) + rows * K * I * 2
     fc2_bytes = tiles * (H * I // 2 + H * I // 32) + rows * K * I * 2 + rows * K * H * 2
     shared_bytes = 3 * H * S + rows * (H + 2 * S * 2 + S * 2 + H * 2)
     router_bytes = 2 * E * H + rows * H * 2
     step_bytes = fc1_bytes + fc2_bytes + shared_bytes + router_bytes + rows * (K + 2) * H * 2
     # few rows: the shared expert's projections stream inside the same two launches
-    shared_fc1_bytes = 2 * S * H + (2 * S // 128) * (H // 128) + rows * (H + H // 128) + rows * S * 2
-    shared_fc2_bytes = H * S + (H // 128) * (S // 128) + rows * S * 2 + rows * H * 2
+    shared_fc1_bytes = 2 * S * H + (2 * S // BN) * (H // BK) + rows * (H + H // B) + rows * S * 2
+    shared_fc2_bytes = H * S + (H // BN) * (S // BK) + rows * S * 2 + rows * H * 2
     phase1_bytes = fc1_bytes + (0 if wide else shared_fc1_bytes)
     phase2_bytes = fc2_bytes + (0 if wide else shared_fc2_bytes)
     fc1_ms = float(parts[2])
@@ -210,18 +217,20 @@ def main():
         "metric": "MoE-layer tokens/s", "value": value, "unit": "tokens/s", "n_gpus": 1, "steps": args.steps, "warmup": args.warmup,
         "ms_per_step": ms_per_step, "higher_is_better": True, "scaling": "weak", "vs_baseline": None,
         "dtype": "fp4 (e2m1 weights, ue8m0 scales) x fp8 (e4m3 activations), f32 accumulate",
-        "data": "synthetic", "config": {"workload": args.config + ": " + cfg["workload"], "numerics": "sigmoid top-k renormalised, 128-wide activation blocks",
+        "data": "synthetic", "config": {"workload": args.config + ": " + cfg["workload"], "numerics": ("sigmoid top-k renormalised, 128-wide activation blocks" if args.numerics == "benchmark" else
+                                                     "reference numerics: sqrt-softplus scores x 1.5, 32-wide activation blocks, 32 x 32 shared weight blocks"),
                                         "input_batches": batches, "distinct_experts_per_step": distinct, "schedule": "HIP graph replay (%d passes a graph)" % batches},
         "roofline": ({"bound": "mfma", "kernel": "tf_gemm<fp4, FC1> (routed FC1 + SwiGLU + FP8 requantization)",
                       "achieved": fc1_flops / (fc1_ms * 1e-3) / 1e12, "peak": MFMA_FP8_PEAK_TFLOPS, "unit": "TFLOP/s",
                       "frac": fc1_flops / (fc1_ms * 1e-3) / 1e12 / MFMA_FP8_PEAK_TFLOPS,
                       "frac_of_fp4_peak": fc1_flops / (fc1_ms * 1e-3) / 1e12 / MFMA_FP4_PEAK_TFLOPS,
                       "operands": "A = FP8 E4M3 activations, B = FP4 E2M1 weights: issues at the FP8 rate (measured)",
-                      "traffic": WIDE_TRAFFIC_BYTES.get(args.config), "traffic_source": "rocprofv3 counters on tf_layer_probe at the same rows (profiles/)",
+                      "traffic": WIDE_TRAFFIC_BYTES.get(args.config) if args.numerics == "benchmark" else None, "traffic_source": "rocprofv3 counters on tf_layer_probe at the same rows (profiles/)",
                       "flops_per_launch": fc1_flops, "avg_launch_ms": fc1_ms, "weight_gbs": fc1_bytes / (fc1_ms * 1e-3) / 1e9} if wide else
                      {"bound": "hbm", "kernel": "tf_phase1_stream (FC1 + SwiGLU of the routed experts and the shared expert in one launch)",
                       "achieved": achieved, "peak": HBM_PEAK_GBS, "unit": "GB/s", "frac": achieved / HBM_PEAK_GBS,
-                      "traffic": (TRAFFIC_OVER_ALGORITHMIC[args.config] * phase1_bytes if args.config in TRAFFIC_OVER_ALGORITHMIC else None),
+                      "traffic": (TRAFFIC_OVER_ALGORITHMIC[args.config] * phase1_bytes
+                                  if args.config in TRAFFIC_OVER_ALGORITHMIC and args.numerics == "benchmark" else None),
                       "bytes_per_launch": phase1_bytes, "avg_launch_ms": fc1_ms}),
         "step_tflops": step_flops / (ms_per_step * 1e-3) / 1e12, "busiest_expert_rows": max_load, "phys_tiles": tiles,
         "step_bytes": step_bytes, "step_gbs": step_bytes / (ms_per_step * 1e-3) / 1e9, "step_hbm_frac": step_bytes / (ms_per_step * 1e-3) / 1e9 / HBM_PEAK_GBS,
