@@ -164,9 +164,10 @@ extern "C" __global__ void __launch_bounds__(512) ca_moe_route_frontend(
     if (gate_w != nullptr && (int)blockIdx.x >= first_logit_block) {
         const int lb = (int)blockIdx.x - first_logit_block, group = lb / per_group, e = (lb - group * per_group) * waves + wave;
         const int first_row = 4 * group;
-        if (e < experts && first_row < owner_rows)
-            tf_logits_expert(input + (size_t)first_row * cols, gate_w, logits + (size_t)first_row * experts, min(4, owner_rows - first_row), cols,
-                             experts, e, lane);
+        __shared__ u4v s_x[4096];                     // four token rows of at most 8,192 columns
+        if (first_row < owner_rows)
+            tf_logits_block(input + (size_t)first_row * cols, gate_w, logits + (size_t)first_row * experts, min(4, owner_rows - first_row), cols,
+                            experts, e, lane, s_x);
         tf_stores_done();
         __syncthreads();
         if (!distributed) {

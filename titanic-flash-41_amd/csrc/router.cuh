@@ -44,6 +44,53 @@ __device__ __forceinline__ void tf_logits_expert(const uint16_t* __restrict__ x,
         }
     }
 }
+// The same product for one workgroup of the experts' front-end: wave `wave` takes expert `e`, all waves share at most four
+// token rows.  One round trip: every lane requests its expert's whole row (hidden / 512 vectors) and the workgroup requests
+// the token rows once (instead of once a wave), which then go through LDS.  Same summation order as tf_logits_expert.
+// Block barrier inside; hidden <= 8192; `s_x` holds rows * hidden / 8 vectors (at most 4,096).
+__device__ __forceinline__ void tf_logits_block(const uint16_t* __restrict__ x, const uint16_t* __restrict__ w, float* __restrict__ out,
+                                                int rows, int hidden, int experts, int e, int lane, u4v* s_x) {
+    const int nj = hidden >> 9, per_row = hidden >> 3, total = rows * per_row;
+    const bool on = e < experts;
+    u4v wv[16], xr[8];
+    const u4v* wrow = reinterpret_cast<const u4v*>(w + (size_t)(on ? e : 0) * hidden);
+#pragma unroll
+    for (int j = 0; j < 16; ++j) if (j < nj) wv[j] = wrow[j * 64 + lane];
+#pragma unroll
+    for (int i = 0; i < 8; ++i) {
+        const int v = (int)threadIdx.x + (int)blockDim.x * i;
+        if (v < total) xr[i] = reinterpret_cast<const u4v*>(x)[v];           // the rows are consecutive: row v / per_row
+    }
+#pragma unroll
+    for (int i = 0; i < 8; ++i) {
+        const int v = (int)threadIdx.x + (int)blockDim.x * i;
+        if (v < total) s_x[v] = xr[i];
+    }
+    __syncthreads();
+    if (!on) return;
+    float acc[4] = {0.f, 0.f, 0.f, 0.f};
+#pragma unroll
+    for (int j = 0; j < 16; ++j)
+        if (j < nj) {
+#pragma unroll
+            for (int r = 0; r < 4; ++r)
+                if (r < rows) {
+                    const u4v xv = s_x[r * per_row + j * 64 + lane];
+#pragma unroll
+                    for (int i = 0; i < 4; ++i) {
+                        acc[r] = __fmaf_rn(tf_bf16_lo(xv[i]), tf_bf16_lo(wv[j][i]), acc[r]);
+                        acc[r] = __fmaf_rn(tf_bf16_hi(xv[i]), tf_bf16_hi(wv[j][i]), acc[r]);
+                    }
+                }
+        }
+#pragma unroll
+    for (int r = 0; r < 4; ++r) {
+        float v = acc[r];
+#pragma unroll
+        for (int o = 32; o > 0; o >>= 1) v = __fadd_rn(v, __shfl_xor(v, o));
+        if (lane == 0 && r < rows) tf_publish_f32(out + (size_t)r * experts + e, v);   // read by another block of the same launch
+    }
+}
 // One wave per expert, up to 16 rows a launch.
 extern "C" __global__ void __launch_bounds__(64) ca_router_logits_rows(
     const uint16_t* __restrict__ x, const uint16_t* __restrict__ w, float* __restrict__ out, int rows, int hidden,
@@ -57,26 +104,49 @@ struct RouteParams {
     long long alt_token;          // token id that selects bias_alt, -1: none
 };
 
-// One wave routes one row.  Lane l holds experts l, l + 64, ... (at most 8 per lane: experts <= 512).  Every lane
-// returns the same ids / weights in registers [k]; topk <= 8.  COHERENT: the logits were written by other workgroups of this
-// launch (device-scope loads); otherwise by an earlier launch (plain loads).
-template <bool COHERENT>
-__device__ __forceinline__ void tf_route_row(const float* logits, const float* bias, int lane, const RouteParams& p,
+// Maximum of 64-bit keys (hi, lo) over the 64 lanes of a wave, in every lane (data-parallel primitives, as tf_wave_max).
+__device__ __forceinline__ void tf_wave_max_key(uint32_t& hi, uint32_t& lo) {
+#define TF_KEY_STEP(CTRL, ROWS, ALL)                                                                                          \
+    {                                                                                                                         \
+        const uint32_t ohi = (uint32_t)__builtin_amdgcn_update_dpp((ALL) ? 0 : (int)hi, (int)hi, CTRL, ROWS, 0xf, ALL);       \
+        const uint32_t olo = (uint32_t)__builtin_amdgcn_update_dpp((ALL) ? 0 : (int)lo, (int)lo, CTRL, ROWS, 0xf, ALL);       \
+        const bool take = ohi > hi || (ohi == hi && olo > lo);                                                                \
+        hi = take ? ohi : hi;                                                                                                 \
+        lo = take ? olo : lo;                                                                                                 \
+    }
+    TF_KEY_STEP(0xb1, 0xf, true)       // quad_perm [1,0,3,2]
+    TF_KEY_STEP(0x4e, 0xf, true)       // quad_perm [2,3,0,1]
+    TF_KEY_STEP(0x141, 0xf, true)      // row_half_mirror
+    TF_KEY_STEP(0x140, 0xf, true)      // row_mirror
+    TF_KEY_STEP(0x142, 0xa, false)     // row_bcast15 -> rows 1, 3
+    TF_KEY_STEP(0x143, 0xc, false)     // row_bcast31 -> rows 2, 3
+#undef TF_KEY_STEP
+    hi = (uint32_t)__builtin_amdgcn_readlane((int)hi, 63);
+    lo = (uint32_t)__builtin_amdgcn_readlane((int)lo, 63);
+}
+
+// One wave routes one row.  Lane l holds experts l, l + 64, ... (at most 8 per lane: experts <= 512): `x` their logits,
+// `b` their selection biases.  Every lane returns the same ids / weights in registers [k]; topk <= 8.
+// Selection = the k largest biased scores, ties to the lowest expert id (a NaN counts as +inf): each candidate is one 64-bit
+// key (the biased score's bits mapped to an unsigned order, then the complemented id), so a round is one wave maximum.
+__device__ __forceinline__ void tf_route_row(const float (&x)[8], const float (&b)[8], int lane, const RouteParams& p,
                                              int32_t* out_ids, float* out_weights) {
-    float score[8], biased[8];
+    float score[8];
+    uint32_t key[8];
 #pragma unroll
     for (int i = 0; i < 8; ++i) {
         const int e = i * 64 + lane;
         score[i] = 0.f;
-        biased[i] = -INFINITY;
+        key[i] = 0u;                                    // below every candidate: -inf maps to 0x007fffff
         if (e < p.experts) {
-            const float x = COHERENT ? tf_acquire_f32(logits + e) : logits[e];
             float s;
-            if (p.scoring == 1) s = __builtin_sqrtf(x > 20.f ? x : tf_log1p_pos(tf_exp(x)));
-            else s = tf_logistic(x);
-            const float v = __fadd_rn(s, bias[e]);
+            if (p.scoring == 1) s = __builtin_sqrtf(x[i] > 20.f ? x[i] : tf_log1p_pos(tf_exp(x[i])));
+            else s = tf_logistic(x[i]);
+            float v = __fadd_rn(s, b[i]);
+            v = (v == v) ? __fadd_rn(v, 0.f) : INFINITY;              // -0 -> +0: equal scores must have equal keys
+            const uint32_t u = __float_as_uint(v);
             score[i] = s;
-            biased[i] = (v == v) ? v : INFINITY;
+            key[i] = (u & 0x80000000u) ? ~u : (u | 0x80000000u);
         }
     }
     float w[8];
@@ -84,20 +154,20 @@ __device__ __forceinline__ void tf_route_row(const float* logits, const float* b
     for (int k = 0; k < 8; ++k) {
         w[k] = 0.f;
         if (k < p.topk) {
-            float best = -INFINITY;
+            uint32_t hi = 0u, lo = 0u;
 #pragma unroll
-            for (int i = 0; i < 8; ++i) best = fmaxf(best, biased[i]);
-            best = tf_wave_max(best);
-            int32_t winner = 0x7fffffff;
-#pragma unroll
-            for (int i = 0; i < 8; ++i)
-                if (i * 64 + lane < p.experts && biased[i] == best) winner = min(winner, i * 64 + lane);
-            winner = tf_wave_min(winner);
+            for (int i = 0; i < 8; ++i) {               // ids ascend with i: a later slot wins only with a larger score
+                const bool take = key[i] > hi;
+                hi = take ? key[i] : hi;
+                lo = take ? ~(uint32_t)(i * 64 + lane) : lo;
+            }
+            tf_wave_max_key(hi, lo);
+            const int32_t winner = (int32_t)~lo;
             float mine = 0.f;
 #pragma unroll
             for (int i = 0; i < 8; ++i)
-                if (i * 64 + lane == winner) { mine = score[i]; biased[i] = -INFINITY; }
-            w[k] = __shfl(mine, winner & 63);
+                if (i * 64 + lane == winner) { mine = score[i]; key[i] = 0u; }
+            w[k] = __int_as_float(__builtin_amdgcn_readlane(__float_as_int(mine), winner & 63));
             out_ids[k] = winner;
         }
     }
@@ -140,14 +210,33 @@ __device__ __forceinline__ void tf_route_block(const float* logits, const float*
                                                int first_row, int row_stride, bool apply_padding, int32_t* s_ids = nullptr,
                                                float* s_weights = nullptr, bool publish = false) {
     const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
-    const int n_live = min(rows, live[0]);
+    const int live_count = live[0];
+    const bool has_alt = bias_alt != nullptr && tokens != nullptr && p.alt_token >= 0;
     for (int row = first_row + wave; row < rows; row += row_stride) {
-        const bool is_live = row < n_live;
+        // everything the row needs is requested at once (one round trip): its logits, both biases, its token id; the live
+        // count requested above is first used below
+        float x[8], b0[8], b1[8];
+#pragma unroll
+        for (int i = 0; i < 8; ++i) {
+            const int e = i * 64 + lane;
+            x[i] = 0.f; b0[i] = 0.f; b1[i] = 0.f;
+            if (e < p.experts) {
+                const float* at = logits + (size_t)row * p.experts + e;
+                x[i] = COHERENT ? tf_acquire_f32(at) : *at;
+                b0[i] = bias[e];
+                if (has_alt) b1[i] = bias_alt[e];
+            }
+        }
+        const long long token = has_alt ? tokens[row] : -1;
+        const bool is_live = row < min(rows, live_count);
         int32_t chosen[8];
         float share[8];
         if (is_live) {
-            const bool alt = bias_alt != nullptr && tokens != nullptr && p.alt_token >= 0 && tokens[row] == p.alt_token;
-            tf_route_row<COHERENT>(logits + (size_t)row * p.experts, alt ? bias_alt : bias, lane, p, chosen, share);
+            if (has_alt && token == p.alt_token) {
+#pragma unroll
+                for (int i = 0; i < 8; ++i) b0[i] = b1[i];
+            }
+            tf_route_row(x, b0, lane, p, chosen, share);
         }
 #pragma unroll
         for (int k = 0; k < 8; ++k)
