@@ -106,7 +106,7 @@ class GpuLayer:
         self.live = z((1,), torch.int32)
         self.tokens = z((rows,), torch.int64)
         self.padding = torch.full((rows,), -1, dtype=torch.int32, device=d)
-        self.sync = z((1024,), torch.int32)
+        self.sync = z((1024 + 8 * 512,), torch.int32)      # arrival counters + the front-end's logit mailbox
 
     def _compact(self, src, kernel, n, k, unit_bytes, unit_elems, extra=None):
         src = src.contiguous()

@@ -65,7 +65,7 @@ def scratch_layout(g, rows):
              ("shared_scale_storage_ptr", rows * H // B), ("intermediate_ptr", padded * I * 2), ("intermediate_codes_ptr", padded * I),
              ("intermediate_scales_ptr", padded * I // B), ("task_expert_ptr", tiles * 4), ("task_valid_rows_ptr", tiles * 4),
              ("expert_tile_base", (g["experts"] + 1) * 4), ("token_map_ptr", padded * 4), ("token_weights_ptr", padded * 4),
-             ("scatter_ptr", pairs * H * 2), ("plan_scratch_ptr", ((pairs + 63) // 64 * g["experts"] + pairs) * 4), ("sync_ptr", 4096)]
+             ("scatter_ptr", pairs * H * 2), ("plan_scratch_ptr", ((pairs + 63) // 64 * g["experts"] + pairs) * 4), ("sync_ptr", 4096 + 8 * 512 * 4)]
     at, offsets = 0, {}
     for name, size in sizes:
         offsets[name] = at

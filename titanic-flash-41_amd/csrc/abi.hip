@@ -508,13 +508,13 @@ int64_t ca_primitives_scratch_bytes(void* context, int32_t index, int32_t rows) 
     auto add = [&](long long n) { bytes += (n + 255) / 256 * 256; };
     const long long H = g.hidden, I = g.intermediate, B = g.act_block;
     // the regions of the runtime contract, in its order, each aligned to 256 bytes: token codes and scales (routed flavour,
-    // shared flavour), intermediate (BF16, codes, scales), tile tables, row maps, route outputs, wide-plan scratch, sync word
+    // shared flavour), intermediate (BF16, codes, scales), tile tables, row maps, route outputs, wide-plan scratch, the front-end's sync region
     add(rows * H); add(rows * H / B); add(rows * H); add(rows * H / B);
     add(padded * I * 2); add(padded * I); add(padded * I / B);
     add(tiles * 4); add(tiles * 4); add((g.experts + 1) * 4ll); add(padded * 4); add(padded * 4);
     add(pairs * H * 2);
     add(((pairs + 63) / 64 * g.experts + pairs) * 4);
-    add(4096);
+    add(TF_SYNC_BYTES);
     return bytes;
 }
 

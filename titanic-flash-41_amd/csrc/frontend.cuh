@@ -4,6 +4,9 @@
 #pragma once
 #include "router.cuh"
 
+// The front-end's `sync` region: 4 KiB of arrival counters (128 bytes apart) + a mailbox of 8 rows x 512 experts words.
+#define TF_SYNC_BYTES (4096 + 8 * 512 * 4)
+
 // Quantizes 8 consecutive BF16 values held by each lane of a group of `block / 8` adjacent lanes (one quantization
 // block per group).  Returns the routed-flavour codes (zero block -> scale byte 0) and, when asked, the shared-flavour
 // ones (amax floored at 1e-4).
@@ -139,10 +142,13 @@ extern "C" __global__ void __launch_bounds__(512) ca_moe_frontend(
 }
 // The front-end with the router's top-k inside: block 0 first routes every owner row from the gate's logits (and
 // applies padding routes), then plans; the other blocks quantize meanwhile (launch one block more).
-// With `gate_w` the gate product runs here too: `logit_blocks` further blocks (one wave per expert and four rows) compute the logits,
-// publish them and count themselves in at `sync` (seventeen words, 128 bytes apart, zero before the first launch); block 0
-// waits for the counts, bounded: if they do not arrive it computes the logits itself, so the kernel always ends.  All blocks
-// of this small grid are resident together.
+// With `gate_w` the gate product runs here too: `logit_blocks` further blocks (one wave per expert and four rows) compute the
+// logits.  Owners of at most eight rows: the logits are handed to block 0 through a mailbox of one word a logit (`sync` +
+// 4 KiB: zero = empty; block 0 polls every word, takes the value and empties the word again), so neither side waits for a
+// store to complete or for a counter.  Larger owners: the blocks publish the logits and count themselves in at `sync`
+// (seventeen words, 128 bytes apart).  The whole `sync` region is zero before the first launch and every launch leaves it
+// zero.  Every wait is bounded: if the logits do not arrive block 0 computes them itself, so the kernel always ends.  All
+// blocks of this small grid are resident together.
 extern "C" __global__ void __launch_bounds__(512) ca_moe_route_frontend(
     const uint16_t* input, int32_t* ids, float* weights, uint8_t* packed, uint8_t* scales, int32_t* token_map,
     float* token_weights, int32_t* task_expert, int32_t* task_valid_rows, int32_t* expert_tile_base,
@@ -160,21 +166,18 @@ extern "C" __global__ void __launch_bounds__(512) ca_moe_route_frontend(
     // the whole owner instead of one per eight rows in block 0) and block 0 only collects, applies padding and plans.
     const int row_groups = (owner_rows + 3) >> 2, per_group = (experts + waves - 1) / waves;
     const bool distributed = gate_w != nullptr && row_groups > 2;
-    uint32_t* routed_groups = sync + 32 * 16;            // arrival words: 128 bytes apart; [0, 16) per row group or per lb % 8, [16] routed groups
+    uint32_t* routed_groups = sync + 32 * 16;            // arrival words: 128 bytes apart; [0, 16) per row group, [16] routed groups
+    uint32_t* mailbox = sync + 1024;                     // owners of at most eight rows: [row][expert], zero = empty
     if (gate_w != nullptr && (int)blockIdx.x >= first_logit_block) {
         const int lb = (int)blockIdx.x - first_logit_block, group = lb / per_group, e = (lb - group * per_group) * waves + wave;
         const int first_row = 4 * group;
         __shared__ u4v s_x[4096];                     // four token rows of at most 8,192 columns
         if (first_row < owner_rows)
             tf_logits_block(input + (size_t)first_row * cols, gate_w, logits + (size_t)first_row * experts, min(4, owner_rows - first_row), cols,
-                            experts, e, lane, s_x);
+                            experts, e, lane, s_x, distributed ? nullptr : mailbox + (size_t)first_row * experts);
+        if (!distributed) return;
         tf_stores_done();
         __syncthreads();
-        if (!distributed) {
-            // arrivals are spread over eight words: atomics on one address serialize
-            if (threadIdx.x == 0) atomicAdd(sync + 32 * (lb & 7), 1u);
-            return;
-        }
         __shared__ int last;
         if (threadIdx.x == 0) {
             last = atomicAdd(sync + 32 * group, 1u) == (uint32_t)(per_group - 1);
@@ -193,32 +196,42 @@ extern "C" __global__ void __launch_bounds__(512) ca_moe_route_frontend(
         bool routed = false;
         if (gate_w != nullptr) {
             __shared__ int arrived;
-            if (threadIdx.x < 64) {
-                int ok = 0;
-                if (distributed) {
+            __shared__ float s_logits[8 * 512];           // owners of at most eight rows: the logits taken from the mailbox
+            if (threadIdx.x == 0) arrived = 1;
+            __syncthreads();
+            if (distributed) {
+                if (threadIdx.x < 64) {
+                    int ok = 0;
                     for (int spin = 0; spin < (1 << 18); ++spin) {
                         if (__hip_atomic_load(routed_groups, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT) >= (uint32_t)row_groups) { ok = 1; break; }
                         __builtin_amdgcn_s_sleep(2);
                     }
                     if (lane == 0) __hip_atomic_store(routed_groups, 0u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
-                } else {                 // lanes 0 .. 7 of the first wave watch one arrival word each
-                    const int word = lane & 7;
-                    const uint32_t expected = (uint32_t)((logit_blocks - word + 7) >> 3);        // logit blocks lb with lb % 8 == word
-                    for (int spin = 0; spin < (1 << 18); ++spin) {
-                        const bool here = __hip_atomic_load(sync + 32 * word, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT) >= expected;
-                        if (__all(here)) { ok = 1; break; }
-                        __builtin_amdgcn_s_sleep(2);
-                    }
-                    if (lane < 8) __hip_atomic_store(sync + 32 * word, 0u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+                    if (lane == 0 && !ok) arrived = 0;
                 }
-                if (lane == 0) arrived = ok;
+            } else {
+                // every thread takes its words of the mailbox as they arrive and empties them for the next launch
+                for (int i = threadIdx.x; i < owner_rows * experts; i += blockDim.x) {
+                    uint32_t word = 0;
+                    for (int spin = 0; spin < (1 << 18); ++spin) {
+                        word = __hip_atomic_load(mailbox + i, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+                        if (word != 0u) break;
+                        __builtin_amdgcn_s_sleep(1);
+                    }
+                    if (word != 0u) {
+                        s_logits[i] = __uint_as_float(~word);
+                        __hip_atomic_store(mailbox + i, 0u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+                    } else {
+                        arrived = 0;
+                    }
+                }
             }
             __syncthreads();
-            if (!arrived)                // the bound expired: this block forms the logits (and routes) itself, so the kernel always ends
+            if (!arrived) {              // the bound expired: this block forms the logits (and routes) itself, so the kernel always ends
                 for (int e = wave; e < experts; e += waves) tf_logits_expert(input, gate_w, logits, owner_rows, cols, experts, e, lane);
-            tf_stores_done();
-            __syncthreads();
-            if (arrived && distributed) {
+                tf_stores_done();
+                __syncthreads();
+            } else if (distributed) {
                 // collect the groups' routes (written by other workgroups of this launch), then padding rows
                 for (int i = threadIdx.x; i < owner_rows * topk; i += blockDim.x) {
                     s_ids[i] = (int32_t)__hip_atomic_load(reinterpret_cast<const uint32_t*>(ids) + i, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
@@ -226,6 +239,9 @@ extern "C" __global__ void __launch_bounds__(512) ca_moe_route_frontend(
                 }
                 __syncthreads();
                 tf_apply_padding(padding, ids, weights, owner_rows, topk, s_ids, s_weights);
+                routed = true;
+            } else {
+                tf_route_block<false>(s_logits, bias, bias_alt, tokens, live, padding, ids, weights, owner_rows, p, 0, waves, true, s_ids, s_weights);
                 routed = true;
             }
         }

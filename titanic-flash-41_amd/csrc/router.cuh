@@ -48,8 +48,11 @@ __device__ __forceinline__ void tf_logits_expert(const uint16_t* __restrict__ x,
 // token rows.  One round trip: every lane requests its expert's whole row (hidden / 512 vectors) and the workgroup requests
 // the token rows once (instead of once a wave), which then go through LDS.  Same summation order as tf_logits_expert.
 // Block barrier inside; hidden <= 8192; `s_x` holds rows * hidden / 8 vectors (at most 4,096).
+// `mailbox` (may be null): the consumer polls these words instead of waiting for a counter: a word is zero while empty and
+// holds the complement of the logit's bits once written (no sum of BF16 products has all bits set: the low half of every
+// widened BF16 operand is zero and a NaN keeps an operand's payload).
 __device__ __forceinline__ void tf_logits_block(const uint16_t* __restrict__ x, const uint16_t* __restrict__ w, float* __restrict__ out,
-                                                int rows, int hidden, int experts, int e, int lane, u4v* s_x) {
+                                                int rows, int hidden, int experts, int e, int lane, u4v* s_x, uint32_t* mailbox = nullptr) {
     const int nj = hidden >> 9, per_row = hidden >> 3, total = rows * per_row;
     const bool on = e < experts;
     u4v wv[16], xr[8];
@@ -88,7 +91,14 @@ __device__ __forceinline__ void tf_logits_block(const uint16_t* __restrict__ x, 
         float v = acc[r];
 #pragma unroll
         for (int o = 32; o > 0; o >>= 1) v = __fadd_rn(v, __shfl_xor(v, o));
-        if (lane == 0 && r < rows) tf_publish_f32(out + (size_t)r * experts + e, v);   // read by another block of the same launch
+        if (lane == 0 && r < rows) {
+            if (mailbox != nullptr) {
+                out[(size_t)r * experts + e] = v;
+                tf_publish_u32(mailbox + (size_t)r * experts + e, ~__float_as_uint(v));
+            } else {
+                tf_publish_f32(out + (size_t)r * experts + e, v);   // read by another block of the same launch
+            }
+        }
     }
 }
 // One wave per expert, up to 16 rows a launch.

@@ -330,7 +330,7 @@ Workspace::Workspace(std::shared_ptr<const Native> native, size_t rows) : native
     add("token_map_ptr", padded * 4); add("token_weights_ptr", padded * 4);
     add("scatter_ptr", pairs * H * 2);
     add("plan_scratch_ptr", ((pairs + 63) / 64 * g.experts + pairs) * 4);
-    add("sync_ptr", 4096);
+    add("sync_ptr", 4096 + 8 * 512 * 4);           // arrival counters + the front-end's logit mailbox (8 rows x 512 experts words)
     scratch_ = Buffer<uint8_t>(at);
     scratch_.zero();                                                                                          // scratch_initializer "zero", src/moe.rs:440
     output_ = Buffer<uint16_t>(rows * H);
