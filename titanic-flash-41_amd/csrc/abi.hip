@@ -139,7 +139,9 @@ int launch_dynamic(const Context& c, bool route, const uint64_t* p, const int32_
             // with the gate weight (and a zeroed sync word) the gate product runs inside this launch too (owner rows <= 64)
             const bool gate = p[P_GATE_W] != 0;
             if (gate && (!p[P_SYNC] || owner > TF_STREAM_MAX_ROWS || g.hidden > 8192)) return -1;
-            const int logit_blocks = gate ? ((owner + 3) / 4) * ((g.experts + 7) / 8) : 0;     // per group of four rows: eight waves a block, one expert a wave
+            // per group of four rows: one expert a wave, eight waves a block (four for owners of at most eight rows)
+            const int row_groups = (owner + 3) / 4;
+            const int logit_blocks = gate ? row_groups * (row_groups > 2 ? (g.experts + 7) / 8 : (g.experts + 3) / 4) : 0;
             ca_moe_route_frontend<<<quant_blocks + 1 + logit_blocks, 512, 0, s>>>(
                 x, ids, weights, (uint8_t*)p[P_PACKED], (uint8_t*)p[P_SCALES], (int32_t*)p[P_TOKEN_MAP], (float*)p[P_TOKEN_WEIGHTS],
                 (int32_t*)p[P_TASK_EXPERT], (int32_t*)p[P_TASK_VALID], (int32_t*)p[P_TILE_BASE], (float*)p[P_LOGITS],

@@ -121,7 +121,7 @@ __device__ __forceinline__ void tf_frontend_run(const uint16_t* input, const int
                                                 int32_t* token_map, float* token_weights, int32_t* task_expert,
                                                 int32_t* task_valid_rows, int32_t* expert_tile_base, int rows, int topk,
                                                 int experts, int cols, int groups, int tile_m, int act_block, int first) {
-    __shared__ int32_t s_ids[1024];
+    __shared__ __attribute__((aligned(16))) int32_t s_ids[1024];
     __shared__ float s_weights[1024];
     if (blockIdx.x == 0)
         tf_plan_block(ids, weights, token_map, token_weights, task_expert, task_valid_rows, expert_tile_base,
@@ -156,22 +156,28 @@ extern "C" __global__ void __launch_bounds__(512) ca_moe_route_frontend(
     const int32_t* padding, int32_t rows, int32_t topk, int32_t experts, int32_t cols, int32_t groups, int32_t tile_m,
     int32_t owner_rows, int32_t act_block, uint8_t* packed_min, uint8_t* scales_min, int32_t scoring,
     float route_scale, long long alt_token, const uint16_t* gate_w, uint32_t* sync, int32_t logit_blocks) {
-    __shared__ int32_t s_ids[1024];
+    __shared__ __attribute__((aligned(16))) int32_t s_ids[1024];
     __shared__ float s_weights[1024];
+    // logit blocks: the token rows; block 0 (owners of at most eight rows): logits, biases, token ids, live count
+    __shared__ __attribute__((aligned(16))) uint8_t s_pool[65536];
     const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6, waves = blockDim.x >> 6;
     const int first_logit_block = (int)gridDim.x - logit_blocks;
     const RouteParams p{experts, topk, scoring, route_scale, alt_token};
     // Logit blocks are group-major: block lb works on row group lb / per_group (four rows), experts 8 (lb % per_group) ..
     // More than two row groups: the last block of a group to finish routes the group's rows itself (one routing round for
     // the whole owner instead of one per eight rows in block 0) and block 0 only collects, applies padding and plans.
-    const int row_groups = (owner_rows + 3) >> 2, per_group = (experts + waves - 1) / waves;
+    const int row_groups = (owner_rows + 3) >> 2;
     const bool distributed = gate_w != nullptr && row_groups > 2;
+    // experts a logit block takes: a wave each; owners of at most eight rows use four of the eight waves (one a SIMD: the
+    // product is bound by the vector pipe, and twice the blocks still fit the chip at once)
+    const int expert_waves = distributed ? waves : 4, per_group = (experts + expert_waves - 1) / expert_waves;
     uint32_t* routed_groups = sync + 32 * 16;            // arrival words: 128 bytes apart; [0, 16) per row group, [16] routed groups
     uint32_t* mailbox = sync + 1024;                     // owners of at most eight rows: [row][expert], zero = empty
     if (gate_w != nullptr && (int)blockIdx.x >= first_logit_block) {
-        const int lb = (int)blockIdx.x - first_logit_block, group = lb / per_group, e = (lb - group * per_group) * waves + wave;
+        const int lb = (int)blockIdx.x - first_logit_block, group = lb / per_group;
+        const int e = wave < expert_waves ? (lb - group * per_group) * expert_waves + wave : experts;
         const int first_row = 4 * group;
-        __shared__ u4v s_x[4096];                     // four token rows of at most 8,192 columns
+        u4v* s_x = reinterpret_cast<u4v*>(s_pool);    // four token rows of at most 8,192 columns
         if (first_row < owner_rows)
             tf_logits_block(input + (size_t)first_row * cols, gate_w, logits + (size_t)first_row * experts, min(4, owner_rows - first_row), cols,
                             experts, e, lane, s_x, distributed ? nullptr : mailbox + (size_t)first_row * experts);
@@ -196,7 +202,20 @@ extern "C" __global__ void __launch_bounds__(512) ca_moe_route_frontend(
         bool routed = false;
         if (gate_w != nullptr) {
             __shared__ int arrived;
-            __shared__ float s_logits[8 * 512];           // owners of at most eight rows: the logits taken from the mailbox
+            float* s_logits = reinterpret_cast<float*>(s_pool);                       // [8][512]
+            float* s_bias = s_logits + 8 * 512;                                       // [2][512]: bias, bias_alt
+            long long* s_tokens = reinterpret_cast<long long*>(s_bias + 2 * 512);    // [8]
+            int32_t* s_live = reinterpret_cast<int32_t*>(s_tokens + 8);
+            // what routing needs besides the logits is requested now and lands while the logits are awaited
+            const int t = threadIdx.x;
+            float my_bias = 0.f, my_alt = 0.f;
+            long long my_token = -1;
+            int32_t my_live = 0;
+            if (!distributed) {
+                if (t < experts) { my_bias = bias[t]; if (bias_alt != nullptr) my_alt = bias_alt[t]; }
+                if (t < owner_rows && tokens != nullptr) my_token = tokens[t];
+                if (t == 0) my_live = live[0];
+            }
             if (threadIdx.x == 0) arrived = 1;
             __syncthreads();
             if (distributed) {
@@ -225,6 +244,9 @@ extern "C" __global__ void __launch_bounds__(512) ca_moe_route_frontend(
                         arrived = 0;
                     }
                 }
+                if (t < experts) { s_bias[t] = my_bias; s_bias[512 + t] = my_alt; }
+                if (t < owner_rows) s_tokens[t] = my_token;
+                if (t == 0) *s_live = my_live;
             }
             __syncthreads();
             if (!arrived) {              // the bound expired: this block forms the logits (and routes) itself, so the kernel always ends
@@ -241,7 +263,8 @@ extern "C" __global__ void __launch_bounds__(512) ca_moe_route_frontend(
                 tf_apply_padding(padding, ids, weights, owner_rows, topk, s_ids, s_weights);
                 routed = true;
             } else {
-                tf_route_block<false>(s_logits, bias, bias_alt, tokens, live, padding, ids, weights, owner_rows, p, 0, waves, true, s_ids, s_weights);
+                tf_route_block<false>(s_logits, s_bias, bias_alt != nullptr ? s_bias + 512 : nullptr, tokens != nullptr ? s_tokens : nullptr, s_live,
+                                      padding, ids, weights, owner_rows, p, 0, waves, true, s_ids, s_weights);
                 routed = true;
             }
         }

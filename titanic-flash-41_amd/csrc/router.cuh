@@ -58,7 +58,7 @@ __device__ __forceinline__ void tf_logits_block(const uint16_t* __restrict__ x, 
     u4v wv[16], xr[8];
     const u4v* wrow = reinterpret_cast<const u4v*>(w + (size_t)(on ? e : 0) * hidden);
 #pragma unroll
-    for (int j = 0; j < 16; ++j) if (j < nj) wv[j] = wrow[j * 64 + lane];
+    for (int j = 0; j < 16; ++j) if (on && j < nj) wv[j] = wrow[j * 64 + lane];
 #pragma unroll
     for (int i = 0; i < 8; ++i) {
         const int v = (int)threadIdx.x + (int)blockDim.x * i;
@@ -139,12 +139,14 @@ __device__ __forceinline__ void tf_wave_max_key(uint32_t& hi, uint32_t& lo) {
 // `b` their selection biases.  Every lane returns the same ids / weights in registers [k]; topk <= 8.
 // Selection = the k largest biased scores, ties to the lowest expert id (a NaN counts as +inf): each candidate is one 64-bit
 // key (the biased score's bits mapped to an unsigned order, then the complemented id), so a round is one wave maximum.
+// SLOTS = 4 for at most 256 experts (half the scans of a round), else 8.
+template <int SLOTS>
 __device__ __forceinline__ void tf_route_row(const float (&x)[8], const float (&b)[8], int lane, const RouteParams& p,
                                              int32_t* out_ids, float* out_weights) {
-    float score[8];
-    uint32_t key[8];
+    float score[SLOTS];
+    uint32_t key[SLOTS];
 #pragma unroll
-    for (int i = 0; i < 8; ++i) {
+    for (int i = 0; i < SLOTS; ++i) {
         const int e = i * 64 + lane;
         score[i] = 0.f;
         key[i] = 0u;                                    // below every candidate: -inf maps to 0x007fffff
@@ -166,7 +168,7 @@ __device__ __forceinline__ void tf_route_row(const float (&x)[8], const float (&
         if (k < p.topk) {
             uint32_t hi = 0u, lo = 0u;
 #pragma unroll
-            for (int i = 0; i < 8; ++i) {               // ids ascend with i: a later slot wins only with a larger score
+            for (int i = 0; i < SLOTS; ++i) {           // ids ascend with i: a later slot wins only with a larger score
                 const bool take = key[i] > hi;
                 hi = take ? key[i] : hi;
                 lo = take ? ~(uint32_t)(i * 64 + lane) : lo;
@@ -175,7 +177,7 @@ __device__ __forceinline__ void tf_route_row(const float (&x)[8], const float (&
             const int32_t winner = (int32_t)~lo;
             float mine = 0.f;
 #pragma unroll
-            for (int i = 0; i < 8; ++i)
+            for (int i = 0; i < SLOTS; ++i)
                 if (i * 64 + lane == winner) { mine = score[i]; key[i] = 0u; }
             w[k] = __int_as_float(__builtin_amdgcn_readlane(__float_as_int(mine), winner & 63));
             out_ids[k] = winner;
@@ -246,7 +248,8 @@ __device__ __forceinline__ void tf_route_block(const float* logits, const float*
 #pragma unroll
                 for (int i = 0; i < 8; ++i) b0[i] = b1[i];
             }
-            tf_route_row(x, b0, lane, p, chosen, share);
+            if (p.experts <= 256) tf_route_row<4>(x, b0, lane, p, chosen, share);
+            else tf_route_row<8>(x, b0, lane, p, chosen, share);
         }
 #pragma unroll
         for (int k = 0; k < 8; ++k)
