@@ -282,3 +282,44 @@ def test_code_object_loads_and_resolves_every_kernel_by_name():
     want = oracle.ffn_add(u16(a), u16(b))
     assert np.array_equal(u16(out), want)
     assert hip.hipModuleUnload(module) == 0
+
+
+def test_format_conversions_match_the_oracle_on_every_rounding_boundary():
+    # every sign / exponent / leading-mantissa pattern with the low-bit patterns around each rounding boundary of both formats
+    # (E4M3 keeps 3 mantissa bits, BF16 keeps 7), the saturation range of E4M3, specials, and a million random bit patterns
+    hi = np.arange(1 << 16, dtype=np.uint32) << 16                       # sign, exponent, 7 mantissa bits
+    lows = np.array([0, 1, 0x7fff, 0x8000, 0x8001, 0xffff], np.uint32)
+    bits = [(hi[:, None] | lows[None, :]).ravel()]
+    top = np.arange(1 << 12, dtype=np.uint32) << 20                      # sign, exponent, 3 mantissa bits
+    low20 = np.array([0, 1, 0x7ffff, 0x80000, 0x80001, 0xfffff], np.uint32)
+    bits.append((top[:, None] | low20[None, :]).ravel())
+    around_448 = np.frombuffer(np.arange(440.0, 500.0, 0.125, dtype=np.float32).tobytes(), np.uint32)
+    bits += [around_448, around_448 | np.uint32(0x80000000)]
+    bits.append(np.random.default_rng(7).integers(0, 1 << 32, size=1 << 20, dtype=np.uint64).astype(np.uint32))
+    bits = np.concatenate(bits)
+    bits = bits[: len(bits) // 4 * 4]
+    values = bits.view(np.float32)
+    d_in = torch.from_numpy(values.copy()).cuda()
+    d8 = torch.zeros(len(bits), dtype=torch.uint8, device="cuda")
+    d16 = torch.zeros(len(bits), dtype=torch.int16, device="cuda")
+    native.launch("ca_convert_formats", 1024, 256, [d_in, d8, d16, ctypes.c_int64(len(bits))])
+    torch.cuda.synchronize()
+    L = oracle.lib()
+    want8 = np.array([L.orc_f32_to_e4m3(float(v)) if v == v else 0x7f for v in values[: 1 << 16]], np.uint8)
+    assert np.array_equal(np_of(d8)[: 1 << 16], want8)
+    # the whole set against numpy restatements of the two roundings (checked against the oracle on the first 65,536 above)
+    def e4m3_np(u):
+        sign, a = (u >> 24) & 0x80, u & 0x7fffffff
+        normal = np.minimum(((a.astype(np.uint64) + 0x7ffff + ((a >> 20) & 1)) >> 20).astype(np.int64) - 960, 0x7e)
+        tiny = (np.abs(u.view(np.float32)).astype(np.float32) + np.float32(24576.0)).view(np.uint32).astype(np.int64) - 0x46c00000
+        q = np.where(a < 0x3c800000, tiny, normal)
+        return np.where(a > 0x7f800000, 0x7f, sign | q).astype(np.uint8)
+    def bf16_np(u):
+        nan = (u & 0x7fffffff) > 0x7f800000
+        r = ((u.astype(np.uint64) + 0x7fff + ((u >> 16) & 1)) >> 16).astype(np.uint32)
+        return np.where(nan, (u >> 16) | 0x40, r).astype(np.uint16)
+    assert np.array_equal(e4m3_np(bits[: 1 << 16]), want8)
+    assert np.array_equal(np_of(d8), e4m3_np(bits))
+    assert np.array_equal(np_of(d16).view(np.uint16), bf16_np(bits))
+    want16 = np.array([L.orc_f32_to_bf16(float(v)) for v in values[: 1 << 16] if v == v], np.uint16)
+    assert np.array_equal(np_of(d16).view(np.uint16)[: 1 << 16][values[: 1 << 16] == values[: 1 << 16]], want16)

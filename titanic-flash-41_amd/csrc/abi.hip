@@ -339,7 +339,7 @@ const KernelName kKernels[] = {
     TF_KERNEL(ca_expert_expand_scales), TF_KERNEL(ca_dense_compact_fp8), TF_KERNEL(ca_moe_nibble_permute_words),
     TF_KERNEL(ca_expert_scale_code1), TF_KERNEL(ca_expert_scale_code1_check), TF_KERNEL(ca_expert_scale_code1_census),
     TF_KERNEL(ca_expert_scale_codes4), TF_KERNEL(ca_router_logits_mfma), TF_KERNEL(ca_codec_encode), TF_KERNEL(ca_codec_decode),
-    TF_KERNEL(ca_codec_pack_bf16), TF_KERNEL(ca_codec_unpack_routed), TF_KERNEL(ca_codec_local_live),
+    TF_KERNEL(ca_codec_pack_bf16), TF_KERNEL(ca_codec_unpack_routed), TF_KERNEL(ca_codec_local_live), TF_KERNEL(ca_convert_formats),
 };
 constexpr int kKernelCount = sizeof(kKernels) / sizeof(kKernels[0]);
 

@@ -165,3 +165,20 @@ extern "C" __global__ void ca_expert_scale_codes4(const uint8_t* source, uint8_t
         out[16 + n + (size_t)tile * 128 * (columns / 2) + (size_t)(pair / 2) * nr * 2 + r * 2 + pair % 2] = packed;
     }
 }
+
+// The number-format conversions alone (parity tests): E4M3 code and BF16 bits of every input.
+extern "C" __global__ void __launch_bounds__(256) ca_convert_formats(const float* __restrict__ in, uint8_t* __restrict__ e4m3,
+                                                                     uint16_t* __restrict__ bf16, long long n) {
+    for (long long i = (long long)blockIdx.x * blockDim.x + threadIdx.x; i < n; i += (long long)gridDim.x * blockDim.x) {
+        const float v = in[i];
+        e4m3[i] = (uint8_t)tf_to_e4m3(v);
+        bf16[i] = tf_to_bf16(v);
+        if ((i & 3) == 0 && i + 3 < n) {          // the four-value packer too: it must agree with the single conversions
+            const uint32_t w = tf_pack_e4m3(v, in[i + 1], in[i + 2], in[i + 3]);
+            if ((w & 0xffu) != tf_to_e4m3(v) || ((w >> 8) & 0xffu) != tf_to_e4m3(in[i + 1]) || ((w >> 16) & 0xffu) != tf_to_e4m3(in[i + 2]) ||
+                (w >> 24) != tf_to_e4m3(in[i + 3]))
+                bf16[i] = 0xdead;                 // no BF16 value of a test input: the test fails on it
+        }
+    }
+}
+
