@@ -356,16 +356,19 @@ __device__ __forceinline__ void tf_fc2_items(const StreamArgs& p, int item_first
             loaded_tile = r.tile;
         }
         if (item + 1 < item_last) load_unit(next, item + 1);
+        // the partial sums of consecutive items alternate between two sets of LDS slots, so one barrier an item is enough:
+        // a set is written again two items later, behind the next item's barrier
+        float (*set)[2][4][64] = red + (item & 1) * 8;
 #pragma unroll
         for (int t = 0; t < NT; ++t) {
             const v4f c = tf_dot_unit<FP8, 4, KS>(a, cur, t);
 #pragma unroll
-            for (int i = 0; i < 4; ++i) red[(t >> 1) * 4 + wave][t & 1][i][lane] = c[i];
+            for (int i = 0; i < 4; ++i) set[(t >> 1) * 4 + wave][t & 1][i][lane] = c[i];
         }
         __syncthreads();
         // wave w finishes 16-column tile w of the item (routed: 4 tiles; shared: 2)
         if (wave < NT) {
-            float (*slot)[2][4][64] = red + (wave >> 1) * 4;
+            float (*slot)[2][4][64] = set + (wave >> 1) * 4;
             const int which = wave & 1;
 #pragma unroll
             for (int i = 0; i < 4; ++i) {
@@ -383,7 +386,6 @@ __device__ __forceinline__ void tf_fc2_items(const StreamArgs& p, int item_first
                 }
             }
         }
-        __syncthreads();
         if (item + 1 < item_last) cur = next;
     }
 }
@@ -409,7 +411,7 @@ __global__ void __launch_bounds__(256, 2) tf_phase1_stream(const StreamArgs rout
 }
 template <int KSR, int KSS>
 __global__ void __launch_bounds__(256, 2) tf_phase2_stream(const StreamArgs routed, const StreamArgs shared) {
-    __shared__ float red[8][2][4][64];
+    __shared__ float red[16][2][4][64];
     extern __shared__ uint8_t dyn[];
     __shared__ PlanLds plan;
     if (routed.w) tf_plan_preload(routed, plan);
