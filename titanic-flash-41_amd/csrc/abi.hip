@@ -125,6 +125,12 @@ int launch_dynamic(const Context& c, bool route, const uint64_t* p, const int32_
     if (few ? tile_m != 16 : tile_m != TF_GEMM_TILE_M) return -1;
     if (few && max_tiles > TF_LDS_TILES) return -1;
 
+    StreamArgs sa{}, sb{};                 // few rows: the shared expert's two projections
+    if (sh && few) {
+        for (int i = 0; i < H_COUNT; ++i) if (!sh[i] && i != H_UP_TAP && i != H_ACT_CODES && i != H_ACT_SCALES) return -1;
+        if (!supported_k(g.shared_intermediate)) return -4;
+        shared_stream_args(c, sh, rows, sa, sb);
+    }
     mark(c, 0, s);
     const uint16_t* x = (const uint16_t*)p[P_A];
     int32_t* ids = (int32_t*)p[P_IDS];
@@ -141,7 +147,24 @@ int launch_dynamic(const Context& c, bool route, const uint64_t* p, const int32_
             if (gate && (!p[P_SYNC] || owner > TF_STREAM_MAX_ROWS || g.hidden > 8192)) return -1;
             // per group of four rows: one expert a wave, eight waves a block (four for owners of at most eight rows)
             const int row_groups = (owner + 3) / 4;
-            const int logit_blocks = gate ? row_groups * (row_groups > 2 ? (g.experts + 7) / 8 : (g.experts + 3) / 4) : 0;
+            int logit_blocks = gate ? row_groups * (row_groups > 2 ? (g.experts + 7) / 8 : (g.experts + 3) / 4) : 0;
+            // owners of at most eight rows: the shared expert's first projection streams in this launch, beside the front-end's
+            // chain of dependent steps, instead of lengthening the routed experts' first launch
+            const int shared_blocks = g.shared_intermediate / 16;          // one item a block
+            const int dense_logit_blocks = row_groups * ((g.experts + 7) / 8);
+            const bool early_shared = sa.w != nullptr && gate && owner <= 8 && g.hidden <= 4096 && (phases & 3) == 3 &&
+                                      quant_blocks + 1 + dense_logit_blocks + shared_blocks <= c.cus;    // all resident, one block a CU
+            if (early_shared) {
+                logit_blocks = dense_logit_blocks;
+                ca_moe_route_frontend_shared<<<quant_blocks + 1 + logit_blocks + shared_blocks, 512, 0, s>>>(
+                    x, ids, weights, (uint8_t*)p[P_PACKED], (uint8_t*)p[P_SCALES], (int32_t*)p[P_TOKEN_MAP], (float*)p[P_TOKEN_WEIGHTS],
+                    (int32_t*)p[P_TASK_EXPERT], (int32_t*)p[P_TASK_VALID], (int32_t*)p[P_TILE_BASE], (float*)p[P_LOGITS],
+                    (const float*)p[P_BIAS], (const float*)p[P_BIAS_ALT], (const long long*)p[P_TOKENS], (const int32_t*)p[P_LIVE],
+                    (const int32_t*)p[P_PADDING], rows, g.topk, g.experts, g.hidden, groups, tile_m, owner, g.act_block,
+                    (uint8_t*)p[P_PACKED_MIN], (uint8_t*)p[P_SCALES_MIN], g.scoring, g.route_scale, (long long)g.alt_token,
+                    (const uint16_t*)p[P_GATE_W], (uint32_t*)p[P_SYNC], logit_blocks, sa, shared_blocks);
+                sa.w = nullptr;            // done: the routed experts' first launch runs without it
+            } else
             ca_moe_route_frontend<<<quant_blocks + 1 + logit_blocks, 512, 0, s>>>(
                 x, ids, weights, (uint8_t*)p[P_PACKED], (uint8_t*)p[P_SCALES], (int32_t*)p[P_TOKEN_MAP], (float*)p[P_TOKEN_WEIGHTS],
                 (int32_t*)p[P_TASK_EXPERT], (int32_t*)p[P_TASK_VALID], (int32_t*)p[P_TILE_BASE], (float*)p[P_LOGITS],
@@ -191,12 +214,6 @@ int launch_dynamic(const Context& c, bool route, const uint64_t* p, const int32_
         a.k = g.hidden; a.inter = g.intermediate; a.hidden = g.hidden; a.act_block = g.act_block; a.limit = g.swiglu_limit;
         a.out = (uint16_t*)p[P_INTER];
         a.table_tiles = max_tiles;
-        StreamArgs sa{}, sb{};
-        if (sh) {
-            for (int i = 0; i < H_COUNT; ++i) if (!sh[i] && i != H_UP_TAP && i != H_ACT_CODES && i != H_ACT_SCALES) return -1;
-            if (!supported_k(g.shared_intermediate)) return -4;
-            shared_stream_args(c, sh, rows, sa, sb);
-        }
         StreamArgs b = a;
         b.a_codes = nullptr; b.a_scales = nullptr; b.a_bf16 = (const uint16_t*)p[P_INTER];
         b.q_codes = (uint8_t*)p[P_INTER_CODES]; b.q_scales = (uint8_t*)p[P_INTER_SCALES]; b.min_amax = 0.f;
@@ -332,7 +349,7 @@ struct KernelName { const char* name; const void* function; };
 #define TF_KERNEL(k) {#k, (const void*)k}
 const KernelName kKernels[] = {
     TF_KERNEL(ca_router_logits_rows), TF_KERNEL(ca_route_topk), TF_KERNEL(ca_route_padding_rows), TF_KERNEL(ca_route_census),
-    TF_KERNEL(ca_moe_frontend), TF_KERNEL(ca_moe_route_frontend), TF_KERNEL(ca_quantize_rows), TF_KERNEL(ca_plan_wave_counts),
+    TF_KERNEL(ca_moe_frontend), TF_KERNEL(ca_moe_route_frontend), TF_KERNEL(ca_moe_route_frontend_shared), TF_KERNEL(ca_quantize_rows), TF_KERNEL(ca_plan_wave_counts),
     TF_KERNEL(ca_plan_scan), TF_KERNEL(ca_plan_tiles), TF_KERNEL(ca_plan_scatter), TF_KERNEL(ca_shared_swiglu_rows), TF_KERNEL(ca_shared_swiglu_quant),
     TF_KERNEL(ca_ffn_add_rows), TF_KERNEL(ca_moe_topk_sum), TF_KERNEL(ca_ffn_sum_shared), TF_KERNEL(ca_moe_group_sum_rows),
     TF_KERNEL(ca_expert_compact_words), TF_KERNEL(ca_expert_expand_words), TF_KERNEL(ca_expert_compact_scales),

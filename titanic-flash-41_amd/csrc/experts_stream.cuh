@@ -423,3 +423,99 @@ __global__ void __launch_bounds__(256, 2) tf_phase2_stream(const StreamArgs rout
     if (lo < r_items) tf_fc2_items<false, KSR>(routed, (int)lo, (int)(hi < r_items ? hi : r_items), red, dyn, dyn + 16 * (size_t)kmax, plan);
     if (hi > r_items) tf_fc2_items<true, KSS>(shared, (int)(lo > r_items ? lo - r_items : 0), (int)(hi - r_items), red, dyn, dyn + 16 * (size_t)kmax, plan);
 }
+
+// The experts' front-end with the shared expert's first projection in the same launch (owners of at most eight rows, hidden <=
+// 4,096).  The front-end proper keeps a handful of workgroups busy for its whole length (gate product, routing, plan: a
+// chain of dependent steps) while the rest of the chip idles; the shared expert does not depend on the routing, so its
+// up / gate weights (two thirds of its bytes) stream here instead of inside the routed experts' first launch, whose length
+// they would add to.  `shared_blocks` = intermediate / 16 further blocks, one item (16 intermediate columns) each: the block
+// quantizes the token rows itself (shared flavour, into LDS: no dependency on the launch's quantizer blocks), waves 0 - 3
+// take the item's gate tile and waves 4 - 7 its up tile (a K quarter each), and wave 0 finishes the item as tf_fc1_items
+// does (same summation order, same activation).
+template <int KS>
+__device__ __forceinline__ void tf_front_shared_item(const StreamArgs& p, const uint16_t* __restrict__ input, int rows, uint8_t* s_pool, int item) {
+    const int k = p.k, per_row = k >> 3, group_lanes = p.act_block >> 3;
+    uint8_t* s_codes = s_pool;                                        // [rows][k]            (at most 32 KiB)
+    uint8_t* s_scales = s_pool + 8 * 4096;                            // [rows][k / act_block] (at most 1 KiB)
+    float (*red)[4][4][64] = reinterpret_cast<float (*)[4][4][64]>(s_pool + 8 * 4096 + 1024);      // [gate / up][wave][i][lane]
+    const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6, half = wave >> 2, quarter = wave & 3, ks_first = quarter * KS;
+    const int per_tile = p.inter / 16;
+    // the weights first: they come from HBM, the rows from L2
+    Unit<2, KS> u;
+    const int nt[2] = {half * per_tile + item, 0};
+    tf_load_fp8<2, KS>(u, p.w, p.ws, nt, k, ks_first, lane, p.bn, p.bk);
+    const int total = rows * per_row, padded = (total + 63) & ~63;
+    for (int q = threadIdx.x; q < padded; q += blockDim.x) {
+        const bool on = q < total;
+        float v[8];
+        if (on) {
+            const u4v wv = reinterpret_cast<const u4v*>(input)[q];
+#pragma unroll
+            for (int i = 0; i < 4; ++i) { v[2 * i] = tf_bf16_lo(wv[i]); v[2 * i + 1] = tf_bf16_hi(wv[i]); }
+        } else {
+#pragma unroll
+            for (int i = 0; i < 8; ++i) v[i] = 0.f;
+        }
+        const float amax = tf_group_amax(v, group_lanes);
+        if (!on) continue;
+        const Quant8 c = tf_quant8(v, amax, 1e-4f);
+        reinterpret_cast<u2v*>(s_codes)[q] = u2v{c.lo, c.hi};
+        if ((q & (group_lanes - 1)) == 0) s_scales[q / group_lanes] = (uint8_t)c.exponent;
+    }
+    __syncthreads();
+    ATile<KS> a;
+    tf_load_a<KS>(a, s_codes, s_scales, (lane & 15) < rows ? (lane & 15) : -1, k, p.act_block, ks_first, lane);
+    const v4f c = tf_dot_unit<true, 2, KS>(a, u, 0);
+#pragma unroll
+    for (int i = 0; i < 4; ++i) red[half][quarter][i][lane] = c[i];
+    __syncthreads();
+    if (wave != 0) return;
+#pragma unroll
+    for (int i = 0; i < 4; ++i) {
+        const int m = 4 * (lane >> 4) + i;
+        if (m < rows) {
+            float first = red[0][0][i][lane], second = red[1][0][i][lane];
+#pragma unroll
+            for (int w2 = 1; w2 < 4; ++w2) {
+                first = __fadd_rn(first, red[0][w2][i][lane]);
+                second = __fadd_rn(second, red[1][w2][i][lane]);
+            }
+            const uint16_t gb = tf_to_bf16(first), ub = tf_to_bf16(second);
+            if (p.tap != nullptr) {
+                p.tap[(size_t)m * 2 * p.inter + 16 * item + (lane & 15)] = gb;
+                p.tap[(size_t)m * 2 * p.inter + p.inter + 16 * item + (lane & 15)] = ub;
+            }
+            const float hi = tf_bf16(tf_to_bf16(p.limit)), lo = tf_bf16(tf_to_bf16(-p.limit));
+            const float g = fminf(tf_bf16(gb), hi);
+            const float up = fminf(fmaxf(tf_bf16(ub), lo), hi);
+            const float value = __fmul_rn(g / __fadd_rn(1.0f, tf_exp(-g)), up);
+            p.out[(size_t)m * p.inter + 16 * item + (lane & 15)] = tf_to_bf16(value);
+        }
+    }
+}
+extern "C" __global__ void __launch_bounds__(512) ca_moe_route_frontend_shared(
+    const uint16_t* input, int32_t* ids, float* weights, uint8_t* packed, uint8_t* scales, int32_t* token_map,
+    float* token_weights, int32_t* task_expert, int32_t* task_valid_rows, int32_t* expert_tile_base,
+    float* logits, const float* bias, const float* bias_alt, const long long* tokens, const int32_t* live,
+    const int32_t* padding, int32_t rows, int32_t topk, int32_t experts, int32_t cols, int32_t groups, int32_t tile_m,
+    int32_t owner_rows, int32_t act_block, uint8_t* packed_min, uint8_t* scales_min, int32_t scoring,
+    float route_scale, long long alt_token, const uint16_t* gate_w, uint32_t* sync, int32_t logit_blocks, const StreamArgs shared,
+    int32_t shared_blocks) {
+    __shared__ __attribute__((aligned(16))) uint8_t s_pool[TF_FRONT_POOL_BYTES];
+    const int grid_blocks = (int)gridDim.x - shared_blocks;
+    if ((int)blockIdx.x >= grid_blocks) {
+        const int block = (int)blockIdx.x - grid_blocks;
+        switch (shared.k) {
+            case 512: tf_front_shared_item<1>(shared, input, rows, s_pool, block); break;
+            case 1024: tf_front_shared_item<2>(shared, input, rows, s_pool, block); break;
+            case 2048: tf_front_shared_item<4>(shared, input, rows, s_pool, block); break;
+            case 4096: tf_front_shared_item<8>(shared, input, rows, s_pool, block); break;
+            default: break;
+        }
+        return;
+    }
+    tf_route_frontend(input, ids, weights, packed, scales, token_map, token_weights, task_expert, task_valid_rows, expert_tile_base, logits, bias,
+                      bias_alt, tokens, live, padding, rows, topk, experts, cols, groups, tile_m, owner_rows, act_block, packed_min, scales_min,
+                      scoring, route_scale, alt_token, gate_w, sync, logit_blocks, grid_blocks, s_pool);
+}
+

@@ -149,28 +149,31 @@ extern "C" __global__ void __launch_bounds__(512) ca_moe_frontend(
 // (seventeen words, 128 bytes apart).  The whole `sync` region is zero before the first launch and every launch leaves it
 // zero.  Every wait is bounded: if the logits do not arrive block 0 computes them itself, so the kernel always ends.  All
 // blocks of this small grid are resident together.
-extern "C" __global__ void __launch_bounds__(512) ca_moe_route_frontend(
+#define TF_FRONT_POOL_BYTES 69632          // 68 KiB: two workgroups of the front-end still share a CU
+// `grid_blocks`: the blocks of the launch that belong to the front-end (block ids [0, grid_blocks)); `s_pool`: TF_FRONT_POOL_BYTES
+// of LDS (logit blocks: the token rows; block 0 of owners of at most eight rows: logits, biases, token ids, live count).
+__device__ __forceinline__ void tf_route_frontend(
     const uint16_t* input, int32_t* ids, float* weights, uint8_t* packed, uint8_t* scales, int32_t* token_map,
     float* token_weights, int32_t* task_expert, int32_t* task_valid_rows, int32_t* expert_tile_base,
     float* logits, const float* bias, const float* bias_alt, const long long* tokens, const int32_t* live,
     const int32_t* padding, int32_t rows, int32_t topk, int32_t experts, int32_t cols, int32_t groups, int32_t tile_m,
     int32_t owner_rows, int32_t act_block, uint8_t* packed_min, uint8_t* scales_min, int32_t scoring,
-    float route_scale, long long alt_token, const uint16_t* gate_w, uint32_t* sync, int32_t logit_blocks) {
+    float route_scale, long long alt_token, const uint16_t* gate_w, uint32_t* sync, int32_t logit_blocks, int grid_blocks,
+    uint8_t* s_pool) {
     __shared__ __attribute__((aligned(16))) int32_t s_ids[1024];
     __shared__ float s_weights[1024];
-    // logit blocks: the token rows; block 0 (owners of at most eight rows): logits, biases, token ids, live count
-    __shared__ __attribute__((aligned(16))) uint8_t s_pool[65536];
     const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6, waves = blockDim.x >> 6;
-    const int first_logit_block = (int)gridDim.x - logit_blocks;
+    const int first_logit_block = grid_blocks - logit_blocks;
     const RouteParams p{experts, topk, scoring, route_scale, alt_token};
     // Logit blocks are group-major: block lb works on row group lb / per_group (four rows), experts 8 (lb % per_group) ..
     // More than two row groups: the last block of a group to finish routes the group's rows itself (one routing round for
     // the whole owner instead of one per eight rows in block 0) and block 0 only collects, applies padding and plans.
     const int row_groups = (owner_rows + 3) >> 2;
     const bool distributed = gate_w != nullptr && row_groups > 2;
-    // experts a logit block takes: a wave each; owners of at most eight rows use four of the eight waves (one a SIMD: the
-    // product is bound by the vector pipe, and twice the blocks still fit the chip at once)
-    const int expert_waves = distributed ? waves : 4, per_group = (experts + expert_waves - 1) / expert_waves;
+    // experts a logit block takes: a wave each; owners of at most eight rows may use four of the eight waves (one a SIMD: the
+    // product is bound by the vector pipe), when the launcher has the room for twice the blocks
+    const int expert_waves = !distributed && logit_blocks == row_groups * ((experts + 3) >> 2) ? 4 : waves;      // the launcher's choice
+    const int per_group = (experts + expert_waves - 1) / expert_waves;
     uint32_t* routed_groups = sync + 32 * 16;            // arrival words: 128 bytes apart; [0, 16) per row group, [16] routed groups
     uint32_t* mailbox = sync + 1024;                     // owners of at most eight rows: [row][expert], zero = empty
     if (gate_w != nullptr && (int)blockIdx.x >= first_logit_block) {
@@ -282,6 +285,18 @@ extern "C" __global__ void __launch_bounds__(512) ca_moe_route_frontend(
     const long long total = (long long)rows * (cols >> 3);
     tf_quantize_span(input, packed, scales, packed_min, scales_min, total, act_block,
                      (long long)(blockIdx.x - 1) * blockDim.x + threadIdx.x, (long long)(first_logit_block - 1) * blockDim.x);
+}
+extern "C" __global__ void __launch_bounds__(512) ca_moe_route_frontend(
+    const uint16_t* input, int32_t* ids, float* weights, uint8_t* packed, uint8_t* scales, int32_t* token_map,
+    float* token_weights, int32_t* task_expert, int32_t* task_valid_rows, int32_t* expert_tile_base,
+    float* logits, const float* bias, const float* bias_alt, const long long* tokens, const int32_t* live,
+    const int32_t* padding, int32_t rows, int32_t topk, int32_t experts, int32_t cols, int32_t groups, int32_t tile_m,
+    int32_t owner_rows, int32_t act_block, uint8_t* packed_min, uint8_t* scales_min, int32_t scoring,
+    float route_scale, long long alt_token, const uint16_t* gate_w, uint32_t* sync, int32_t logit_blocks) {
+    __shared__ __attribute__((aligned(16))) uint8_t s_pool[TF_FRONT_POOL_BYTES];
+    tf_route_frontend(input, ids, weights, packed, scales, token_map, token_weights, task_expert, task_valid_rows, expert_tile_base, logits, bias,
+                      bias_alt, tokens, live, padding, rows, topk, experts, cols, groups, tile_m, owner_rows, act_block, packed_min, scales_min,
+                      scoring, route_scale, alt_token, gate_w, sync, logit_blocks, (int)gridDim.x, s_pool);
 }
 // Row quantizer alone (any number of rows).
 extern "C" __global__ void __launch_bounds__(256) ca_quantize_rows(
