@@ -44,9 +44,9 @@ MFMA_FP8_PEAK_TFLOPS, MFMA_FP4_PEAK_TFLOPS = 5000.0, 10100.0
 # (rocprofv3 --pmc FETCH_SIZE, then WRITE_SIZE, on tf_layer_probe: the same geometry, rows and schedule with random operands;
 # each counter scaled by its reading for a 256 MiB copy kernel).  The line's `traffic` is this ratio times the algorithmic
 # bytes of this run's launches; None where no counter run exists for the configuration.
-TRAFFIC_OVER_ALGORITHMIC = {"c2": 1.008}
+TRAFFIC_OVER_ALGORITHMIC = {"c2": 1.0003}
 # Many rows: HBM bytes a launch of the routed FC1 kernel, measured the same way at the same number of rows.
-WIDE_TRAFFIC_BYTES = {"c4": 3.62e9, "c5": 8.41e9}
+WIDE_TRAFFIC_BYTES = {"c4": 3.61e9, "c5": 8.38e9}
 
 
 def make_inputs(synth, name, cfg, device, batches=BATCHES):
