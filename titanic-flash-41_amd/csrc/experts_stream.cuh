@@ -424,22 +424,26 @@ __global__ void __launch_bounds__(256, 2) tf_phase2_stream(const StreamArgs rout
     if (hi > r_items) tf_fc2_items<true, KSS>(shared, (int)(lo > r_items ? lo - r_items : 0), (int)(hi - r_items), red, dyn, dyn + 16 * (size_t)kmax, plan);
 }
 
-// The experts' front-end with the shared expert's first projection in the same launch (owners of at most eight rows, hidden <=
-// 4,096).  The front-end proper keeps a handful of workgroups busy for its whole length (gate product, routing, plan: a
-// chain of dependent steps) while the rest of the chip idles; the shared expert does not depend on the routing, so its
-// up / gate weights (two thirds of its bytes) stream here instead of inside the routed experts' first launch, whose length
-// they would add to.  `shared_blocks` = intermediate / 16 further blocks, one item (16 intermediate columns) each: the block
-// quantizes the token rows itself (shared flavour, into LDS: no dependency on the launch's quantizer blocks), waves 0 - 3
-// take the item's gate tile and waves 4 - 7 its up tile (a K quarter each), and wave 0 finishes the item as tf_fc1_items
-// does (same summation order, same activation).
+// The experts' front-end with the shared expert's first projection in the same launch (few-row owners, hidden <= 4,096).
+// The front-end proper keeps a handful of workgroups busy for its whole length (gate product, routing, plan: a chain of
+// dependent steps) while the rest of the chip idles, or idles again once the logit blocks are done; the shared expert does
+// not depend on the routing, so its up / gate weights (two thirds of its bytes) stream here instead of inside the routed
+// experts' first launch, whose length they would add to.  `shared_blocks` = row tiles x intermediate / 16 further blocks (the
+// highest block ids: dispatched last, they wait for nothing and nothing waits for them), one item (a 16-row tile x 16
+// intermediate columns) each: the block quantizes the tile's token rows itself (shared flavour, into LDS: no dependency on
+// the launch's quantizer blocks), waves 0 - 3 take the item's gate tile and waves 4 - 7 its up tile (a K quarter each), and
+// wave 0 finishes the item as tf_fc1_items does (same summation order, same activation).
 template <int KS>
-__device__ __forceinline__ void tf_front_shared_item(const StreamArgs& p, const uint16_t* __restrict__ input, int rows, uint8_t* s_pool, int item) {
+__device__ __forceinline__ void tf_front_shared_item(const StreamArgs& p, const uint16_t* __restrict__ all_rows, int all_row_count, uint8_t* s_pool,
+                                                     int block) {
     const int k = p.k, per_row = k >> 3, group_lanes = p.act_block >> 3;
-    uint8_t* s_codes = s_pool;                                        // [rows][k]            (at most 32 KiB)
-    uint8_t* s_scales = s_pool + 8 * 4096;                            // [rows][k / act_block] (at most 1 KiB)
-    float (*red)[4][4][64] = reinterpret_cast<float (*)[4][4][64]>(s_pool + 8 * 4096 + 1024);      // [gate / up][wave][i][lane]
+    const int per_tile = p.inter / 16, tile = block / per_tile, item = block - tile * per_tile;
+    const int rows = min(16, all_row_count - 16 * tile);                // of this tile
+    const uint16_t* input = all_rows + (size_t)tile * 16 * k;
+    uint8_t* s_codes = s_pool;                                        // [rows][k]             (at most 64 KiB)
+    uint8_t* s_scales = s_pool + 16 * 4096;                           // [rows][k / act_block] (at most 2 KiB)
+    float (*red)[4][4][64] = reinterpret_cast<float (*)[4][4][64]>(s_pool + 16 * 4096 + 2048);     // [gate / up][wave][i][lane]: 8 KiB
     const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6, half = wave >> 2, quarter = wave & 3, ks_first = quarter * KS;
-    const int per_tile = p.inter / 16;
     // the weights first: they come from HBM, the rows from L2
     Unit<2, KS> u;
     const int nt[2] = {half * per_tile + item, 0};
@@ -481,15 +485,16 @@ __device__ __forceinline__ void tf_front_shared_item(const StreamArgs& p, const 
                 second = __fadd_rn(second, red[1][w2][i][lane]);
             }
             const uint16_t gb = tf_to_bf16(first), ub = tf_to_bf16(second);
+            const size_t row = (size_t)(tile * 16 + m);
             if (p.tap != nullptr) {
-                p.tap[(size_t)m * 2 * p.inter + 16 * item + (lane & 15)] = gb;
-                p.tap[(size_t)m * 2 * p.inter + p.inter + 16 * item + (lane & 15)] = ub;
+                p.tap[row * 2 * p.inter + 16 * item + (lane & 15)] = gb;
+                p.tap[row * 2 * p.inter + p.inter + 16 * item + (lane & 15)] = ub;
             }
             const float hi = tf_bf16(tf_to_bf16(p.limit)), lo = tf_bf16(tf_to_bf16(-p.limit));
             const float g = fminf(tf_bf16(gb), hi);
             const float up = fminf(fmaxf(tf_bf16(ub), lo), hi);
             const float value = __fmul_rn(g / __fadd_rn(1.0f, tf_exp(-g)), up);
-            p.out[(size_t)m * p.inter + 16 * item + (lane & 15)] = tf_to_bf16(value);
+            p.out[row * p.inter + 16 * item + (lane & 15)] = tf_to_bf16(value);
         }
     }
 }

@@ -149,7 +149,7 @@ extern "C" __global__ void __launch_bounds__(512) ca_moe_frontend(
 // (seventeen words, 128 bytes apart).  The whole `sync` region is zero before the first launch and every launch leaves it
 // zero.  Every wait is bounded: if the logits do not arrive block 0 computes them itself, so the kernel always ends.  All
 // blocks of this small grid are resident together.
-#define TF_FRONT_POOL_BYTES 69632          // 68 KiB: two workgroups of the front-end still share a CU
+#define TF_FRONT_POOL_BYTES 77824          // 76 KiB: the shared expert's item blocks hold a 16-row tile's codes (64 KiB), scales and partial sums
 // `grid_blocks`: the blocks of the launch that belong to the front-end (block ids [0, grid_blocks)); `s_pool`: TF_FRONT_POOL_BYTES
 // of LDS (logit blocks: the token rows; block 0 of owners of at most eight rows: logits, biases, token ids, live count).
 __device__ __forceinline__ void tf_route_frontend(
