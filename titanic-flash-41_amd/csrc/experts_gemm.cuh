@@ -241,10 +241,12 @@ __global__ void __launch_bounds__(512) tf_gemm(const GemmArgs p) {
                                 const BFrag<FP8>& bj = b[u][j];
                                 if constexpr (FP8) {
                                     const v8i bv = v8i{(int)bj.lo[0], (int)bj.lo[1], (int)bj.lo[2], (int)bj.lo[3], (int)bj.hi[0], (int)bj.hi[1], (int)bj.hi[2], (int)bj.hi[3]};
-                                    acc[f][j] = __builtin_amdgcn_mfma_scale_f32_16x16x128_f8f6f4(a_now, bv, acc[f][j], 0, 0, 0, sa[f], 0, (int)sbk[u][j]);
+                                    if constexpr (FC1) acc[f][j] = __builtin_amdgcn_mfma_scale_f32_16x16x128_f8f6f4(bv, a_now, acc[f][j], 0, 0, 0, (int)sbk[u][j], 0, sa[f]);
+                                    else acc[f][j] = __builtin_amdgcn_mfma_scale_f32_16x16x128_f8f6f4(a_now, bv, acc[f][j], 0, 0, 0, sa[f], 0, (int)sbk[u][j]);
                                 } else {
                                     const v8i bv = v8i{(int)bj.lo[0], (int)bj.lo[1], (int)bj.lo[2], (int)bj.lo[3], 0, 0, 0, 0};
-                                    acc[f][j] = __builtin_amdgcn_mfma_scale_f32_16x16x128_f8f6f4(a_now, bv, acc[f][j], 0, 4, 0, sa[f], 0, (int)(sb[j] >> (8 * u)));
+                                    if constexpr (FC1) acc[f][j] = __builtin_amdgcn_mfma_scale_f32_16x16x128_f8f6f4(bv, a_now, acc[f][j], 4, 0, 0, (int)(sb[j] >> (8 * u)), 0, sa[f]);
+                                    else acc[f][j] = __builtin_amdgcn_mfma_scale_f32_16x16x128_f8f6f4(a_now, bv, acc[f][j], 0, 4, 0, sa[f], 0, (int)(sb[j] >> (8 * u)));
                                 }
                             }
                             // a use the optimizer cannot move: without it every product of the unrolled k-steps is sunk below the
@@ -272,83 +274,85 @@ __global__ void __launch_bounds__(512) tf_gemm(const GemmArgs p) {
         else main_loop(std::integral_constant<int, 0>{});
 
         // ---- epilogue --------------------------------------------------------------------------------------------------
-        // lane (g, r16) of fragment f holds rows 64 mh + 16 f + 4 g + i (i < 4) and, per weight tile j, column r16 of the tile
         if constexpr (FC1) {
+            // The weight tile is the instruction's first operand and the token fragment its second, so lane (g, r16) of product
+            // (f, j) holds tile row 64 mh + 16 f + r16 and the four consecutive columns 4 g + i (i < 4) of weight tile j: a lane
+            // packs its four values into one store (four E4M3 codes a word, four BF16 values a pair of words).
             const float hi_lim = tf_bf16(tf_to_bf16(p.limit)), lo_lim = tf_bf16(tf_to_bf16(-p.limit));
             float hv[4][2][4];
-            float amax[4][4];
+            float amax[4];
 #pragma unroll
-            for (int f = 0; f < 4; ++f)
+            for (int f = 0; f < 4; ++f) {
+                const int row = 64 * mh + 16 * f + r16;
+                float m = 0.f;
 #pragma unroll
-                for (int i = 0; i < 4; ++i) {
-                    float m = 0.f;
+                for (int j = 0; j < 2; ++j) {
+                    if (MODE == TF_GEMM_FC1_SHARED) {
+                        uint16_t gb[4], ub[4];
 #pragma unroll
-                    for (int j = 0; j < 2; ++j) {
-                        float value;
-                        if (MODE == TF_GEMM_FC1_SHARED) {
-                            const uint16_t gb = tf_to_bf16(acc[f][j][i]), ub = tf_to_bf16(acc[f][2 + j][i]);
-                            if (p.tap != nullptr && f < my_frags) {
-                                const int row = 64 * mh + 16 * f + 4 * g + i;
-                                if (row < valid) {
-                                    const size_t at = (size_t)(tile * 128 + row) * 2 * p.inter + ng * 128 + nq * 32 + j * 16 + r16;
-                                    p.tap[at] = gb;
-                                    p.tap[at + p.inter] = ub;
-                                }
-                            }
-                            const float gv = fminf(tf_bf16(gb), hi_lim), uv = fminf(fmaxf(tf_bf16(ub), lo_lim), hi_lim);
-                            value = __fmul_rn(gv / __fadd_rn(1.0f, tf_exp(-gv)), uv);
-                        } else {
-                            // routed experts: no bit-level definition of this step exists (the reference's is inside a binary), the
-                            // result is rounded to BF16 next; the many-row path takes the hardware exponential and reciprocal
-                            const float gv = fminf(acc[f][2 + j][i], p.limit), uv = fminf(p.limit, fmaxf(-p.limit, acc[f][j][i]));
-                            value = __fmul_rn(__fmul_rn(gv, tf_logistic_fast(gv)), uv);
+                        for (int i = 0; i < 4; ++i) { gb[i] = tf_to_bf16(acc[f][j][i]); ub[i] = tf_to_bf16(acc[f][2 + j][i]); }
+                        if (p.tap != nullptr && f < my_frags && row < valid) {
+                            const size_t at = (size_t)(tile * 128 + row) * 2 * p.inter + ng * 128 + nq * 32 + j * 16 + 4 * g;
+                            *reinterpret_cast<u2v*>(p.tap + at) = u2v{(uint32_t)gb[0] | ((uint32_t)gb[1] << 16), (uint32_t)gb[2] | ((uint32_t)gb[3] << 16)};
+                            *reinterpret_cast<u2v*>(p.tap + at + p.inter) = u2v{(uint32_t)ub[0] | ((uint32_t)ub[1] << 16), (uint32_t)ub[2] | ((uint32_t)ub[3] << 16)};
                         }
-                        value = tf_bf16(tf_to_bf16(value));
-                        hv[f][j][i] = value;
-                        m = fmaxf(m, fabsf(value));
+#pragma unroll
+                        for (int i = 0; i < 4; ++i) {
+                            const float gv = fminf(tf_bf16(gb[i]), hi_lim), uv = fminf(fmaxf(tf_bf16(ub[i]), lo_lim), hi_lim);
+                            hv[f][j][i] = tf_bf16(tf_to_bf16(__fmul_rn(gv / __fadd_rn(1.0f, tf_exp(-gv)), uv)));
+                        }
+                    } else {
+                        // routed experts: no bit-level definition of this step exists (the reference's is inside a binary), the
+                        // result is rounded to BF16 next; the many-row path takes the hardware exponential and reciprocal
+#pragma unroll
+                        for (int i = 0; i < 4; ++i) {
+                            const float gv = fminf(acc[f][2 + j][i], p.limit), uv = fminf(p.limit, fmaxf(-p.limit, acc[f][j][i]));
+                            hv[f][j][i] = tf_bf16(tf_to_bf16(__fmul_rn(__fmul_rn(gv, tf_logistic_fast(gv)), uv)));
+                        }
                     }
-                    amax[f][i] = tf_row16_max(m);
+#pragma unroll
+                    for (int i = 0; i < 4; ++i) m = fmaxf(m, fabsf(hv[f][j][i]));
                 }
+                // the row's 32 columns of this wave sit in the four lanes r16 + 16 g
+                m = fmaxf(m, __shfl_xor(m, 16));
+                amax[f] = fmaxf(m, __shfl_xor(m, 32));
+            }
             if (p.act_block == 128) {          // one scale per row and 128 columns: across the four column quarters
 #pragma unroll
-                for (int f = 0; f < 4; ++f)
-#pragma unroll
-                    for (int i = 0; i < 4; ++i) if (r16 == 0) s_amax[nq][64 * mh + 16 * f + 4 * g + i] = amax[f][i];
+                for (int f = 0; f < 4; ++f) if (g == 0) s_amax[nq][64 * mh + 16 * f + r16] = amax[f];
                 __syncthreads();
 #pragma unroll
-                for (int f = 0; f < 4; ++f)
-#pragma unroll
-                    for (int i = 0; i < 4; ++i) {
-                        const int row = 64 * mh + 16 * f + 4 * g + i;
-                        amax[f][i] = fmaxf(fmaxf(s_amax[0][row], s_amax[1][row]), fmaxf(s_amax[2][row], s_amax[3][row]));
-                    }
+                for (int f = 0; f < 4; ++f) {
+                    const int row = 64 * mh + 16 * f + r16;
+                    amax[f] = fmaxf(fmaxf(s_amax[0][row], s_amax[1][row]), fmaxf(s_amax[2][row], s_amax[3][row]));
+                }
             }
             const float min_amax = MODE == TF_GEMM_FC1_SHARED ? 1e-4f : 0.f;
 #pragma unroll
             for (int f = 0; f < 4; ++f) {
-                if (f < my_frags) {
+                const int row = 64 * mh + 16 * f + r16;
+                if (f < my_frags && row < valid) {
+                    const uint32_t exponent = tf_block_exponent(min_amax > 0.f ? fmaxf(amax[f], min_amax) : amax[f]);
+                    const float inv = tf_block_inverse(exponent);
+                    const size_t phys = (size_t)tile * 128 + row;
+                    const int col = ng * 128 + nq * 32 + 4 * g;
 #pragma unroll
-                    for (int i = 0; i < 4; ++i) {
-                        const int row = 64 * mh + 16 * f + 4 * g + i;
-                        if (row < valid) {
-                            const uint32_t exponent = tf_block_exponent(min_amax > 0.f ? fmaxf(amax[f][i], min_amax) : amax[f][i]);
-                            const float inv = tf_block_inverse(exponent);
-                            const size_t phys = (size_t)tile * 128 + row;
-                            const int col = ng * 128 + nq * 32 + r16;
-#pragma unroll
-                            for (int j = 0; j < 2; ++j) {
-                                p.h_codes[phys * p.inter + col + 16 * j] = (uint8_t)tf_to_e4m3(__fmul_rn(hv[f][j][i], inv));
-                                if (p.h_bf16 != nullptr) p.h_bf16[phys * p.inter + col + 16 * j] = tf_to_bf16(hv[f][j][i]);
-                            }
-                            if (r16 == 0) {
-                                if (p.act_block == 32) p.h_scales[phys * (p.inter / 32) + ng * 4 + nq] = (uint8_t)exponent;
-                                else if (nq == 0) p.h_scales[phys * (p.inter / 128) + ng] = (uint8_t)exponent;
-                            }
-                        }
+                    for (int j = 0; j < 2; ++j) {
+                        *reinterpret_cast<uint32_t*>(p.h_codes + phys * p.inter + col + 16 * j) =
+                            tf_pack_e4m3(__fmul_rn(hv[f][j][0], inv), __fmul_rn(hv[f][j][1], inv), __fmul_rn(hv[f][j][2], inv), __fmul_rn(hv[f][j][3], inv));
+                        if (p.h_bf16 != nullptr)
+                            *reinterpret_cast<u2v*>(p.h_bf16 + phys * p.inter + col + 16 * j) =
+                                u2v{tf_pack_bf16(hv[f][j][0], hv[f][j][1]), tf_pack_bf16(hv[f][j][2], hv[f][j][3])};
+                    }
+                    if (g == 0) {
+                        if (p.act_block == 32) p.h_scales[phys * (p.inter / 32) + ng * 4 + nq] = (uint8_t)exponent;
+                        else if (nq == 0) p.h_scales[phys * (p.inter / 128) + ng] = (uint8_t)exponent;
                     }
                 }
             }
         } else {
+            // the token fragment is the first operand here: lane (g, r16) of product (f, j) holds tile rows 64 mh + 16 f + 4 g + i
+            // (i < 4) and column r16 of weight tile j
 #pragma unroll
             for (int f = 0; f < 4; ++f) {
                 if (f < my_frags) {
