@@ -36,6 +36,7 @@ def run_case(rows, hidden, experts, topk, inter, shared, mode, live=None, paddin
     (3, 4096, 16, 1, 2048, 2048, "benchmark"),      # top-1
     (16, 2048, 64, 8, 1024, 512, "benchmark"),      # top-8, H 2048 / I 1024, another shared width
     (6, 1024, 384, 6, 512, 1024, "reference"),      # the reference's expert count and row count
+    (40, 2048, 64, 6, 1024, 1024, "reference"),     # three row tiles, the last partly filled: the shared expert's items take the rows' codes from the quantizer blocks of their launch
     (64, 1024, 32, 4, 512, 512, "reference"),       # the last row count of the streaming path
     (65, 1024, 32, 4, 512, 512, "benchmark"),       # the first of the grouped-GEMM path
     (130, 2048, 16, 2, 1024, 1024, "reference"),    # a second, partly filled row tile; K 1024 in FC2

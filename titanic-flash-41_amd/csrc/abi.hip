@@ -150,7 +150,7 @@ int launch_dynamic(const Context& c, bool route, const uint64_t* p, const int32_
             int logit_blocks = gate ? row_groups * (row_groups > 2 ? (g.experts + 7) / 8 : (g.experts + 3) / 4) : 0;
             // hidden <= 4,096: the shared expert's first projection streams in this launch, beside the front-end's chain of
             // dependent steps, instead of lengthening the routed experts' first launch
-            const int shared_blocks = ((rows + 15) / 16) * (g.shared_intermediate / 16);          // one item (row tile x 16 columns) a block
+            const int shared_blocks = g.shared_intermediate / 16;          // one item (16 columns, every row tile) a block
             const int dense_logit_blocks = row_groups * ((g.experts + 7) / 8);
             const bool early_shared = sa.w != nullptr && gate && g.hidden <= 4096 && (phases & 3) == 3;
             if (early_shared) {

@@ -55,6 +55,29 @@ __device__ __forceinline__ void tf_load_a(ATile<KSMAX>& t, const uint8_t* codes,
     }
 }
 
+// The same from global memory that other workgroups of this launch have published (device-scope loads).
+template <int KS, int KSMAX = KS>
+__device__ __forceinline__ void tf_load_a_acquire(ATile<KSMAX>& t, const uint8_t* codes, const uint8_t* scales, long long row, int k,
+                                                  int act_block, int ks_first, int lane) {
+    const int g = lane >> 4;
+#pragma unroll
+    for (int q = 0; q < (KS + 3) / 4; ++q) t.scale[q] = 0x7f7f7f7fu;
+#pragma unroll
+    for (int s = 0; s < KS; ++s) {
+        const int ks = ks_first + s;
+        if (row >= 0) {
+            const uint8_t* base = codes + row * k + ks * 128 + 16 * g;
+            const u4v lo = tf_acquire_u4v(reinterpret_cast<const u4v*>(base));
+            const u4v hi = tf_acquire_u4v(reinterpret_cast<const u4v*>(base + 64));
+            t.a[s] = v8i{(int)lo[0], (int)lo[1], (int)lo[2], (int)lo[3], (int)hi[0], (int)hi[1], (int)hi[2], (int)hi[3]};
+            const uint32_t byte = __hip_atomic_load(scales + row * (k / act_block) + (ks * 128 + 32 * g) / act_block, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+            t.scale[s >> 2] = (t.scale[s >> 2] & ~(0xffu << (8 * (s & 3)))) | (byte << (8 * (s & 3)));
+        } else {
+            t.a[s] = v8i{0, 0, 0, 0, 0, 0, 0, 0};
+        }
+    }
+}
+
 // One pipeline unit of streamed weights for this wave: N 16-byte loads a lane (N KiB a wave).
 //   FP4 (routed): TILES weight tiles of 16 rows, KS k-steps each: d[t * KS + s].
 //   FP8 (shared): TILES / 2 weight tiles, each k-step as two 16-byte planes: d[(t * KS + s) * 2 + half].
@@ -428,76 +451,112 @@ __global__ void __launch_bounds__(256, 2) tf_phase2_stream(const StreamArgs rout
 // The front-end proper keeps a handful of workgroups busy for its whole length (gate product, routing, plan: a chain of
 // dependent steps) while the rest of the chip idles, or idles again once the logit blocks are done; the shared expert does
 // not depend on the routing, so its up / gate weights (two thirds of its bytes) stream here instead of inside the routed
-// experts' first launch, whose length they would add to.  `shared_blocks` = row tiles x intermediate / 16 further blocks (the
-// highest block ids: dispatched last, they wait for nothing and nothing waits for them), one item (a 16-row tile x 16
-// intermediate columns) each: the block quantizes the tile's token rows itself (shared flavour, into LDS: no dependency on
-// the launch's quantizer blocks), waves 0 - 3 take the item's gate tile and waves 4 - 7 its up tile (a K quarter each), and
-// wave 0 finishes the item as tf_fc1_items does (same summation order, same activation).
-template <int KS>
+// experts' first launch, whose length they would add to.  `shared_blocks` = intermediate / 16 further blocks (the highest
+// block ids: dispatched last; nothing waits for them), one item (16 intermediate columns, every row tile of the owner) each:
+// waves 0 - 3 take the item's gate tile and waves 4 - 7 its up tile (a K quarter each), loaded once; per row tile the block
+// takes the token rows' codes (shared flavour) -- one row tile: it quantizes the few rows itself, into LDS, and waits for
+// nobody; more: from the launch's quantizer blocks -- and wave 0 finishes the tile as tf_fc1_items does (same summation
+// order, same activation).
+template <int KS, bool HANDOFF>
 __device__ __forceinline__ void tf_front_shared_item(const StreamArgs& p, const uint16_t* __restrict__ all_rows, int all_row_count, uint8_t* s_pool,
-                                                     int block) {
+                                                     int item, uint32_t* sync, int quant_blocks, int shared_blocks) {
     const int k = p.k, per_row = k >> 3, group_lanes = p.act_block >> 3;
-    const int per_tile = p.inter / 16, tile = block / per_tile, item = block - tile * per_tile;
-    const int rows = min(16, all_row_count - 16 * tile);                // of this tile
-    const uint16_t* input = all_rows + (size_t)tile * 16 * k;
+    const int per_tile = p.inter / 16, tiles = (all_row_count + 15) >> 4;
     uint8_t* s_codes = s_pool;                                        // [rows][k]             (at most 64 KiB)
     uint8_t* s_scales = s_pool + 16 * 4096;                           // [rows][k / act_block] (at most 2 KiB)
-    float (*red)[4][4][64] = reinterpret_cast<float (*)[4][4][64]>(s_pool + 16 * 4096 + 2048);     // [gate / up][wave][i][lane]: 8 KiB
+    // [row tile parity][gate / up][wave][i][lane]: 2 x 8 KiB; consecutive row tiles alternate, so one barrier a tile is enough
+    float (*red)[2][4][4][64] = reinterpret_cast<float (*)[2][4][4][64]>(s_pool + 16 * 4096 + 2048);
     const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6, half = wave >> 2, quarter = wave & 3, ks_first = quarter * KS;
-    // the weights first: they come from HBM, the rows from L2
+    // `quant_blocks` > 0: the launch's quantizer blocks publish the rows' codes (shared flavour) and count themselves in; this
+    // block waits for all of them (a bounded wait: they have lower block ids, none of them waits for anything) and reads its
+    // operand from their output instead of quantizing every row again.  Should the bound expire it quantizes them itself.
+    // The wait comes before the first weight request: a workgroup barrier waits for every load in flight.
+    bool ready = false;
+    if constexpr (HANDOFF) {
+        __shared__ int s_ready;
+        if (threadIdx.x == 0) {
+            int ok = 0;
+            for (int spin = 0; spin < (1 << 18); ++spin) {
+                if (__hip_atomic_load(sync + 32 * TF_SYNC_QUANT_DONE, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT) >= (uint32_t)quant_blocks) { ok = 1; break; }
+                __builtin_amdgcn_s_sleep(2);
+            }
+            s_ready = ok;
+        }
+        __syncthreads();
+        ready = s_ready != 0;
+    }
+    // the weights first: they come from HBM, the rows from L2; every row tile of the owner uses them
     Unit<2, KS> u;
     const int nt[2] = {half * per_tile + item, 0};
     tf_load_fp8<2, KS>(u, p.w, p.ws, nt, k, ks_first, lane, p.bn, p.bk);
-    const int total = rows * per_row, padded = (total + 63) & ~63;
-    for (int q = threadIdx.x; q < padded; q += blockDim.x) {
-        const bool on = q < total;
-        float v[8];
-        if (on) {
-            const u4v wv = reinterpret_cast<const u4v*>(input)[q];
-#pragma unroll
-            for (int i = 0; i < 4; ++i) { v[2 * i] = tf_bf16_lo(wv[i]); v[2 * i + 1] = tf_bf16_hi(wv[i]); }
+    for (int tile = 0; tile < tiles; ++tile) {
+        const int rows = min(16, all_row_count - 16 * tile);                // of this tile
+        ATile<KS> a;
+        if (HANDOFF && ready) {
+            tf_load_a_acquire<KS>(a, p.a_codes + (size_t)tile * 16 * k, p.a_scales + (size_t)tile * 16 * (k / p.act_block),
+                                  (lane & 15) < rows ? (lane & 15) : -1, k, p.act_block, ks_first, lane);
         } else {
+            // (the previous tile's operand left LDS before that tile's barrier below)
+            const uint16_t* input = all_rows + (size_t)tile * 16 * k;
+            const int total = rows * per_row, padded = (total + 63) & ~63;
+            for (int q = threadIdx.x; q < padded; q += blockDim.x) {
+                const bool on = q < total;
+                float v[8];
+                if (on) {
+                    const u4v wv = reinterpret_cast<const u4v*>(input)[q];
 #pragma unroll
-            for (int i = 0; i < 8; ++i) v[i] = 0.f;
+                    for (int i = 0; i < 4; ++i) { v[2 * i] = tf_bf16_lo(wv[i]); v[2 * i + 1] = tf_bf16_hi(wv[i]); }
+                } else {
+#pragma unroll
+                    for (int i = 0; i < 8; ++i) v[i] = 0.f;
+                }
+                const float amax = tf_group_amax(v, group_lanes);
+                if (!on) continue;
+                const Quant8 c = tf_quant8(v, amax, 1e-4f);
+                reinterpret_cast<u2v*>(s_codes)[q] = u2v{c.lo, c.hi};
+                if ((q & (group_lanes - 1)) == 0) s_scales[q / group_lanes] = (uint8_t)c.exponent;
+            }
+            __syncthreads();
+            tf_load_a<KS>(a, s_codes, s_scales, (lane & 15) < rows ? (lane & 15) : -1, k, p.act_block, ks_first, lane);
         }
-        const float amax = tf_group_amax(v, group_lanes);
-        if (!on) continue;
-        const Quant8 c = tf_quant8(v, amax, 1e-4f);
-        reinterpret_cast<u2v*>(s_codes)[q] = u2v{c.lo, c.hi};
-        if ((q & (group_lanes - 1)) == 0) s_scales[q / group_lanes] = (uint8_t)c.exponent;
+        const v4f c = tf_dot_unit<true, 2, KS>(a, u, 0);
+        float (*set)[4][4][64] = red[tile & 1];
+#pragma unroll
+        for (int i = 0; i < 4; ++i) set[half][quarter][i][lane] = c[i];
+        __syncthreads();
+        if (wave != 0) continue;
+#pragma unroll
+        for (int i = 0; i < 4; ++i) {
+            const int m = 4 * (lane >> 4) + i;
+            if (m < rows) {
+                float first = set[0][0][i][lane], second = set[1][0][i][lane];
+#pragma unroll
+                for (int w2 = 1; w2 < 4; ++w2) {
+                    first = __fadd_rn(first, set[0][w2][i][lane]);
+                    second = __fadd_rn(second, set[1][w2][i][lane]);
+                }
+                const uint16_t gb = tf_to_bf16(first), ub = tf_to_bf16(second);
+                const size_t row = (size_t)(tile * 16 + m);
+                if (p.tap != nullptr) {
+                    p.tap[row * 2 * p.inter + 16 * item + (lane & 15)] = gb;
+                    p.tap[row * 2 * p.inter + p.inter + 16 * item + (lane & 15)] = ub;
+                }
+                const float hi = tf_bf16(tf_to_bf16(p.limit)), lo = tf_bf16(tf_to_bf16(-p.limit));
+                const float g = fminf(tf_bf16(gb), hi);
+                const float up = fminf(fmaxf(tf_bf16(ub), lo), hi);
+                const float value = __fmul_rn(g / __fadd_rn(1.0f, tf_exp(-g)), up);
+                p.out[row * p.inter + 16 * item + (lane & 15)] = tf_to_bf16(value);
+            }
+        }
     }
-    __syncthreads();
-    ATile<KS> a;
-    tf_load_a<KS>(a, s_codes, s_scales, (lane & 15) < rows ? (lane & 15) : -1, k, p.act_block, ks_first, lane);
-    const v4f c = tf_dot_unit<true, 2, KS>(a, u, 0);
-#pragma unroll
-    for (int i = 0; i < 4; ++i) red[half][quarter][i][lane] = c[i];
-    __syncthreads();
-    if (wave != 0) return;
-#pragma unroll
-    for (int i = 0; i < 4; ++i) {
-        const int m = 4 * (lane >> 4) + i;
-        if (m < rows) {
-            float first = red[0][0][i][lane], second = red[1][0][i][lane];
-#pragma unroll
-            for (int w2 = 1; w2 < 4; ++w2) {
-                first = __fadd_rn(first, red[0][w2][i][lane]);
-                second = __fadd_rn(second, red[1][w2][i][lane]);
-            }
-            const uint16_t gb = tf_to_bf16(first), ub = tf_to_bf16(second);
-            const size_t row = (size_t)(tile * 16 + m);
-            if (p.tap != nullptr) {
-                p.tap[row * 2 * p.inter + 16 * item + (lane & 15)] = gb;
-                p.tap[row * 2 * p.inter + p.inter + 16 * item + (lane & 15)] = ub;
-            }
-            const float hi = tf_bf16(tf_to_bf16(p.limit)), lo = tf_bf16(tf_to_bf16(-p.limit));
-            const float g = fminf(tf_bf16(gb), hi);
-            const float up = fminf(fmaxf(tf_bf16(ub), lo), hi);
-            const float value = __fmul_rn(g / __fadd_rn(1.0f, tf_exp(-g)), up);
-            p.out[row * p.inter + 16 * item + (lane & 15)] = tf_to_bf16(value);
-        }
+    // every wave's operands have been consumed (the last tile's barrier): the last item block to get here empties both arrival
+    // words for the next launch
+    if (HANDOFF && threadIdx.x == 0 && atomicAdd(sync + 32 * TF_SYNC_SHARED_PASSED, 1u) == (uint32_t)(shared_blocks - 1)) {
+        __hip_atomic_store(sync + 32 * TF_SYNC_QUANT_DONE, 0u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+        __hip_atomic_store(sync + 32 * TF_SYNC_SHARED_PASSED, 0u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
     }
 }
+
 extern "C" __global__ void __launch_bounds__(512) ca_moe_route_frontend_shared(
     const uint16_t* input, int32_t* ids, float* weights, uint8_t* packed, uint8_t* scales, int32_t* token_map,
     float* token_weights, int32_t* task_expert, int32_t* task_valid_rows, int32_t* expert_tile_base,
@@ -508,19 +567,33 @@ extern "C" __global__ void __launch_bounds__(512) ca_moe_route_frontend_shared(
     int32_t shared_blocks) {
     __shared__ __attribute__((aligned(16))) uint8_t s_pool[TF_FRONT_POOL_BYTES];
     const int grid_blocks = (int)gridDim.x - shared_blocks;
+    // more than one row tile: the item blocks take the rows' codes from the launch's quantizer blocks (one tile: they quantize the
+    // few rows themselves and wait for nobody)
+    const bool handoff = rows > 16 && packed_min != nullptr && scales_min != nullptr && shared.a_codes == packed_min && shared.a_scales == scales_min;
     if ((int)blockIdx.x >= grid_blocks) {
         const int block = (int)blockIdx.x - grid_blocks;
-        switch (shared.k) {
-            case 512: tf_front_shared_item<1>(shared, input, rows, s_pool, block); break;
-            case 1024: tf_front_shared_item<2>(shared, input, rows, s_pool, block); break;
-            case 2048: tf_front_shared_item<4>(shared, input, rows, s_pool, block); break;
-            case 4096: tf_front_shared_item<8>(shared, input, rows, s_pool, block); break;
-            default: break;
+        const int quant_blocks = grid_blocks - logit_blocks - 1;
+        if (handoff) {
+            switch (shared.k) {
+                case 512: tf_front_shared_item<1, true>(shared, input, rows, s_pool, block, sync, quant_blocks, shared_blocks); break;
+                case 1024: tf_front_shared_item<2, true>(shared, input, rows, s_pool, block, sync, quant_blocks, shared_blocks); break;
+                case 2048: tf_front_shared_item<4, true>(shared, input, rows, s_pool, block, sync, quant_blocks, shared_blocks); break;
+                case 4096: tf_front_shared_item<8, true>(shared, input, rows, s_pool, block, sync, quant_blocks, shared_blocks); break;
+                default: break;
+            }
+        } else {
+            switch (shared.k) {
+                case 512: tf_front_shared_item<1, false>(shared, input, rows, s_pool, block, sync, 0, shared_blocks); break;
+                case 1024: tf_front_shared_item<2, false>(shared, input, rows, s_pool, block, sync, 0, shared_blocks); break;
+                case 2048: tf_front_shared_item<4, false>(shared, input, rows, s_pool, block, sync, 0, shared_blocks); break;
+                case 4096: tf_front_shared_item<8, false>(shared, input, rows, s_pool, block, sync, 0, shared_blocks); break;
+                default: break;
+            }
         }
         return;
     }
     tf_route_frontend(input, ids, weights, packed, scales, token_map, token_weights, task_expert, task_valid_rows, expert_tile_base, logits, bias,
                       bias_alt, tokens, live, padding, rows, topk, experts, cols, groups, tile_m, owner_rows, act_block, packed_min, scales_min,
-                      scoring, route_scale, alt_token, gate_w, sync, logit_blocks, grid_blocks, s_pool);
+                      scoring, route_scale, alt_token, gate_w, sync, logit_blocks, grid_blocks, s_pool, handoff);
 }
 

@@ -32,10 +32,11 @@ __device__ __forceinline__ float tf_group_amax(const float (&v)[8], int group_la
 }
 // Quantizes `rows` x `cols` BF16 values in blocks of `block` (32 or 128) columns.  Work item = 8 values; items are
 // dealt to threads [first, first + count) of a virtual 1-D thread space with stride `stride`.
+// `publish_min`: the floored flavour is written with device-scope stores, for readers in other workgroups of the same launch.
 __device__ __forceinline__ void tf_quantize_span(const uint16_t* __restrict__ input, uint8_t* __restrict__ codes,
                                                  uint8_t* __restrict__ scales, uint8_t* __restrict__ codes_min,
                                                  uint8_t* __restrict__ scales_min, long long total_items,
-                                                 int block, long long thread, long long stride) {
+                                                 int block, long long thread, long long stride, bool publish_min = false) {
     const int group_lanes = block >> 3;
     // Whole groups stay together: thread and stride are multiples of 64 apart across waves, group_lanes divides 64.
     const long long padded = (total_items + 63) & ~63ll;
@@ -59,8 +60,14 @@ __device__ __forceinline__ void tf_quantize_span(const uint16_t* __restrict__ in
         }
         if (codes_min != nullptr) {
             const Quant8 b = tf_quant8(v, amax, 1e-4f);
-            reinterpret_cast<u2v*>(codes_min)[q] = u2v{b.lo, b.hi};
-            if ((q & (group_lanes - 1)) == 0) scales_min[q / group_lanes] = (uint8_t)b.exponent;
+            if (publish_min) {
+                __hip_atomic_store(reinterpret_cast<unsigned long long*>(codes_min) + q, (unsigned long long)b.lo | ((unsigned long long)b.hi << 32),
+                                   __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+                if ((q & (group_lanes - 1)) == 0) __hip_atomic_store(scales_min + q / group_lanes, (uint8_t)b.exponent, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+            } else {
+                reinterpret_cast<u2v*>(codes_min)[q] = u2v{b.lo, b.hi};
+                if ((q & (group_lanes - 1)) == 0) scales_min[q / group_lanes] = (uint8_t)b.exponent;
+            }
         }
     }
 }
@@ -149,7 +156,9 @@ extern "C" __global__ void __launch_bounds__(512) ca_moe_frontend(
 // (seventeen words, 128 bytes apart).  The whole `sync` region is zero before the first launch and every launch leaves it
 // zero.  Every wait is bounded: if the logits do not arrive block 0 computes them itself, so the kernel always ends.  All
 // blocks of this small grid are resident together.
-#define TF_FRONT_POOL_BYTES 77824          // 76 KiB: the shared expert's item blocks hold a 16-row tile's codes (64 KiB), scales and partial sums
+#define TF_SYNC_QUANT_DONE 17             // arrival words (128 bytes apart) of the launch that also runs the shared expert's first projection:
+#define TF_SYNC_SHARED_PASSED 18          // quantizer blocks that are done; item blocks that have read the quantizer's output
+#define TF_FRONT_POOL_BYTES 83968          // 82 KiB: the shared expert's item blocks hold a 16-row tile's codes (64 KiB), scales (2) and partial sums (16)
 // `grid_blocks`: the blocks of the launch that belong to the front-end (block ids [0, grid_blocks)); `s_pool`: TF_FRONT_POOL_BYTES
 // of LDS (logit blocks: the token rows; block 0 of owners of at most eight rows: logits, biases, token ids, live count).
 __device__ __forceinline__ void tf_route_frontend(
@@ -159,7 +168,7 @@ __device__ __forceinline__ void tf_route_frontend(
     const int32_t* padding, int32_t rows, int32_t topk, int32_t experts, int32_t cols, int32_t groups, int32_t tile_m,
     int32_t owner_rows, int32_t act_block, uint8_t* packed_min, uint8_t* scales_min, int32_t scoring,
     float route_scale, long long alt_token, const uint16_t* gate_w, uint32_t* sync, int32_t logit_blocks, int grid_blocks,
-    uint8_t* s_pool) {
+    uint8_t* s_pool, bool publish_min = false) {
     __shared__ __attribute__((aligned(16))) int32_t s_ids[1024];
     __shared__ float s_weights[1024];
     const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6, waves = blockDim.x >> 6;
@@ -284,7 +293,12 @@ __device__ __forceinline__ void tf_route_frontend(
     }
     const long long total = (long long)rows * (cols >> 3);
     tf_quantize_span(input, packed, scales, packed_min, scales_min, total, act_block,
-                     (long long)(blockIdx.x - 1) * blockDim.x + threadIdx.x, (long long)(first_logit_block - 1) * blockDim.x);
+                     (long long)(blockIdx.x - 1) * blockDim.x + threadIdx.x, (long long)(first_logit_block - 1) * blockDim.x, publish_min);
+    if (publish_min) {           // readers in this launch wait for every quantizer block (TF_SYNC_QUANT_DONE)
+        tf_stores_done();
+        __syncthreads();
+        if (threadIdx.x == 0) atomicAdd(sync + 32 * TF_SYNC_QUANT_DONE, 1u);
+    }
 }
 extern "C" __global__ void __launch_bounds__(512) ca_moe_route_frontend(
     const uint16_t* input, int32_t* ids, float* weights, uint8_t* packed, uint8_t* scales, int32_t* token_map,
