@@ -356,22 +356,34 @@ __device__ __forceinline__ void tf_fc2_items(const StreamArgs& p, int item_first
                 }
             }
             __syncthreads();
-            // quantize rows [0, valid) of the tile: 8 values a lane-step, groups of act_block / 8 lanes
-            const int per_row = p.k >> 3, group_lanes = p.act_block >> 3;
-            for (int q = threadIdx.x; q < r.valid * per_row; q += blockDim.x) {
-                const int m = q / per_row, c8 = q - m * per_row;
-                const u4v wv = reinterpret_cast<const u4v*>(p.a_bf16 + (size_t)(r.tile * 16 + m) * p.k)[c8];
-                float v[8];
+            // quantize rows [0, valid) of the tile: 8 values a lane-step, groups of act_block / 8 lanes.  Four steps' loads are
+            // requested together (a step at a time, each row would cost a round trip of its own); a wave's 64 steps are all
+            // inside the tile's rows or all outside (k / 8 is a multiple of 64)
+            const int per_row = p.k >> 3, group_lanes = p.act_block >> 3, total = r.valid * per_row;
+            for (int q0 = threadIdx.x; q0 < total; q0 += 4 * blockDim.x) {
+                u4v wv[4];
 #pragma unroll
-                for (int i = 0; i < 4; ++i) { v[2 * i] = tf_bf16_lo(wv[i]); v[2 * i + 1] = tf_bf16_hi(wv[i]); }
-                const float amax = tf_group_amax(v, group_lanes);
-                const Quant8 c = tf_quant8(v, amax, p.min_amax);
-                reinterpret_cast<u2v*>(s_codes + (size_t)m * p.k)[c8] = u2v{c.lo, c.hi};
-                if ((c8 & (group_lanes - 1)) == 0) s_scales[m * (p.k / p.act_block) + c8 / group_lanes] = (uint8_t)c.exponent;
-                if (p.q_codes != nullptr && r.j == 0) {
-                    reinterpret_cast<u2v*>(p.q_codes + (size_t)(r.tile * 16 + m) * p.k)[c8] = u2v{c.lo, c.hi};
-                    if ((c8 & (group_lanes - 1)) == 0)
-                        p.q_scales[(size_t)(r.tile * 16 + m) * (p.k / p.act_block) + c8 / group_lanes] = (uint8_t)c.exponent;
+                for (int b = 0; b < 4; ++b) {
+                    const int q = min(q0 + b * (int)blockDim.x, total - 1), m = q / per_row, c8 = q - m * per_row;
+                    wv[b] = reinterpret_cast<const u4v*>(p.a_bf16 + (size_t)(r.tile * 16 + m) * p.k)[c8];
+                }
+#pragma unroll
+                for (int b = 0; b < 4; ++b) {
+                    const int q = q0 + b * (int)blockDim.x;
+                    if (q >= total) break;
+                    const int m = q / per_row, c8 = q - m * per_row;
+                    float v[8];
+#pragma unroll
+                    for (int i = 0; i < 4; ++i) { v[2 * i] = tf_bf16_lo(wv[b][i]); v[2 * i + 1] = tf_bf16_hi(wv[b][i]); }
+                    const float amax = tf_group_amax(v, group_lanes);
+                    const Quant8 c = tf_quant8(v, amax, p.min_amax);
+                    reinterpret_cast<u2v*>(s_codes + (size_t)m * p.k)[c8] = u2v{c.lo, c.hi};
+                    if ((c8 & (group_lanes - 1)) == 0) s_scales[m * (p.k / p.act_block) + c8 / group_lanes] = (uint8_t)c.exponent;
+                    if (p.q_codes != nullptr && r.j == 0) {
+                        reinterpret_cast<u2v*>(p.q_codes + (size_t)(r.tile * 16 + m) * p.k)[c8] = u2v{c.lo, c.hi};
+                        if ((c8 & (group_lanes - 1)) == 0)
+                            p.q_scales[(size_t)(r.tile * 16 + m) * (p.k / p.act_block) + c8 / group_lanes] = (uint8_t)c.exponent;
+                    }
                 }
             }
             __syncthreads();
