@@ -1,9 +1,11 @@
 // Many-row (prefill) expert projections: grouped GEMM on v_mfma_scale_f32_16x16x128_f8f6f4.
 //
 // One task = one M tile of 128 physical rows (one expert's rows, gathered through the permutation map) x one column
-// group.  A workgroup of eight waves (512 threads, two waves a SIMD) keeps a 128 x 256 accumulator: wave (mh, nq) holds
-// rows 64 mh .. of the tile x 64 weight rows (four 16-row fragments x four 16-row weight tiles):
-//   FC1: 128 intermediate columns = 128 "up" + 128 "gate" weight rows (a wave: 32 + 32 of the same 32 columns), so SwiGLU
+// group.  A workgroup of eight waves (512 threads, two waves a SIMD) keeps a 128 x 256 accumulator: wave nq holds all
+// 128 rows (eight 16-row fragments) x 32 weight rows (two 16-row weight tiles), so every weight byte is requested by
+// exactly one wave of the workgroup (the fetch path of a CU, not the matrix cores, bounds this kernel; the token tile is
+// shared through LDS anyway):
+//   FC1: 128 intermediate columns = 128 "up" + 128 "gate" weight rows (a wave: 16 + 16 of the same 16 columns), so SwiGLU
 //        and the FP8 requantization of the result (one scale a row and `act_block` columns) run in the epilogue, from
 //        registers;
 //   FC2 / dense: 256 output columns; routed rows are scaled by their routing weight and scattered to route order.
@@ -61,13 +63,13 @@ __global__ void __launch_bounds__(512) tf_gemm(const GemmArgs p) {
     constexpr int GROUP_COLS = FC1 ? 128 : 256;          // output columns a task covers
     __shared__ __attribute__((aligned(16))) uint8_t s_a[2][16384];     // [stage][m-frag 8][half 2][lane 64][16 B]
     __shared__ __attribute__((aligned(16))) uint8_t s_scale[128 * (TF_GEMM_MAX_SCALES_ROW + 4)];    // [row][k-block]: the tile's activation scales; the row stride is an odd number of words
-    __shared__ float s_amax[4][128];
+    __shared__ float s_amax[8][128];
     __shared__ long long s_row[128];                                    // source row of each tile row
     __shared__ int32_t s_route[128];                                    // routed FC2: route (output row) of each tile row
     __shared__ float s_weight[128];                                     // routed FC2: routing weight of each tile row
-    // eight waves: row half mh (64 rows = four 16-row fragments) x column quarter nq (64 weight rows = four 16-row tiles)
+    // eight waves: wave nq takes 32 weight rows (two 16-row tiles) against every row fragment of the tile
     // the wave's index as a scalar: everything derived from it (weight tile addresses, LDS fragment offsets) stays out of the vector registers
-    const int tid = threadIdx.x, lane = tid & 63, wave = __builtin_amdgcn_readfirstlane(tid >> 6), mh = wave >> 2, nq = wave & 3, g = lane >> 4, r16 = lane & 15;
+    const int tid = threadIdx.x, lane = tid & 63, wave = __builtin_amdgcn_readfirstlane(tid >> 6), nq = wave, g = lane >> 4, r16 = lane & 15;
     const int ksteps = p.k / 128;
     const int scales_row = p.k / p.act_block, scale_words_row = scales_row / 4, scale_stride = scales_row + 4;
     const int act_shift = p.act_block == 32 ? 5 : 7;
@@ -126,11 +128,11 @@ __global__ void __launch_bounds__(512) tf_gemm(const GemmArgs p) {
         }
         // weight row tiles of this wave: FC1 routed: two "up" tiles then two "gate" tiles of the same 32 intermediate columns;
         // FC1 shared: gate tiles then up tiles; FC2 / dense: four tiles of 64 output columns
-        int ntile[4];
+        int ntile[2];
 #pragma unroll
-        for (int j = 0; j < 4; ++j) {
-            if (FC1) ntile[j] = (j >> 1) * (p.inter / 16) + (ng * 128 + nq * 32) / 16 + (j & 1);
-            else ntile[j] = (ng * 256 + nq * 64) / 16 + j;
+        for (int j = 0; j < 2; ++j) {
+            if (FC1) ntile[j] = j * (p.inter / 16) + (ng * 128 + nq * 16) / 16;
+            else ntile[j] = (ng * 256 + nq * 32) / 16 + j;
         }
         auto load_a = [&](int ks, u4v (&ra)[2]) {
 #pragma unroll
@@ -159,9 +161,9 @@ __global__ void __launch_bounds__(512) tf_gemm(const GemmArgs p) {
         };
         // B operand of one k-step: plain loads (an expert's weight slice is re-read by the expert's other tiles from this
         // XCD's L2).  FP8: with the lane's block scale of the k-step; FP4: scales come a word per four k-steps (load_b_scales).
-        auto load_b = [&](int ks, BFrag<FP8> (&b)[4], uint32_t (&sb)[4]) {
+        auto load_b = [&](int ks, BFrag<FP8> (&b)[2], uint32_t (&sb)[2]) {
 #pragma unroll
-            for (int j = 0; j < 4; ++j) {
+            for (int j = 0; j < 2; ++j) {
                 if constexpr (FP8) {
                     const u4v* src = reinterpret_cast<const u4v*>(w) + (((size_t)ntile[j] * ksteps + ks) * 2) * 64 + lane;
                     b[j].lo = src[0];
@@ -172,17 +174,16 @@ __global__ void __launch_bounds__(512) tf_gemm(const GemmArgs p) {
                 }
             }
         };
-        auto load_b_scales = [&](int ks, uint32_t (&sb)[4]) {
+        auto load_b_scales = [&](int ks, uint32_t (&sb)[2]) {
 #pragma unroll
-            for (int j = 0; j < 4; ++j) sb[j] = reinterpret_cast<const uint32_t*>(ws)[((size_t)ntile[j] * (p.k / 512) + ks / 4) * 64 + lane];
+            for (int j = 0; j < 2; ++j) sb[j] = reinterpret_cast<const uint32_t*>(ws)[((size_t)ntile[j] * (p.k / 512) + ks / 4) * 64 + lane];
         };
-        v4f acc[4][4];
+        v4f acc[8][2];
 #pragma unroll
-        for (int f = 0; f < 4; ++f)
+        for (int f = 0; f < 8; ++f)
 #pragma unroll
-            for (int j = 0; j < 4; ++j) acc[f][j] = v4f{0.f, 0.f, 0.f, 0.f};
-        const int frags = (valid + 15) >> 4;                       // of the tile
-        const int my_frags = min(4, max(0, frags - 4 * mh));       // of this wave's row half
+            for (int j = 0; j < 2; ++j) acc[f][j] = v4f{0.f, 0.f, 0.f, 0.f};
+        const int my_frags = (valid + 15) >> 4;                    // 16-row fragments of the tile with valid rows: every wave runs them all
 
         // Main loop, compiled for 0, 2 or 4 row fragments of the wave's half so that its products sit under no branch (every
         // wave runs the same loads, LDS stores and barriers whatever its count).  Operands of k-step ks + D - 1 are requested
@@ -193,9 +194,9 @@ __global__ void __launch_bounds__(512) tf_gemm(const GemmArgs p) {
             constexpr int FR = decltype(fr_constant)::value;
             constexpr int D = FP8 ? 2 : 4;         // ksteps % 4 == 0
             u4v ra[D][2];
-            BFrag<FP8> b[D][4];
-            uint32_t sbk[D][4];                  // FP8: the slot's scale bytes
-            uint32_t sb[4] = {0, 0, 0, 0}, sb_next[4] = {0, 0, 0, 0};   // FP4: scale words of the current / next four k-steps
+            BFrag<FP8> b[D][2];
+            uint32_t sbk[D][2];                  // FP8: the slot's scale bytes
+            uint32_t sb[2] = {0, 0}, sb_next[2] = {0, 0};   // FP4: scale words of the current / next four k-steps
 #pragma unroll
             for (int d = 0; d < D - 1; ++d) { load_a(d, ra[d]); load_b(d, b[d], sbk[d]); }
             if constexpr (!FP8) load_b_scales(0, sb);
@@ -217,16 +218,16 @@ __global__ void __launch_bounds__(512) tf_gemm(const GemmArgs p) {
                         if constexpr (!FP8) {
                             if (u == 0 && ks > 0) {
 #pragma unroll
-                                for (int j = 0; j < 4; ++j) sb[j] = sb_next[j];
+                                for (int j = 0; j < 2; ++j) sb[j] = sb_next[j];
                             }
                         }
                         // the next fragment's rows leave LDS while the current fragment's products run: two register sets
                         v8i av[2];
                         int sa[FR > 0 ? FR : 1];
 #pragma unroll
-                        for (int f = 0; f < FR; ++f) sa[f] = s_scale[((4 * mh + f) * 16 + r16) * scale_stride + ((ks * 128 + 32 * g) >> act_shift)];
+                        for (int f = 0; f < FR; ++f) sa[f] = s_scale[(f * 16 + r16) * scale_stride + ((ks * 128 + 32 * g) >> act_shift)];
                         auto read_frag = [&](int f, v8i& a) {
-                            const int tf = 4 * mh + f;             // fragment of the tile
+                            const int tf = f;                      // fragment of the tile
                             const u4v lo = *reinterpret_cast<const u4v*>(&s_a[stage][((tf * 2) * 64 + lane) * 16]);
                             const u4v hi = *reinterpret_cast<const u4v*>(&s_a[stage][((tf * 2 + 1) * 64 + lane) * 16]);
                             a = v8i{(int)lo[0], (int)lo[1], (int)lo[2], (int)lo[3], (int)hi[0], (int)hi[1], (int)hi[2], (int)hi[3]};
@@ -237,7 +238,7 @@ __global__ void __launch_bounds__(512) tf_gemm(const GemmArgs p) {
                             if (f + 1 < FR) read_frag(f + 1, av[(f + 1) & 1]);
                             const v8i a_now = av[f & 1];
 #pragma unroll
-                            for (int j = 0; j < 4; ++j) {
+                            for (int j = 0; j < 2; ++j) {
                                 const BFrag<FP8>& bj = b[u][j];
                                 if constexpr (FP8) {
                                     const v8i bv = v8i{(int)bj.lo[0], (int)bj.lo[1], (int)bj.lo[2], (int)bj.lo[3], (int)bj.hi[0], (int)bj.hi[1], (int)bj.hi[2], (int)bj.hi[3]};
@@ -252,7 +253,7 @@ __global__ void __launch_bounds__(512) tf_gemm(const GemmArgs p) {
                             // a use the optimizer cannot move: without it every product of the unrolled k-steps is sunk below the
                             // barriers, the k-steps' A fragments stay alive until then and spill
 #pragma unroll
-                            for (int j = 0; j < 4; ++j) asm volatile("" :: "v"(acc[f][j]));
+                            for (int j = 0; j < 2; ++j) asm volatile("" :: "v"(acc[f][j]));
                         }
                         // issue order of the k-step: fragment f + 1's LDS reads go out before fragment f's four products
                         if constexpr (FR > 0) {
@@ -260,7 +261,7 @@ __global__ void __launch_bounds__(512) tf_gemm(const GemmArgs p) {
 #pragma unroll
                             for (int f = 0; f < FR; ++f) {
                                 if (f + 1 < FR) __builtin_amdgcn_sched_group_barrier(0x100, 2, 0);
-                                __builtin_amdgcn_sched_group_barrier(0x008, 4, 0);
+                                __builtin_amdgcn_sched_group_barrier(0x008, 2, 0);
                             }
                         }
                         store_a(stage ^ 1, ra[(u + 1) % D]);
@@ -269,104 +270,105 @@ __global__ void __launch_bounds__(512) tf_gemm(const GemmArgs p) {
                 }
             }
         };
-        if (my_frags > 2) main_loop(std::integral_constant<int, 4>{});
-        else if (my_frags > 0) main_loop(std::integral_constant<int, 2>{});
-        else main_loop(std::integral_constant<int, 0>{});
+        if (my_frags > 6) main_loop(std::integral_constant<int, 8>{});
+        else if (my_frags > 4) main_loop(std::integral_constant<int, 6>{});
+        else if (my_frags > 2) main_loop(std::integral_constant<int, 4>{});
+        else main_loop(std::integral_constant<int, 2>{});
 
         // ---- epilogue --------------------------------------------------------------------------------------------------
         if constexpr (FC1) {
             // The weight tile is the instruction's first operand and the token fragment its second, so lane (g, r16) of product
-            // (f, j) holds tile row 64 mh + 16 f + r16 and the four consecutive columns 4 g + i (i < 4) of weight tile j: a lane
-            // packs its four values into one store (four E4M3 codes a word, four BF16 values a pair of words).
+            // (f, j) holds tile row 16 f + r16 and the four consecutive columns 4 g + i (i < 4) of weight tile j: a lane packs
+            // its four values into one store (four E4M3 codes a word, four BF16 values a pair of words).  j = 0 / 1: the up and
+            // gate tiles (shared expert: gate, up) of the wave's 16 intermediate columns.
             const float hi_lim = tf_bf16(tf_to_bf16(p.limit)), lo_lim = tf_bf16(tf_to_bf16(-p.limit));
-            float hv[4][2][4];
-            float amax[4];
+            float hv[8][4];
+            float amax[8];
 #pragma unroll
-            for (int f = 0; f < 4; ++f) {
-                const int row = 64 * mh + 16 * f + r16;
+            for (int f = 0; f < 8; ++f) {
+                const int row = 16 * f + r16;
                 float m = 0.f;
+                if (MODE == TF_GEMM_FC1_SHARED) {
+                    uint16_t gb[4], ub[4];
 #pragma unroll
-                for (int j = 0; j < 2; ++j) {
-                    if (MODE == TF_GEMM_FC1_SHARED) {
-                        uint16_t gb[4], ub[4];
-#pragma unroll
-                        for (int i = 0; i < 4; ++i) { gb[i] = tf_to_bf16(acc[f][j][i]); ub[i] = tf_to_bf16(acc[f][2 + j][i]); }
-                        if (p.tap != nullptr && f < my_frags && row < valid) {
-                            const size_t at = (size_t)(tile * 128 + row) * 2 * p.inter + ng * 128 + nq * 32 + j * 16 + 4 * g;
-                            *reinterpret_cast<u2v*>(p.tap + at) = u2v{(uint32_t)gb[0] | ((uint32_t)gb[1] << 16), (uint32_t)gb[2] | ((uint32_t)gb[3] << 16)};
-                            *reinterpret_cast<u2v*>(p.tap + at + p.inter) = u2v{(uint32_t)ub[0] | ((uint32_t)ub[1] << 16), (uint32_t)ub[2] | ((uint32_t)ub[3] << 16)};
-                        }
-#pragma unroll
-                        for (int i = 0; i < 4; ++i) {
-                            const float gv = fminf(tf_bf16(gb[i]), hi_lim), uv = fminf(fmaxf(tf_bf16(ub[i]), lo_lim), hi_lim);
-                            hv[f][j][i] = tf_bf16(tf_to_bf16(__fmul_rn(gv / __fadd_rn(1.0f, tf_exp(-gv)), uv)));
-                        }
-                    } else {
-                        // routed experts: no bit-level definition of this step exists (the reference's is inside a binary), the
-                        // result is rounded to BF16 next; the many-row path takes the hardware exponential and reciprocal
-#pragma unroll
-                        for (int i = 0; i < 4; ++i) {
-                            const float gv = fminf(acc[f][2 + j][i], p.limit), uv = fminf(p.limit, fmaxf(-p.limit, acc[f][j][i]));
-                            hv[f][j][i] = tf_bf16(tf_to_bf16(__fmul_rn(__fmul_rn(gv, tf_logistic_fast(gv)), uv)));
-                        }
+                    for (int i = 0; i < 4; ++i) { gb[i] = tf_to_bf16(acc[f][0][i]); ub[i] = tf_to_bf16(acc[f][1][i]); }
+                    if (p.tap != nullptr && f < my_frags && row < valid) {
+                        const size_t at = (size_t)(tile * 128 + row) * 2 * p.inter + ng * 128 + nq * 16 + 4 * g;
+                        *reinterpret_cast<u2v*>(p.tap + at) = u2v{(uint32_t)gb[0] | ((uint32_t)gb[1] << 16), (uint32_t)gb[2] | ((uint32_t)gb[3] << 16)};
+                        *reinterpret_cast<u2v*>(p.tap + at + p.inter) = u2v{(uint32_t)ub[0] | ((uint32_t)ub[1] << 16), (uint32_t)ub[2] | ((uint32_t)ub[3] << 16)};
                     }
 #pragma unroll
-                    for (int i = 0; i < 4; ++i) m = fmaxf(m, fabsf(hv[f][j][i]));
+                    for (int i = 0; i < 4; ++i) {
+                        const float gv = fminf(tf_bf16(gb[i]), hi_lim), uv = fminf(fmaxf(tf_bf16(ub[i]), lo_lim), hi_lim);
+                        hv[f][i] = tf_bf16(tf_to_bf16(__fmul_rn(gv / __fadd_rn(1.0f, tf_exp(-gv)), uv)));
+                    }
+                } else {
+                    // routed experts: no bit-level definition of this step exists (the reference's is inside a binary), the
+                    // result is rounded to BF16 next; the many-row path takes the hardware exponential and reciprocal
+#pragma unroll
+                    for (int i = 0; i < 4; ++i) {
+                        const float gv = fminf(acc[f][1][i], p.limit), uv = fminf(p.limit, fmaxf(-p.limit, acc[f][0][i]));
+                        hv[f][i] = tf_bf16(tf_to_bf16(__fmul_rn(__fmul_rn(gv, tf_logistic_fast(gv)), uv)));
+                    }
                 }
-                // the row's 32 columns of this wave sit in the four lanes r16 + 16 g
+#pragma unroll
+                for (int i = 0; i < 4; ++i) m = fmaxf(m, fabsf(hv[f][i]));
+                // the row's 16 columns of this wave sit in the four lanes r16 + 16 g
                 m = fmaxf(m, __shfl_xor(m, 16));
                 amax[f] = fmaxf(m, __shfl_xor(m, 32));
             }
-            if (p.act_block == 128) {          // one scale per row and 128 columns: across the four column quarters
+            // one scale per row and 32 (two waves) or 128 (all eight waves) columns
 #pragma unroll
-                for (int f = 0; f < 4; ++f) if (g == 0) s_amax[nq][64 * mh + 16 * f + r16] = amax[f];
-                __syncthreads();
+            for (int f = 0; f < 8; ++f) if (g == 0) s_amax[nq][16 * f + r16] = amax[f];
+            __syncthreads();
 #pragma unroll
-                for (int f = 0; f < 4; ++f) {
-                    const int row = 64 * mh + 16 * f + r16;
-                    amax[f] = fmaxf(fmaxf(s_amax[0][row], s_amax[1][row]), fmaxf(s_amax[2][row], s_amax[3][row]));
+            for (int f = 0; f < 8; ++f) {
+                const int row = 16 * f + r16;
+                if (p.act_block == 128) {
+                    float m = s_amax[0][row];
+#pragma unroll
+                    for (int w2 = 1; w2 < 8; ++w2) m = fmaxf(m, s_amax[w2][row]);
+                    amax[f] = m;
+                } else {
+                    amax[f] = fmaxf(s_amax[nq & 6][row], s_amax[nq | 1][row]);
                 }
             }
             const float min_amax = MODE == TF_GEMM_FC1_SHARED ? 1e-4f : 0.f;
 #pragma unroll
-            for (int f = 0; f < 4; ++f) {
-                const int row = 64 * mh + 16 * f + r16;
+            for (int f = 0; f < 8; ++f) {
+                const int row = 16 * f + r16;
                 if (f < my_frags && row < valid) {
                     const uint32_t exponent = tf_block_exponent(min_amax > 0.f ? fmaxf(amax[f], min_amax) : amax[f]);
                     const float inv = tf_block_inverse(exponent);
                     const size_t phys = (size_t)tile * 128 + row;
-                    const int col = ng * 128 + nq * 32 + 4 * g;
-#pragma unroll
-                    for (int j = 0; j < 2; ++j) {
-                        *reinterpret_cast<uint32_t*>(p.h_codes + phys * p.inter + col + 16 * j) =
-                            tf_pack_e4m3(__fmul_rn(hv[f][j][0], inv), __fmul_rn(hv[f][j][1], inv), __fmul_rn(hv[f][j][2], inv), __fmul_rn(hv[f][j][3], inv));
-                        if (p.h_bf16 != nullptr)
-                            *reinterpret_cast<u2v*>(p.h_bf16 + phys * p.inter + col + 16 * j) =
-                                u2v{tf_pack_bf16(hv[f][j][0], hv[f][j][1]), tf_pack_bf16(hv[f][j][2], hv[f][j][3])};
-                    }
+                    const int col = ng * 128 + nq * 16 + 4 * g;
+                    *reinterpret_cast<uint32_t*>(p.h_codes + phys * p.inter + col) =
+                        tf_pack_e4m3(__fmul_rn(hv[f][0], inv), __fmul_rn(hv[f][1], inv), __fmul_rn(hv[f][2], inv), __fmul_rn(hv[f][3], inv));
+                    if (p.h_bf16 != nullptr)
+                        *reinterpret_cast<u2v*>(p.h_bf16 + phys * p.inter + col) = u2v{tf_pack_bf16(hv[f][0], hv[f][1]), tf_pack_bf16(hv[f][2], hv[f][3])};
                     if (g == 0) {
-                        if (p.act_block == 32) p.h_scales[phys * (p.inter / 32) + ng * 4 + nq] = (uint8_t)exponent;
+                        if (p.act_block == 32) { if ((nq & 1) == 0) p.h_scales[phys * (p.inter / 32) + ng * 4 + (nq >> 1)] = (uint8_t)exponent; }
                         else if (nq == 0) p.h_scales[phys * (p.inter / 128) + ng] = (uint8_t)exponent;
                     }
                 }
             }
         } else {
-            // the token fragment is the first operand here: lane (g, r16) of product (f, j) holds tile rows 64 mh + 16 f + 4 g + i
+            // the token fragment is the first operand here: lane (g, r16) of product (f, j) holds tile rows 16 f + 4 g + i
             // (i < 4) and column r16 of weight tile j
 #pragma unroll
-            for (int f = 0; f < 4; ++f) {
+            for (int f = 0; f < 8; ++f) {
                 if (f < my_frags) {
 #pragma unroll
                     for (int i = 0; i < 4; ++i) {
-                        const int row = 64 * mh + 16 * f + 4 * g + i;
+                        const int row = 16 * f + 4 * g + i;
                         if (row < valid) {
                             size_t out_row = (size_t)tile * 128 + row;
                             float scale = 1.f;
                             if (MODE == TF_GEMM_FC2_ROUTED) { out_row = (size_t)s_route[row]; scale = s_weight[row]; }
 #pragma unroll
-                            for (int j = 0; j < 4; ++j) {
+                            for (int j = 0; j < 2; ++j) {
                                 const float v = MODE == TF_GEMM_FC2_ROUTED ? __fmul_rn(acc[f][j][i], scale) : acc[f][j][i];
-                                p.out[out_row * p.hidden + ng * 256 + nq * 64 + 16 * j + r16] = tf_to_bf16(v);
+                                p.out[out_row * p.hidden + ng * 256 + nq * 32 + 16 * j + r16] = tf_to_bf16(v);
                             }
                         }
                     }
