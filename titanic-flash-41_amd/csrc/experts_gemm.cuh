@@ -62,7 +62,7 @@ __global__ void __launch_bounds__(512) tf_gemm(const GemmArgs p) {
     constexpr bool ROUTED = MODE == TF_GEMM_FC1_ROUTED || MODE == TF_GEMM_FC2_ROUTED;
     constexpr int GROUP_COLS = FC1 ? 128 : 256;          // output columns a task covers
     __shared__ __attribute__((aligned(16))) uint8_t s_a[2][16384];     // [stage][m-frag 8][half 2][lane 64][16 B]
-    __shared__ __attribute__((aligned(16))) uint8_t s_scale[128 * (TF_GEMM_MAX_SCALES_ROW + 4)];    // [row][k-block]: the tile's activation scales; the row stride is an odd number of words
+    __shared__ __attribute__((aligned(16))) uint8_t s_scale[128 * (TF_GEMM_MAX_SCALES_ROW + 16)];   // [row][k-block]: the tile's activation scales; the 16 rows a fragment reads at once fall into different banks
     __shared__ float s_amax[8][128];
     __shared__ long long s_row[128];                                    // source row of each tile row
     __shared__ int32_t s_route[128];                                    // routed FC2: route (output row) of each tile row
@@ -71,7 +71,7 @@ __global__ void __launch_bounds__(512) tf_gemm(const GemmArgs p) {
     // the wave's index as a scalar: everything derived from it (weight tile addresses, LDS fragment offsets) stays out of the vector registers
     const int tid = threadIdx.x, lane = tid & 63, wave = __builtin_amdgcn_readfirstlane(tid >> 6), nq = wave, g = lane >> 4, r16 = lane & 15;
     const int ksteps = p.k / 128;
-    const int scales_row = p.k / p.act_block, scale_words_row = scales_row / 4, scale_stride = scales_row + 4;
+    const int scales_row = p.k / p.act_block, scale_words_row = scales_row / 4, scale_stride = scales_row + 16;
     const int act_shift = p.act_block == 32 ? 5 : 7;
     const int n_cols = FC1 ? p.inter : p.hidden, groups = n_cols / GROUP_COLS;
     const int tiles = ROUTED ? p.expert_tile_base[p.experts] : (p.dense_rows + 127) / 128;
@@ -190,8 +190,12 @@ __global__ void __launch_bounds__(512) tf_gemm(const GemmArgs p) {
         // while k-step ks is multiplied (a ring of D register sets, indexed statically by unrolling D times): the token tile
         // goes registers -> LDS one k-step ahead of its use (two LDS stages, one barrier a k-step), the weights stay in
         // registers.  Two waves share a SIMD, so one wave's loads, LDS traffic and scalar work run under the other's products.
-        auto main_loop = [&](auto fr_constant) {
+        auto main_loop = [&](auto fr_constant, auto words_constant) {
             constexpr int FR = decltype(fr_constant)::value;
+            // 128-wide activation blocks: a k-step has one scale a row, so a word holds the scales of four k-steps (the
+            // instruction selects the byte); 32-wide blocks: a byte a row, k-step and lane group
+            constexpr bool WORDS = decltype(words_constant)::value;
+            constexpr int U = 4;                   // k-steps an unrolled round
             constexpr int D = FP8 ? 2 : 4;         // ksteps % 4 == 0
             u4v ra[D][2];
             BFrag<FP8> b[D][2];
@@ -203,9 +207,15 @@ __global__ void __launch_bounds__(512) tf_gemm(const GemmArgs p) {
             store_scales();
             store_a(0, ra[0]);
             __syncthreads();
-            for (int ks0 = 0; ks0 < ksteps; ks0 += D) {
+            int sw[FR];
+            for (int ks0 = 0; ks0 < ksteps; ks0 += U) {
+                if constexpr (WORDS) {
 #pragma unroll
-                for (int u = 0; u < D; ++u) {
+                    for (int f = 0; f < FR; ++f) sw[f] = *reinterpret_cast<const int*>(&s_scale[(f * 16 + r16) * scale_stride + ks0]);
+                }
+                // one k-step; its index within the round is a compile-time constant (it selects ring slots and scale bytes)
+                auto k_step = [&](auto u_constant) {
+                    constexpr int u = decltype(u_constant)::value;
                     const int ks = ks0 + u;
                     {
                         // No load sits under a condition (the last D - 1 k-steps request the last k-step again rather than
@@ -223,9 +233,10 @@ __global__ void __launch_bounds__(512) tf_gemm(const GemmArgs p) {
                         }
                         // the next fragment's rows leave LDS while the current fragment's products run: two register sets
                         v8i av[2];
-                        int sa[FR > 0 ? FR : 1];
+                        int sa[FR];
 #pragma unroll
-                        for (int f = 0; f < FR; ++f) sa[f] = s_scale[(f * 16 + r16) * scale_stride + ((ks * 128 + 32 * g) >> act_shift)];
+                        for (int f = 0; f < FR; ++f) sa[f] = WORDS ? sw[f] : s_scale[(f * 16 + r16) * scale_stride + ((ks * 128 + 32 * g) >> act_shift)];
+                        constexpr int SEL = WORDS ? u : 0;        // byte of the activation scale register
                         auto read_frag = [&](int f, v8i& a) {
                             const int tf = f;                      // fragment of the tile
                             const u4v lo = *reinterpret_cast<const u4v*>(&s_a[stage][((tf * 2) * 64 + lane) * 16]);
@@ -239,15 +250,15 @@ __global__ void __launch_bounds__(512) tf_gemm(const GemmArgs p) {
                             const v8i a_now = av[f & 1];
 #pragma unroll
                             for (int j = 0; j < 2; ++j) {
-                                const BFrag<FP8>& bj = b[u][j];
+                                const BFrag<FP8>& bj = b[u % D][j];
                                 if constexpr (FP8) {
                                     const v8i bv = v8i{(int)bj.lo[0], (int)bj.lo[1], (int)bj.lo[2], (int)bj.lo[3], (int)bj.hi[0], (int)bj.hi[1], (int)bj.hi[2], (int)bj.hi[3]};
-                                    if constexpr (FC1) acc[f][j] = __builtin_amdgcn_mfma_scale_f32_16x16x128_f8f6f4(bv, a_now, acc[f][j], 0, 0, 0, (int)sbk[u][j], 0, sa[f]);
-                                    else acc[f][j] = __builtin_amdgcn_mfma_scale_f32_16x16x128_f8f6f4(a_now, bv, acc[f][j], 0, 0, 0, sa[f], 0, (int)sbk[u][j]);
+                                    if constexpr (FC1) acc[f][j] = __builtin_amdgcn_mfma_scale_f32_16x16x128_f8f6f4(bv, a_now, acc[f][j], 0, 0, 0, (int)sbk[u % D][j], SEL, sa[f]);
+                                    else acc[f][j] = __builtin_amdgcn_mfma_scale_f32_16x16x128_f8f6f4(a_now, bv, acc[f][j], 0, 0, SEL, sa[f], 0, (int)sbk[u % D][j]);
                                 } else {
                                     const v8i bv = v8i{(int)bj.lo[0], (int)bj.lo[1], (int)bj.lo[2], (int)bj.lo[3], 0, 0, 0, 0};
-                                    if constexpr (FC1) acc[f][j] = __builtin_amdgcn_mfma_scale_f32_16x16x128_f8f6f4(bv, a_now, acc[f][j], 4, 0, 0, (int)(sb[j] >> (8 * u)), 0, sa[f]);
-                                    else acc[f][j] = __builtin_amdgcn_mfma_scale_f32_16x16x128_f8f6f4(a_now, bv, acc[f][j], 0, 4, 0, sa[f], 0, (int)(sb[j] >> (8 * u)));
+                                    if constexpr (FC1) acc[f][j] = __builtin_amdgcn_mfma_scale_f32_16x16x128_f8f6f4(bv, a_now, acc[f][j], 4, 0, u, (int)sb[j], SEL, sa[f]);
+                                    else acc[f][j] = __builtin_amdgcn_mfma_scale_f32_16x16x128_f8f6f4(a_now, bv, acc[f][j], 0, 4, SEL, sa[f], u, (int)sb[j]);
                                 }
                             }
                             // a use the optimizer cannot move: without it every product of the unrolled k-steps is sunk below the
@@ -267,13 +278,24 @@ __global__ void __launch_bounds__(512) tf_gemm(const GemmArgs p) {
                         store_a(stage ^ 1, ra[(u + 1) % D]);
                         __syncthreads();
                     }
-                }
+                };
+                k_step(std::integral_constant<int, 0>{});
+                k_step(std::integral_constant<int, 1>{});
+                k_step(std::integral_constant<int, 2>{});
+                k_step(std::integral_constant<int, 3>{});
             }
         };
-        if (my_frags > 6) main_loop(std::integral_constant<int, 8>{});
-        else if (my_frags > 4) main_loop(std::integral_constant<int, 6>{});
-        else if (my_frags > 2) main_loop(std::integral_constant<int, 4>{});
-        else main_loop(std::integral_constant<int, 2>{});
+        if (p.act_block == 128) {
+            if (my_frags > 6) main_loop(std::integral_constant<int, 8>{}, std::true_type{});
+            else if (my_frags > 4) main_loop(std::integral_constant<int, 6>{}, std::true_type{});
+            else if (my_frags > 2) main_loop(std::integral_constant<int, 4>{}, std::true_type{});
+            else main_loop(std::integral_constant<int, 2>{}, std::true_type{});
+        } else {
+            if (my_frags > 6) main_loop(std::integral_constant<int, 8>{}, std::false_type{});
+            else if (my_frags > 4) main_loop(std::integral_constant<int, 6>{}, std::false_type{});
+            else if (my_frags > 2) main_loop(std::integral_constant<int, 4>{}, std::false_type{});
+            else main_loop(std::integral_constant<int, 2>{}, std::false_type{});
+        }
 
         // ---- epilogue --------------------------------------------------------------------------------------------------
         if constexpr (FC1) {
