@@ -46,7 +46,7 @@ MFMA_FP8_PEAK_TFLOPS, MFMA_FP4_PEAK_TFLOPS = 5000.0, 10100.0
 # bytes of this run's launches; None where no counter run exists for the configuration.
 TRAFFIC_OVER_ALGORITHMIC = {"c2": 1.0003}
 # Many rows: HBM bytes a launch of the routed FC1 kernel, measured the same way at the same number of rows.
-WIDE_TRAFFIC_BYTES = {"c4": 3.61e9, "c5": 8.38e9}
+WIDE_TRAFFIC_BYTES = {"c4": 3.24e9, "c5": 6.92e9}
 
 
 def make_inputs(synth, name, cfg, device, batches=BATCHES):
