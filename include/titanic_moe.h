@@ -22,11 +22,11 @@ extern "C" {
 #endif
 
 typedef struct ca_geometry {
-    int32_t hidden;               /* H, multiple of 512 */
+    int32_t hidden;               /* H: multiple of 512 up to 4,096, or of 1,024 up to 8,192 */
     int32_t experts;              /* E <= 512 */
     int32_t topk;                 /* K <= 8 */
-    int32_t intermediate;         /* routed expert intermediate I, multiple of 512 */
-    int32_t shared_intermediate;  /* shared expert intermediate, multiple of 512 */
+    int32_t intermediate;         /* routed expert intermediate I, multiple of 512 up to 4,096 */
+    int32_t shared_intermediate;  /* shared expert intermediate, multiple of 512 up to 4,096 */
     int32_t scoring;              /* 0 sigmoid, 1 sqrt(softplus) (reference: 1, src/ffn.rs:249) */
     float route_scale;            /* routed_scaling_factor (reference: 1.5, src/ffn.rs:250) */
     int32_t act_block;            /* activation quantization block: 32 (reference) or 128 */

@@ -1,6 +1,6 @@
 """GPU parity over the shapes between and around the benchmark configurations, through the C++ host mirror: one row (the
 reference's 1-row micro plan), the 64 / 65-row boundary between the streaming and the grouped-GEMM paths, every supported
-contraction length, top-1 and top-8, the reference's expert count, live prefixes and padding rows on the many-row path.
+contraction length class (multiples of 512 up to 4,096; token widths up to 8,192), top-1 and top-8, the reference's expert count, live prefixes and padding rows on the many-row path.
 Same checks as the benchmark shapes (bit-exact routing, plan, codes; staged tolerance behind the matrix cores)."""
 import numpy as np
 import pytest
@@ -40,6 +40,12 @@ def run_case(rows, hidden, experts, topk, inter, shared, mode, live=None, paddin
     (64, 1024, 32, 4, 512, 512, "reference"),       # the last row count of the streaming path
     (65, 1024, 32, 4, 512, 512, "benchmark"),       # the first of the grouped-GEMM path
     (130, 2048, 16, 2, 1024, 1024, "reference"),    # a second, partly filled row tile; K 1024 in FC2
+    (6, 5120, 32, 6, 2560, 2560, "reference"),      # the reference's token width (src/ffn.rs:65-66): eight-wave FC1 launch, five k-steps a wave
+    (40, 5120, 64, 6, 1536, 512, "benchmark"),      # the same with three row tiles; K 1536 in FC2 (three k-steps a wave: scale words straddled)
+    (130, 5120, 32, 2, 1024, 512, "reference"),     # many rows at that width: 160 activation scale bytes a row, staged in two passes
+    (5, 1536, 16, 2, 3072, 3584, "benchmark"),      # three, six and seven k-steps a wave
+    (70, 6144, 16, 2, 512, 512, "reference"),       # many rows, K 6,144
+    (3, 8192, 8, 2, 1024, 1024, "benchmark"),       # the widest token row
 ])
 def test_shape(rows, hidden, experts, topk, inter, shared, mode):
     run_case(rows, hidden, experts, topk, inter, shared, mode)

@@ -14,7 +14,9 @@ namespace {
 
 ca_geometry g_geometry = {5120, 384, 6, 576, 576, 1, 1.5f, 32, 32, 32, 129264, 10.f};   // src/ffn.rs:65-66, 245-258
 
-bool supported_k(int k) { return k == 512 || k == 1024 || k == 2048 || k == 4096; }
+// contraction lengths: multiples of 512 up to 4,096 everywhere; the token width (FC1) also multiples of 1,024 up to 8,192
+bool supported_k(int k) { return k >= 512 && k <= 4096 && k % 512 == 0; }
+bool supported_hidden(int k) { return supported_k(k) || (k > 4096 && k <= 8192 && k % 1024 == 0); }
 int check_geometry(const ca_geometry& g) {
     if (g.hidden <= 0 || g.hidden % 512 || g.experts <= 0 || g.experts > 512 || g.topk <= 0 || g.topk > 8 ||
         g.topk > g.experts || g.intermediate <= 0 || g.intermediate % 512 || g.shared_intermediate <= 0 ||
@@ -43,11 +45,20 @@ void mark(const Context& c, int i, hipStream_t s) {
 int launch_phase1(const StreamArgs& routed, const StreamArgs& shared, int wgs, hipStream_t s) {
     const int k = routed.w ? routed.k : shared.k;
     if (routed.w && shared.w && routed.k != shared.k) return -4;
+    const int wide = wgs >= 2 ? wgs / 2 : 1;       // eight-wave workgroups: one a CU
     switch (k) {
         case 512: tf_phase1_stream<1, 1><<<wgs, 256, 0, s>>>(routed, shared); break;
         case 1024: tf_phase1_stream<2, 2><<<wgs, 256, 0, s>>>(routed, shared); break;
+        case 1536: tf_phase1_stream<3, 3><<<wgs, 256, 0, s>>>(routed, shared); break;
         case 2048: tf_phase1_stream<4, 4><<<wgs, 256, 0, s>>>(routed, shared); break;
+        case 2560: tf_phase1_stream<5, 5><<<wgs, 256, 0, s>>>(routed, shared); break;
+        case 3072: tf_phase1_stream<6, 6><<<wgs, 256, 0, s>>>(routed, shared); break;
+        case 3584: tf_phase1_stream<7, 7><<<wgs, 256, 0, s>>>(routed, shared); break;
         case 4096: tf_phase1_stream<8, 8><<<wgs, 256, 0, s>>>(routed, shared); break;
+        case 5120: tf_phase1_stream<5, 5, 8><<<wide, 512, 0, s>>>(routed, shared); break;
+        case 6144: tf_phase1_stream<6, 6, 8><<<wide, 512, 0, s>>>(routed, shared); break;
+        case 7168: tf_phase1_stream<7, 7, 8><<<wide, 512, 0, s>>>(routed, shared); break;
+        case 8192: tf_phase1_stream<8, 8, 8><<<wide, 512, 0, s>>>(routed, shared); break;
         default: return -4;
     }
     return launch_status();
@@ -63,7 +74,11 @@ int launch_phase2(const StreamArgs& routed, const StreamArgs& shared, int wgs, h
     switch (k) {
         case 512: tf_phase2_stream<1, 1><<<wgs, 256, lds, s>>>(routed, shared); break;
         case 1024: tf_phase2_stream<2, 2><<<wgs, 256, lds, s>>>(routed, shared); break;
+        case 1536: tf_phase2_stream<3, 3><<<wgs, 256, lds, s>>>(routed, shared); break;
         case 2048: tf_phase2_stream<4, 4><<<wgs, 256, lds, s>>>(routed, shared); break;
+        case 2560: tf_phase2_stream<5, 5><<<wgs, 256, lds, s>>>(routed, shared); break;
+        case 3072: tf_phase2_stream<6, 6><<<wgs, 256, lds, s>>>(routed, shared); break;
+        case 3584: tf_phase2_stream<7, 7><<<wgs, 256, lds, s>>>(routed, shared); break;
         case 4096: tf_phase2_stream<8, 8><<<wgs, 256, lds, s>>>(routed, shared); break;
         default: return -4;
     }
@@ -114,7 +129,7 @@ int launch_dynamic(const Context& c, bool route, const uint64_t* p, const int32_
         if (!p[i] && i != P_PACKED_MIN && i != P_SCALES_MIN && i != P_INTER_CODES && i != P_INTER_SCALES && i != P_PLAN_SCRATCH &&
             !(i == P_INTER && rows > TF_STREAM_MAX_ROWS))
             return -1;
-    if (!supported_k(g.hidden) || !supported_k(g.intermediate)) return -4;
+    if (!supported_hidden(g.hidden) || !supported_k(g.intermediate)) return -4;
     if (packed_input && g.act_block != 32) return -4;      // the wire row carries 32-wide blocks
     const long long pairs = (long long)rows * g.topk;
     // capacity of the reference's contracts (max_phys_tiles): A = min(E, pairs) experts open a tile each and the other routes fill
@@ -286,7 +301,7 @@ int launch_quant(const Context& c, const uint64_t* p, const int32_t* sc, hipStre
 int launch_dense(const Context& c, const uint64_t* p, const int32_t* sc, hipStream_t s) {
     const int m = sc[0], n = sc[1], k = sc[2];
     for (int i = 0; i < 5; ++i) if (!p[i]) return -1;
-    if (m < 1 || n < 64 || n % 64 || !supported_k(k)) return -1;
+    if (m < 1 || n < 64 || n % 64 || !supported_hidden(k)) return -1;
     if (m <= TF_STREAM_MAX_ROWS) {
         StreamArgs a{};
         a.a_codes = (const uint8_t*)p[0]; a.a_scales = (const uint8_t*)p[1];
@@ -305,7 +320,7 @@ int launch_shared(const Context& c, const uint64_t* p, const int32_t* sc, hipStr
     const ca_geometry& g = c.g;
     const int m = sc[0];
     for (int i = 0; i < H_COUNT; ++i) if (!p[i] && i != H_UP_TAP && i != H_ACT_CODES && i != H_ACT_SCALES) return -1;
-    if (m < 1 || !supported_k(g.hidden) || !supported_k(g.shared_intermediate)) return -4;
+    if (m < 1 || !supported_hidden(g.hidden) || !supported_k(g.shared_intermediate)) return -4;
     if (m <= TF_STREAM_MAX_ROWS) {
         StreamArgs a, b, none{};
         shared_stream_args(c, p, m, a, b);

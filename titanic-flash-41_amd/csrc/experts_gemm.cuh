@@ -25,8 +25,8 @@
 
 #define TF_STREAM_MAX_ROWS 64
 #define TF_GEMM_TILE_M 128
-#define TF_GEMM_MAX_SCALES_ROW 128                 // activation scales a row the tile table holds: k / act_block
-#define TF_GEMM_SCALE_WORDS 8                       // words of that table a thread moves: 128 rows x 128 bytes / 512 threads / 4
+#define TF_GEMM_MAX_SCALES_ROW 256                 // activation scales a row the tile table holds: k / act_block
+#define TF_GEMM_SCALE_WORDS 8                       // words of that table a thread moves a pass: 128 rows x 128 bytes / 512 threads / 4 (wider rows: two passes)
 
 struct GemmArgs {
     const uint8_t* a_codes;          // E4M3 [rows][k]: token rows (FC1), physical rows (routed FC2), dense rows
@@ -146,19 +146,22 @@ __global__ void __launch_bounds__(512) tf_gemm(const GemmArgs p) {
         // loop costs a cache line request per row: as many requests as the tile's codes need).  Requested first, stored after
         // the main loop's first operand requests are out.
         uint32_t scale_regs[TF_GEMM_SCALE_WORDS];
-#pragma unroll
-        for (int i = 0; i < TF_GEMM_SCALE_WORDS; ++i) {
-            const int c = min(tid + 512 * i, 128 * scale_words_row - 1);            // word c % per_row of row c / per_row
-            scale_regs[i] = *reinterpret_cast<const uint32_t*>(p.a_scales + s_row[min(c / scale_words_row, valid - 1)] * scales_row + (c % scale_words_row) * 4);
-        }
-        auto store_scales = [&]() {
+        auto load_scales = [&](int pass) {
 #pragma unroll
             for (int i = 0; i < TF_GEMM_SCALE_WORDS; ++i) {
-                const int c = tid + 512 * i;
+                const int c = min(tid + 512 * (i + TF_GEMM_SCALE_WORDS * pass), 128 * scale_words_row - 1);            // word c % per_row of row c / per_row
+                scale_regs[i] = *reinterpret_cast<const uint32_t*>(p.a_scales + s_row[min(c / scale_words_row, valid - 1)] * scales_row + (c % scale_words_row) * 4);
+            }
+        };
+        auto store_scales = [&](int pass) {
+#pragma unroll
+            for (int i = 0; i < TF_GEMM_SCALE_WORDS; ++i) {
+                const int c = tid + 512 * (i + TF_GEMM_SCALE_WORDS * pass);
                 if (c < 128 * scale_words_row)
                     *reinterpret_cast<uint32_t*>(&s_scale[(c / scale_words_row) * scale_stride + (c % scale_words_row) * 4]) = scale_regs[i];
             }
         };
+        load_scales(0);
         // B operand of one k-step: plain loads (an expert's weight slice is re-read by the expert's other tiles from this
         // XCD's L2).  FP8: with the lane's block scale of the k-step; FP4: scales come a word per four k-steps (load_b_scales).
         auto load_b = [&](int ks, BFrag<FP8> (&b)[2], uint32_t (&sb)[2]) {
@@ -204,7 +207,11 @@ __global__ void __launch_bounds__(512) tf_gemm(const GemmArgs p) {
 #pragma unroll
             for (int d = 0; d < D - 1; ++d) { load_a(d, ra[d]); load_b(d, b[d], sbk[d]); }
             if constexpr (!FP8) load_b_scales(0, sb);
-            store_scales();
+            store_scales(0);
+            if (scale_words_row > 4 * TF_GEMM_SCALE_WORDS) {       // more than 128 scale bytes a row (K above 4,096 with 32-wide blocks)
+                load_scales(1);
+                store_scales(1);
+            }
             store_a(0, ra[0]);
             __syncthreads();
             int sw[FR];

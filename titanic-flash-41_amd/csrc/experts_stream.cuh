@@ -88,7 +88,8 @@ struct Unit {
     uint32_t scale[TILES * ((KS + 3) / 4)];
 };
 // FP4: words [n/16][k/128][lane][16 B], scales [n/16][k/512][lane][4 B] (byte q of a word = k-step 4 kq + q).
-// KS is 1, 2 or a multiple of 4, so a wave's k-steps never straddle a scale word.
+// A wave's k-steps start inside a scale word unless KS is a multiple of 4 (KS 1, 2: inside one word); for the other counts
+// one more word is read and the two are funnel-shifted so that byte q of register i is k-step 4 i + q of the wave's share.
 template <int TILES, int KS>
 __device__ __forceinline__ void tf_load_fp4(Unit<TILES, KS>& u, const uint8_t* w, const uint8_t* scales, const int (&ntile)[TILES], int k,
                                             int ks_first, int lane) {
@@ -98,9 +99,19 @@ __device__ __forceinline__ void tf_load_fp4(Unit<TILES, KS>& u, const uint8_t* w
         const u4v* src = reinterpret_cast<const u4v*>(w) + ((size_t)ntile[t] * (k / 128) + ks_first) * 64 + lane;
 #pragma unroll
         for (int s = 0; s < KS; ++s) u.d[t * KS + s] = tf_stream_load(src + s * 64);
-        const uint32_t* sc = reinterpret_cast<const uint32_t*>(scales) + ((size_t)ntile[t] * (k / 512) + ks_first / 4) * 64 + lane;
+        if constexpr (KS <= 2 || KS % 4 == 0) {
+            const uint32_t* sc = reinterpret_cast<const uint32_t*>(scales) + ((size_t)ntile[t] * (k / 512) + ks_first / 4) * 64 + lane;
 #pragma unroll
-        for (int q = 0; q < SW; ++q) u.scale[t * SW + q] = __builtin_nontemporal_load(sc + q * 64) >> (8 * (ks_first & 3));
+            for (int q = 0; q < SW; ++q) u.scale[t * SW + q] = __builtin_nontemporal_load(sc + q * 64) >> (8 * (ks_first & 3));
+        } else {
+            const int words = k / 512, first = ks_first / 4;
+            const uint32_t* sc = reinterpret_cast<const uint32_t*>(scales) + (size_t)ntile[t] * words * 64 + lane;
+            uint32_t raw[SW + 1];
+#pragma unroll
+            for (int q = 0; q <= SW; ++q) raw[q] = __builtin_nontemporal_load(sc + (size_t)min(first + q, words - 1) * 64);   // past the row: unused
+#pragma unroll
+            for (int q = 0; q < SW; ++q) u.scale[t * SW + q] = __builtin_amdgcn_alignbyte(raw[q + 1], raw[q], (uint32_t)(ks_first & 3));
+        }
     }
 }
 // FP8: bytes [n/16][k/128][half][lane][16 B]; scales row-major UE8M0 [n/bn][k/bk].  TILES counts 16-byte planes: tile = t / 2.
@@ -231,7 +242,7 @@ __device__ __forceinline__ int tf_tiles(const StreamArgs& p) {
 // products run.
 // Routed (FP4): rows [0, inter) are up, [inter, 2 inter) gate; h = bf16((g * logistic(g)) * u), g = min(gate, limit),
 // u = clamp(up) in FP32.  Shared (FP8): rows [0, inter) gate, then up; both rounded to BF16 first, clamped in BF16.
-template <bool FP8, int KS>
+template <bool FP8, int KS, int WAVES = 4>
 __device__ __forceinline__ void tf_fc1_items(const StreamArgs& p, int item_first, int item_last, float (*red)[2][4][64],
                                              const PlanLds& plan) {
     const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
@@ -276,7 +287,7 @@ __device__ __forceinline__ void tf_fc1_items(const StreamArgs& p, int item_first
             c0 = tf_dot_unit<false, 2, KS>(a, cur, 0);
             c1 = tf_dot_unit<false, 2, KS>(a, cur, 1);
         }
-        float (*slot)[2][4][64] = red + (item & 1) * 4;
+        float (*slot)[2][4][64] = red + (item & 1) * WAVES;
 #pragma unroll
         for (int i = 0; i < 4; ++i) { slot[wave][0][i][lane] = c0[i]; slot[wave][1][i][lane] = c1[i]; }
         __syncthreads();
@@ -287,7 +298,7 @@ __device__ __forceinline__ void tf_fc1_items(const StreamArgs& p, int item_first
                 if (m < r.valid) {
                     float first = slot[0][0][i][lane], second = slot[0][1][i][lane];
 #pragma unroll
-                    for (int w2 = 1; w2 < 4; ++w2) {
+                    for (int w2 = 1; w2 < WAVES; ++w2) {
                         first = __fadd_rn(first, slot[w2][0][i][lane]);
                         second = __fadd_rn(second, slot[w2][1][i][lane]);
                     }
@@ -427,21 +438,23 @@ __device__ __forceinline__ void tf_fc2_items(const StreamArgs& p, int item_first
 
 // Persistent launch of one phase over the routed experts and, optionally, the shared expert (`shared.w == nullptr`: routed
 // only; `routed.w == nullptr`: dense only).  Every item costs the same bytes (a shared FC1 item counts twice), so workgroup
-// b of G takes the cost range [b C / G, (b + 1) C / G) of the list "routed items, then shared items".  block = 256.
-template <int KSR, int KSS>
-__global__ void __launch_bounds__(256, 2) tf_phase1_stream(const StreamArgs routed, const StreamArgs shared) {
-    __shared__ float red[8][2][4][64];
+// b of G takes the cost range [b C / G, (b + 1) C / G) of the list "routed items, then shared items".  block = 64 WAVES:
+// four waves, two workgroups a CU, for K <= 4,096; eight waves, one workgroup a CU, above (a wave's share of K stays at
+// most eight k-steps: what the registers hold of the A tile and a unit of weights).
+template <int KSR, int KSS, int WAVES = 4>
+__global__ void __launch_bounds__(64 * WAVES, WAVES == 4 ? 2 : 1) tf_phase1_stream(const StreamArgs routed, const StreamArgs shared) {
+    __shared__ float red[2 * WAVES][2][4][64];
     __shared__ PlanLds plan;
     if (routed.w) tf_plan_preload(routed, plan);
     const long long r_items = routed.w ? (long long)plan.tiles * (routed.inter / 16) : 0;
     const long long s_units = shared.w ? (long long)tf_tiles(shared) * (shared.inter / 16) * 2 : 0;
     const long long total = r_items + s_units;
     const long long lo = total * blockIdx.x / gridDim.x, hi = total * (blockIdx.x + 1) / gridDim.x;
-    if (lo < r_items) tf_fc1_items<false, KSR>(routed, (int)lo, (int)(hi < r_items ? hi : r_items), red, plan);
+    if (lo < r_items) tf_fc1_items<false, KSR, WAVES>(routed, (int)lo, (int)(hi < r_items ? hi : r_items), red, plan);
     if (hi > r_items) {
         const long long a = (lo > r_items ? lo - r_items : 0), b = hi - r_items;
         __syncthreads();
-        tf_fc1_items<true, KSS>(shared, (int)((a + 1) / 2), (int)((b + 1) / 2), red, plan);
+        tf_fc1_items<true, KSS, WAVES>(shared, (int)((a + 1) / 2), (int)((b + 1) / 2), red, plan);
     }
 }
 template <int KSR, int KSS>
@@ -589,7 +602,11 @@ extern "C" __global__ void __launch_bounds__(512) ca_moe_route_frontend_shared(
             switch (shared.k) {
                 case 512: tf_front_shared_item<1, true>(shared, input, rows, s_pool, block, sync, quant_blocks, shared_blocks); break;
                 case 1024: tf_front_shared_item<2, true>(shared, input, rows, s_pool, block, sync, quant_blocks, shared_blocks); break;
+                case 1536: tf_front_shared_item<3, true>(shared, input, rows, s_pool, block, sync, quant_blocks, shared_blocks); break;
                 case 2048: tf_front_shared_item<4, true>(shared, input, rows, s_pool, block, sync, quant_blocks, shared_blocks); break;
+                case 2560: tf_front_shared_item<5, true>(shared, input, rows, s_pool, block, sync, quant_blocks, shared_blocks); break;
+                case 3072: tf_front_shared_item<6, true>(shared, input, rows, s_pool, block, sync, quant_blocks, shared_blocks); break;
+                case 3584: tf_front_shared_item<7, true>(shared, input, rows, s_pool, block, sync, quant_blocks, shared_blocks); break;
                 case 4096: tf_front_shared_item<8, true>(shared, input, rows, s_pool, block, sync, quant_blocks, shared_blocks); break;
                 default: break;
             }
@@ -597,7 +614,11 @@ extern "C" __global__ void __launch_bounds__(512) ca_moe_route_frontend_shared(
             switch (shared.k) {
                 case 512: tf_front_shared_item<1, false>(shared, input, rows, s_pool, block, sync, 0, shared_blocks); break;
                 case 1024: tf_front_shared_item<2, false>(shared, input, rows, s_pool, block, sync, 0, shared_blocks); break;
+                case 1536: tf_front_shared_item<3, false>(shared, input, rows, s_pool, block, sync, 0, shared_blocks); break;
                 case 2048: tf_front_shared_item<4, false>(shared, input, rows, s_pool, block, sync, 0, shared_blocks); break;
+                case 2560: tf_front_shared_item<5, false>(shared, input, rows, s_pool, block, sync, 0, shared_blocks); break;
+                case 3072: tf_front_shared_item<6, false>(shared, input, rows, s_pool, block, sync, 0, shared_blocks); break;
+                case 3584: tf_front_shared_item<7, false>(shared, input, rows, s_pool, block, sync, 0, shared_blocks); break;
                 case 4096: tf_front_shared_item<8, false>(shared, input, rows, s_pool, block, sync, 0, shared_blocks); break;
                 default: break;
             }
