@@ -72,3 +72,33 @@ def test_drafter_parameter_set():
     taps, _ = run_case(6, 1024, 128, 3, 512, 512, "reference", tokens=tokens, alt_token=-1)
     again, _ = run_case(6, 1024, 128, 3, 512, 512, "reference", tokens=[7, 1, 2, 3, 4, 5], alt_token=-1)
     assert np.array_equal(taps["ids"], again["ids"]) and np.array_equal(taps["out"], again["out"])
+
+
+@pytest.mark.parametrize("rows,experts,inter,shared", [(6, 16, 576, 576), (40, 8, 2304, 2304), (130, 8, 576, 2304)])
+def test_reference_expert_widths_run_zero_padded(rows, experts, inter, shared):
+    # the reference's expert widths (2,304; 576 a tensor-parallel rank: src/expert_packing.rs:64-66) are no multiples of 512:
+    # the host mirror uploads them with zero weight rows / columns up to the next multiple and the layer runs at that width.
+    # The oracle runs the unpadded operands; every tap must match on the real columns and be zero on the added ones.
+    g = geometry(5120, experts, 6, inter, shared, "reference")
+    name = "padded-%d-%d-%d-%d" % (rows, experts, inter, shared)
+    ops = synth.LayerOperands(g, name, device="cuda")
+    x = synth.activations(name, rows, g.hidden)
+    layer = host.Layer(g, ops, rows)
+    run = layer.run_geometry()
+    assert (run.intermediate, run.shared_intermediate) == ((inter + 511) // 512 * 512, (shared + 511) // 512 * 512)
+    layer.set_tokens()
+    layer.run(x.cuda())
+    taps = layer.taps()
+    layer.close()
+    B, I, S, Sp = g.act_block, inter, shared, run.shared_intermediate
+    for key, width in (("h", I), ("hq", I), ("hs", I // B), ("shared_act", S), ("shared_aq", S), ("shared_as", S // B)):
+        extra = taps[key][:, width:]
+        if key in ("hs", "shared_as"):     # scale bytes of all-zero blocks: 0 (routed flavour), the 1e-4 floor's byte (shared flavour)
+            assert np.all(extra == (0 if key == "hs" else 105)), key
+        else:
+            assert not np.any(extra & (0x7fff if extra.dtype == np.uint16 else 0x7f)), key
+        taps[key] = np.ascontiguousarray(taps[key][:, :width])
+    up = taps["shared_up"]
+    assert not np.any(up[:, S:Sp] & 0x7fff) and not np.any(up[:, Sp + S:] & 0x7fff)
+    taps["shared_up"] = np.ascontiguousarray(np.concatenate([up[:, :S], up[:, Sp:Sp + S]], axis=1))
+    check_layer(g, ops, x, taps, exact_logits=rows <= 16, max_rel=2e-2)

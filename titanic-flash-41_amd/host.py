@@ -180,8 +180,16 @@ class Layer:
         self._check(self.lib.tfh_layer_tap(self.h, name.encode(), out.ctypes.data, size, self._err, 512))
         return out
 
+    def run_geometry(self):
+        """The geometry the layer runs with: the given one with the expert widths padded to multiples of 512 (zero weights)."""
+        out = type(self.g)()
+        self.lib.tfh_layer_geometry.argtypes = [ctypes.c_void_p, ctypes.c_void_p]
+        self.lib.tfh_layer_geometry.restype = None
+        self.lib.tfh_layer_geometry(self.h, ctypes.byref(out))
+        return out
+
     def taps(self):
-        g, rows = self.g, self.rows
+        g, rows = self.run_geometry(), self.rows
         K, H, I, S, B = g.topk, g.hidden, g.intermediate, g.shared_intermediate, g.act_block
         t = {n: self.tap(n) for n in TAPS}
         shape = {"logits": (rows, g.experts), "ids": (rows, K), "weights": (rows, K), "xq": (rows, H), "xs": (rows, H // B),

@@ -35,8 +35,13 @@ extern "C" {
 namespace {
 void build_layer(Handle* h, const char* kernel_library, const ca_geometry* geometry, int rows, const tf::Weights::Host& src, bool on_device,
                  int overlap, int sum_shared, int route_front, int code_scales, int fold_shared, int gate_front) {
-    h->native = std::make_shared<tf::Native>(kernel_library, *geometry);
-    h->weights = on_device ? std::make_shared<tf::Weights>(*geometry, src, true) : std::make_shared<tf::Weights>(*geometry, src);
+    // expert widths that are not multiples of 512 (the reference's 2,304 / 576) run zero-padded
+    const ca_geometry run = tf::padded_geometry(*geometry);
+    tf::Weights::Host padded = src;
+    if (run.intermediate != geometry->intermediate) padded.source_intermediate = (size_t)geometry->intermediate;
+    if (run.shared_intermediate != geometry->shared_intermediate) padded.source_shared_intermediate = (size_t)geometry->shared_intermediate;
+    h->native = std::make_shared<tf::Native>(kernel_library, run);
+    h->weights = on_device ? std::make_shared<tf::Weights>(run, padded, true) : std::make_shared<tf::Weights>(run, padded);
     h->prepared = tf::prepare_layer(*h->native, *h->weights, 0);
     if (code_scales) h->scale_code = tf::code_layer_scales(*h->native, *h->weights, h->prepared);
     tf::LayerFfn::Options options;
@@ -100,6 +105,8 @@ int tfh_checkpoint_layer(const char* root, const char* prefix, const ca_geometry
     });
 }
 void tfh_layer_destroy(void* handle) { delete (Handle*)handle; }
+// The geometry the layer runs with (the caller's, with the expert widths padded to multiples of 512): the widths of the taps.
+void tfh_layer_geometry(void* handle, ca_geometry* out) { *out = ((Handle*)handle)->native->geometry(); }
 // Many rows: drop (0) or keep (1) the BF16 tap of the routed intermediate.
 void tfh_layer_keep_intermediate(void* handle, int on) { ((Handle*)handle)->workspace->keep_intermediate(on != 0); }
 

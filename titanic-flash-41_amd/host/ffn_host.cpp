@@ -104,18 +104,50 @@ void Weights::layout(const ca_geometry& g) {
     add("ffn.shared_experts.w2.prepared", H * S);
     atlas_ = Buffer<uint8_t>(at);
 }
-void Weights::fill(const Host& src, hipMemcpyKind kind) {
+ca_geometry padded_geometry(const ca_geometry& g) {
+    ca_geometry p = g;
+    p.intermediate = (g.intermediate + 511) / 512 * 512;
+    p.shared_intermediate = (g.shared_intermediate + 511) / 512 * 512;
+    return p;
+}
+void Weights::fill(const ca_geometry& g, const Host& src, hipMemcpyKind kind) {
     auto put = [&](const char* name, const void* from) {
         const View& v = view(name);
         check(hipMemcpy((void*)(atlas_.ptr() + v.offset), from, v.bytes, kind), "weight upload");
     };
+    // `count` pieces of `piece` source bytes each, `stride` bytes apart in the (zeroed) view
+    auto put_pieces = [&](const char* name, const void* from, size_t piece, size_t stride, size_t count) {
+        const View& v = view(name);
+        ensure(piece <= stride && stride * count == v.bytes, "padded weight view");
+        check(hipMemset((void*)(atlas_.ptr() + v.offset), 0, v.bytes), "weight padding");
+        check(hipMemcpy2D((void*)(atlas_.ptr() + v.offset), stride, from, piece, piece, count, kind), "weight upload");
+    };
+    const size_t H = g.hidden, E = g.experts, I = g.intermediate, S = g.shared_intermediate;
+    const size_t Is = src.source_intermediate ? src.source_intermediate : I, Ss = src.source_shared_intermediate ? src.source_shared_intermediate : S;
+    ensure(Is <= I && Ss <= S && Is % 32 == 0 && Is % (size_t)g.act_block == 0 && Ss % (size_t)g.act_block == 0 && Ss % (size_t)g.shared_bn == 0 &&
+           Ss % (size_t)g.shared_bk == 0, "narrower expert operands must end on whole quantization blocks");
     put("ffn.gate.weight", src.gate_w); put("ffn.gate.bias", src.bias); put("ffn.gate.bias_vl", src.bias_alt);
-    put("ffn.experts.w13", src.w13); put("ffn.experts.w2", src.w2); put("ffn.experts.s13", src.s13); put("ffn.experts.s2", src.s2);
-    put("ffn.shared_experts.w13.weight", src.sh_w13); put("ffn.shared_experts.w13.scale", src.sh_s13);
-    put("ffn.shared_experts.w2.weight", src.sh_w2); put("ffn.shared_experts.w2.scale", src.sh_s2);
+    if (Is == I) {
+        put("ffn.experts.w13", src.w13); put("ffn.experts.w2", src.w2); put("ffn.experts.s13", src.s13); put("ffn.experts.s2", src.s2);
+    } else {
+        put_pieces("ffn.experts.w13", src.w13, Is * H / 2, I * H / 2, 2 * E);          // per expert: up rows, gate rows
+        put_pieces("ffn.experts.s13", src.s13, Is * H / 32, I * H / 32, 2 * E);
+        put_pieces("ffn.experts.w2", src.w2, Is / 2, I / 2, E * H);                     // per output row: its K columns
+        put_pieces("ffn.experts.s2", src.s2, Is / 32, I / 32, E * H);
+    }
+    if (Ss == S) {
+        put("ffn.shared_experts.w13.weight", src.sh_w13); put("ffn.shared_experts.w13.scale", src.sh_s13);
+        put("ffn.shared_experts.w2.weight", src.sh_w2); put("ffn.shared_experts.w2.scale", src.sh_s2);
+    } else {
+        const size_t bn = g.shared_bn, bk = g.shared_bk;
+        put_pieces("ffn.shared_experts.w13.weight", src.sh_w13, Ss * H, S * H, 2);      // gate rows, up rows
+        put_pieces("ffn.shared_experts.w13.scale", src.sh_s13, (Ss / bn) * (H / bk), (S / bn) * (H / bk), 2);
+        put_pieces("ffn.shared_experts.w2.weight", src.sh_w2, Ss, S, H);
+        put_pieces("ffn.shared_experts.w2.scale", src.sh_s2, Ss / bk, S / bk, H / bn);
+    }
 }
-Weights::Weights(const ca_geometry& g, const Host& host) { layout(g); fill(host, hipMemcpyHostToDevice); }
-Weights::Weights(const ca_geometry& g, const Host& device, bool) { layout(g); fill(device, hipMemcpyDeviceToDevice); }
+Weights::Weights(const ca_geometry& g, const Host& host) { layout(g); fill(g, host, hipMemcpyHostToDevice); }
+Weights::Weights(const ca_geometry& g, const Host& device, bool) { layout(g); fill(g, device, hipMemcpyDeviceToDevice); }
 const View& Weights::view(const std::string& name) const {
     auto it = views_.find(name);
     if (it == views_.end()) throw Error("unknown weight view " + name);

@@ -64,6 +64,13 @@ private:
     int (*pack_bf16_)(const void*, uint8_t*, int, int, void*) = nullptr;
 };
 
+// The kernels take expert widths that are multiples of 512; the reference's are 2,304 (576 a tensor-parallel rank,
+// src/expert_packing.rs:64-66).  Returns `g` with both intermediate widths rounded up to the next multiple of 512: a layer
+// built for that geometry from operands of the narrower widths (Weights::Host::source_*) computes the same outputs, since the
+// added up / gate rows are zero (their activation columns are exactly zero, as are their codes, and whole quantization
+// blocks of them do not touch a real block's scale) and the added down-projection columns multiply those zeros.
+ca_geometry padded_geometry(const ca_geometry& g);
+
 // ---- device atlas (src/weights.rs:276-417: contiguous expert groups, 256-byte aligned views) --------------------------
 struct View { size_t offset = 0, bytes = 0; };
 class Weights {
@@ -73,6 +80,10 @@ public:
         const uint16_t* gate_w; const float* bias; const float* bias_alt;
         const uint8_t* w13; const uint8_t* s13; const uint8_t* w2; const uint8_t* s2;
         const uint8_t* sh_w13; const uint8_t* sh_s13; const uint8_t* sh_w2; const uint8_t* sh_s2;
+        // Expert widths of the operands above when they are narrower than the geometry's (0: the same): the atlas is then
+        // filled with zero weight rows (w13) and zero weight columns (w2) up to the geometry's widths, which changes no
+        // result (see padded_geometry).
+        size_t source_intermediate = 0, source_shared_intermediate = 0;
     };
     Weights(const ca_geometry& g, const Host& host);
     // Same, from device-resident canonical operands (copied device to device into the atlas).
@@ -87,7 +98,7 @@ public:
     size_t bytes() const { return atlas_.bytes(); }
 private:
     void layout(const ca_geometry& g);
-    void fill(const Host& src, hipMemcpyKind kind);
+    void fill(const ca_geometry& g, const Host& src, hipMemcpyKind kind);
     Buffer<uint8_t> atlas_;
     std::map<std::string, View> views_;
     bool expert_ready_ = false;
