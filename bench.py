@@ -1,7 +1,7 @@
 #!/usr/bin/env python3
 """Benchmark of the MoE FFN layer on one MI355X.
 
-    python bench.py [--gpus 1] [--steps K] [--warmup W] [--config c2|c3|c4|c5] [--numerics benchmark|reference]
+    python bench.py [--gpus 1] [--steps K] [--warmup W] [--config c2|c3|c4|c5|r6|r4096] [--numerics benchmark|reference]
 
 A step is one pass of the whole layer (gate product, top-k + plan + token quantization, routed FC1 + SwiGLU, FC2, shared
 expert, ordered sum + shared addition) over one batch of synthetic token rows that is already resident in HBM, replayed
@@ -38,6 +38,12 @@ CONFIGS = {
                workload="prefill chunk of 4096 tokens, uniform routing; H 4096, E 256, top-6, I 2048, 1 shared expert"),
     "c5": dict(rows=16384, hidden=4096, experts=256, topk=6, inter=2048, shared=2048,
                workload="long prefill of 16384 tokens, Zipf(1.1) expert popularity; H 4096, E 256, top-6, I 2048, 1 shared expert"),
+    # not benchmark configurations: the reference's own layer (runtime/model/config.json; src/ffn.rs:65-66, 245-258), in its own numerics
+    # unless --numerics says otherwise.  The expert widths (2,304) are uploaded zero-padded to 2,560; bytes and flops below count 2,304.
+    "r6": dict(rows=6, hidden=5120, experts=384, topk=6, inter=2304, shared=2304,
+               workload="the reference's layer, decode / verify plan of 6 rows; H 5120, E 384, top-6, I 2304, 1 shared expert (I 2304)"),
+    "r4096": dict(rows=4096, hidden=5120, experts=384, topk=6, inter=2304, shared=2304,
+                  workload="the reference's layer, prefill chunk of 4096 tokens; H 5120, E 384, top-6, I 2304, 1 shared expert (I 2304)"),
 }
 MFMA_FP8_PEAK_TFLOPS, MFMA_FP4_PEAK_TFLOPS = 5000.0, 10100.0
 # Measured HBM traffic of the dominant kernel over its algorithmic bytes, from the counter runs summarized under profiles/
@@ -119,7 +125,7 @@ def main():
     ap.add_argument("--steps", type=int, default=2000)
     ap.add_argument("--warmup", type=int, default=200)
     ap.add_argument("--config", default="c2", choices=sorted(CONFIGS))
-    ap.add_argument("--numerics", default="benchmark", choices=["benchmark", "reference"],
+    ap.add_argument("--numerics", default=None, choices=["benchmark", "reference"],
                     help="benchmark: sigmoid scores, renormalised, 128-wide activation blocks, 128 x 128 shared weight blocks (the headline); "
                          "reference: the reference's own numerics (sqrt-softplus x 1.5, 32-wide blocks, 32 x 32, image-token bias)")
     ap.add_argument("--no-cpu-baseline", action="store_true")
@@ -135,6 +141,8 @@ def main():
     pkg = importlib.import_module("titanic-flash-41_amd")
     native, synth, host = pkg.native, pkg.synth, pkg.host
     cfg = CONFIGS[args.config]
+    if args.numerics is None:
+        args.numerics = "reference" if args.config.startswith("r") else "benchmark"
     if args.numerics == "benchmark":
         g = native.Geometry(cfg["hidden"], cfg["experts"], cfg["topk"], cfg["inter"], cfg["shared"], 0, 1.0, 128, 128, 128, -1, 10.0)
     else:
