@@ -240,15 +240,22 @@ def ctypes_i64(v):
 
 
 @pytest.mark.gpu
-@pytest.mark.parametrize("rows", [128, 512])
-def test_gpu_row_transport_pass_equals_the_ordinary_pass(rows):
+@pytest.mark.parametrize("rows,hidden", [(128, 1024), (512, 1024), (128, 5120)])
+def test_gpu_row_transport_pass_equals_the_ordinary_pass(rows, hidden):
     """The one-rank row transport (pack -> routed experts from the wire rows, shared expert from the decoded codes) must give the
     ordinary pass's output bit for bit: both quantizers are reproduced exactly, everything downstream is the same kernels.
-    Reference numerics (32-wide blocks), the small parity geometry at many rows (grouped-GEMM regime)."""
-    from helpers import pkg
+    Reference numerics (32-wide blocks), the small parity geometry at many rows (grouped-GEMM regime), and the reference's
+    token width (wire rows of 5,920 bytes: src/moe.rs:512-583)."""
+    from helpers import geometry, pkg, synth
     from test_gpu_layer import check_layer, make
     host = pkg.host
-    g, ops, x, rows = make("c1", "reference", "cuda", rows=rows, seed_name="codec/transport/%d" % rows)
+    if hidden == 1024:
+        g, ops, x, rows = make("c1", "reference", "cuda", rows=rows, seed_name="codec/transport/%d" % rows)
+    else:
+        g = geometry(hidden, 16, 6, 512, 512, "reference")
+        ops = synth.LayerOperands(g, "codec/transport/wide", device="cuda")
+        x = synth.activations("codec/transport/wide", rows, hidden, device="cuda")
+        assert oracle.codec_row_bytes(hidden) == 5920
     layer = host.Layer(g, ops, rows, overlap=False, sum_shared=False)
     layer.set_tokens()
     print("ordinary pass", rows, flush=True)
