@@ -70,6 +70,14 @@ def test_argument_validation_needs_no_device():
     assert lib.ca_ffn_configure(None) == -1
     good = native.Geometry(1024, 16, 2, 512, 512, 0, 1.0, 128, 128, 128, -1, 10.0)
     assert lib.ca_ffn_configure(ctypes.byref(good)) == 0
+    # accepted widths: token rows of a multiple of 512 up to 4,096 or of 1,024 up to 8,192; expert widths multiples of 512 up to 4,096
+    # (the reference's 5,120 token width is one; its expert width 576 / 2,304 goes in padded: 1,024 / 2,560)
+    for hidden, inter, shared, want in [(5120, 2560, 2560, 0), (5120, 1024, 1024, 0), (8192, 4096, 512, 0), (3584, 1536, 3072, 0),
+                                        (5120, 576, 576, -4), (5120, 2304, 2304, -4), (4608, 512, 512, -4), (9216, 512, 512, -4),
+                                        (4096, 4608, 512, -4), (4096, 512, 8192, -4)]:
+        trial = native.Geometry(hidden, 384, 6, inter, shared, 1, 1.5, 32, 32, 32, 129264, 10.0)
+        assert lib.ca_ffn_configure(ctypes.byref(trial)) == want, (hidden, inter, shared)
+    assert lib.ca_ffn_configure(ctypes.byref(good)) == 0
     back = native.Geometry()
     assert lib.ca_ffn_geometry(ctypes.byref(back)) == 0 and (back.hidden, back.experts, back.act_block) == (1024, 16, 128)
     assert lib.ca_router_logits(0, None, None, None, None) == -1 and lib.ca_router_logits(17, None, None, None, None) == -1

@@ -24,6 +24,7 @@ int check_geometry(const ca_geometry& g) {
         g.shared_bn <= 0 || g.shared_bk <= 0 || g.shared_bk % 32 || g.hidden % g.shared_bk || g.shared_intermediate % g.shared_bk ||
         g.hidden % g.shared_bn || (2 * g.shared_intermediate) % g.shared_bn)
         return -4;
+    if (!supported_hidden(g.hidden) || !supported_k(g.intermediate) || !supported_k(g.shared_intermediate)) return -4;
     return 0;
 }
 int launch_status() { return (int)hipGetLastError(); }
