@@ -90,8 +90,10 @@ int64_t ca_primitives_scratch_bytes(void* context, int32_t index, int32_t rows);
 /* No counterpart in the reference (its per-node timings come from CUDA events around whole graph launches,
  * src/moe.rs:1261-1300): a profiling aid.  With five hipEvent_t in `events`, every later launch of entries 0, 1 and 9 on this
  * context records them on the launch stream: [0] before the first kernel, [1] after the front-end, [2] after FC1 + SwiGLU,
- * [3] after FC2, [4] after the ordered sum (entry 9 with outputs only).  count 0 turns it off.  Not for use while the
- * stream is being captured.  0, or -1 for a null context / event or a count other than 0 or 5. */
+ * [3] after FC2, [4] after the ordered sum (entry 9 with outputs only).  With seven, [5] and [6] also take the start and the
+ * completion of the few-row FC1 + SwiGLU kernel itself (without the gap to its neighbours that [1] .. [2] includes).
+ * count 0 turns it off.  Not for use while the stream is being captured.  0, or -1 for a null context / event or a count
+ * other than 0, 5 or 7. */
 int32_t ca_primitives_marks(void* context, void* const* events, size_t count);
 
 #ifdef __cplusplus

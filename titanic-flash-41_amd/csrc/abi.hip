@@ -7,6 +7,7 @@
 #include "experts_stream.cuh"
 #include "packing.cuh"
 #include "shared.cuh"
+#include <hip/hip_ext.h>
 #include <cstdlib>
 #include <cstring>
 
@@ -33,8 +34,9 @@ struct Context {
     ca_geometry g;
     int cus;
     int stream_wgs;    // persistent workgroups of the streaming kernels
-    hipEvent_t marks[5];   // profiling aid: see ca_primitives_marks
+    hipEvent_t marks[7];   // profiling aid: see ca_primitives_marks
     bool marking;
+    bool kernel_marks;     // marks[5], marks[6]: begin and end of the FC1 + SwiGLU kernel itself
 };
 
 // Records mark `i` on the launch stream when the caller asked for marks (never while a stream is captured: the caller's duty).
@@ -43,23 +45,28 @@ void mark(const Context& c, int i, hipStream_t s) {
 }
 
 // Phase launches of the streaming kernels; either operand set may be absent (w == nullptr).
-int launch_phase1(const StreamArgs& routed, const StreamArgs& shared, int wgs, hipStream_t s) {
+// `begin` / `end` (both or neither): events that take the kernel's own start and completion times (hipExtLaunchKernelGGL).
+int launch_phase1(const StreamArgs& routed, const StreamArgs& shared, int wgs, hipStream_t s, hipEvent_t begin = nullptr, hipEvent_t end = nullptr) {
     const int k = routed.w ? routed.k : shared.k;
     if (routed.w && shared.w && routed.k != shared.k) return -4;
     const int wide = wgs >= 2 ? wgs / 2 : 1;       // eight-wave workgroups: one a CU
+    auto go = [&](auto kernel, int grid, int block) {
+        if (begin != nullptr && end != nullptr) hipExtLaunchKernelGGL(kernel, dim3(grid), dim3(block), 0, s, begin, end, 0, routed, shared);
+        else kernel<<<grid, block, 0, s>>>(routed, shared);
+    };
     switch (k) {
-        case 512: tf_phase1_stream<1, 1><<<wgs, 256, 0, s>>>(routed, shared); break;
-        case 1024: tf_phase1_stream<2, 2><<<wgs, 256, 0, s>>>(routed, shared); break;
-        case 1536: tf_phase1_stream<3, 3><<<wgs, 256, 0, s>>>(routed, shared); break;
-        case 2048: tf_phase1_stream<4, 4><<<wgs, 256, 0, s>>>(routed, shared); break;
-        case 2560: tf_phase1_stream<5, 5><<<wgs, 256, 0, s>>>(routed, shared); break;
-        case 3072: tf_phase1_stream<6, 6><<<wgs, 256, 0, s>>>(routed, shared); break;
-        case 3584: tf_phase1_stream<7, 7><<<wgs, 256, 0, s>>>(routed, shared); break;
-        case 4096: tf_phase1_stream<8, 8><<<wgs, 256, 0, s>>>(routed, shared); break;
-        case 5120: tf_phase1_stream<5, 5, 8><<<wide, 512, 0, s>>>(routed, shared); break;
-        case 6144: tf_phase1_stream<6, 6, 8><<<wide, 512, 0, s>>>(routed, shared); break;
-        case 7168: tf_phase1_stream<7, 7, 8><<<wide, 512, 0, s>>>(routed, shared); break;
-        case 8192: tf_phase1_stream<8, 8, 8><<<wide, 512, 0, s>>>(routed, shared); break;
+        case 512: go(tf_phase1_stream<1, 1, 4>, wgs, 256); break;
+        case 1024: go(tf_phase1_stream<2, 2, 4>, wgs, 256); break;
+        case 1536: go(tf_phase1_stream<3, 3, 4>, wgs, 256); break;
+        case 2048: go(tf_phase1_stream<4, 4, 4>, wgs, 256); break;
+        case 2560: go(tf_phase1_stream<5, 5, 4>, wgs, 256); break;
+        case 3072: go(tf_phase1_stream<6, 6, 4>, wgs, 256); break;
+        case 3584: go(tf_phase1_stream<7, 7, 4>, wgs, 256); break;
+        case 4096: go(tf_phase1_stream<8, 8, 4>, wgs, 256); break;
+        case 5120: go(tf_phase1_stream<5, 5, 8>, wide, 512); break;
+        case 6144: go(tf_phase1_stream<6, 6, 8>, wide, 512); break;
+        case 7168: go(tf_phase1_stream<7, 7, 8>, wide, 512); break;
+        case 8192: go(tf_phase1_stream<8, 8, 8>, wide, 512); break;
         default: return -4;
     }
     return launch_status();
@@ -236,7 +243,7 @@ int launch_dynamic(const Context& c, bool route, const uint64_t* p, const int32_
         b.w_expert_stride = w2_stride; b.ws_expert_stride = s2_stride;
         b.k = g.intermediate; b.out = (uint16_t*)p[P_SCATTER];
         if (phases & 2) {
-            status = launch_phase1(a, sa, c.stream_wgs, s);
+            status = c.marking && c.kernel_marks ? launch_phase1(a, sa, c.stream_wgs, s, c.marks[5], c.marks[6]) : launch_phase1(a, sa, c.stream_wgs, s);
             if (status) return status;
         }
         mark(c, 2, s);
@@ -482,11 +489,12 @@ void* ca_primitives_open(int32_t* status) {
 }
 void ca_primitives_close(void* context) { delete (Context*)context; }
 int32_t ca_primitives_marks(void* context, void* const* events, size_t count) {
-    if (!context || (count != 0 && (count != 5 || !events))) return -1;
+    if (!context || (count != 0 && ((count != 5 && count != 7) || !events))) return -1;
     Context* c = (Context*)context;
-    c->marking = count == 5;
+    c->marking = count != 0;
+    c->kernel_marks = count == 7;
     for (size_t i = 0; i < count; ++i) {
-        if (!events[i]) { c->marking = false; return -1; }
+        if (!events[i]) { c->marking = c->kernel_marks = false; return -1; }
         c->marks[i] = (hipEvent_t)events[i];
     }
     return 0;

@@ -36,7 +36,7 @@ def load():
         lib.tfh_layer_time.argtypes = [vp, ctypes.POINTER(ctypes.c_int), ctypes.c_int, ctypes.c_int, ctypes.c_int, ctypes.POINTER(ctypes.c_float), cp, sz]
         lib.tfh_layer_time_phase.argtypes = [vp, ctypes.c_int, ctypes.c_uint64, ctypes.c_int, ctypes.POINTER(ctypes.c_float), cp, sz]
         lib.tfh_layer_profile_step.argtypes = [vp, ctypes.c_uint64, ctypes.POINTER(ctypes.c_float), cp, sz]
-        lib.tfh_layer_profile_marks.argtypes = [vp, ctypes.POINTER(ctypes.c_uint64), ctypes.c_int, ctypes.c_int, ctypes.POINTER(ctypes.c_float), cp, sz]
+        lib.tfh_layer_profile_marks.argtypes = [vp, ctypes.POINTER(ctypes.c_uint64), ctypes.c_int, ctypes.c_int, ctypes.c_int, ctypes.POINTER(ctypes.c_float), cp, sz]
         lib.tfh_layer_pair_run.argtypes = [vp, ctypes.c_uint64, ctypes.POINTER(ctypes.c_int64), ctypes.c_int, ctypes.c_uint64, ctypes.POINTER(ctypes.c_int64),
                                            ctypes.c_int, vp, vp, cp, sz]
         lib.tfh_layer_tap.restype = ctypes.c_longlong
@@ -156,12 +156,15 @@ class Layer:
         self._check(self.lib.tfh_layer_profile_step(self.h, x.data_ptr(), ms, self._err, 512))
         return list(ms)
 
-    def profile_marks(self, xs, passes):
-        """Mean milliseconds of (front-end, FC1 + SwiGLU, FC2, sum, first mark to last) over `passes` eager passes of the
-        layer's own schedule cycling through the inputs `xs`; events are recorded between the launches on the launch stream."""
+    def profile_marks(self, xs, passes, exact=False):
+        """Mean milliseconds of (front-end, FC1 + SwiGLU, FC2, sum, first mark to last, the FC1 + SwiGLU kernel alone) over `passes`
+        eager passes of the layer's own schedule cycling through the inputs `xs`.  The first five are intervals between events
+        recorded between the launches on the launch stream (a launch plus the gap to its neighbour); the last is between two
+        events that take the kernel's own start and completion (`exact` runs only, whose other intervals carry that launch path's
+        overhead; few rows only; 0 otherwise)."""
         ptrs = (ctypes.c_uint64 * len(xs))(*[x.data_ptr() for x in xs])
-        ms = (ctypes.c_float * 5)()
-        self._check(self.lib.tfh_layer_profile_marks(self.h, ptrs, len(xs), passes, ms, self._err, 512))
+        ms = (ctypes.c_float * 6)()
+        self._check(self.lib.tfh_layer_profile_marks(self.h, ptrs, len(xs), passes, int(exact), ms, self._err, 512))
         return list(ms)
 
     def pair_run(self, xa, tokens_a, live_a, xb, tokens_b, live_b):

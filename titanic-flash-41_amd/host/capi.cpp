@@ -235,29 +235,34 @@ int tfh_layer_profile_step(void* handle, uint64_t input, float* milliseconds, ch
 // the library's marks around every launch of the dynamic entry: mean milliseconds of [0] front-end (gate product, top-k, plan,
 // quantizers), [1] FC1 + SwiGLU, [2] FC2, [3] ordered sum + shared addition, [4] first mark to last.  Needs the schedule that
 // keeps the shared expert inside the routed launches (otherwise there is no sum mark).
-int tfh_layer_profile_marks(void* handle, const uint64_t* inputs, int count, int passes, float* milliseconds, char* error, size_t error_len) {
+// `exact` != 0: the FC1 + SwiGLU kernel is launched with a pair of events that take its own start and completion
+// (milliseconds[5]); that launch path costs a few microseconds more per pass, so the launch-to-launch intervals of such a
+// run are not the schedule's.
+int tfh_layer_profile_marks(void* handle, const uint64_t* inputs, int count, int passes, int exact, float* milliseconds, char* error, size_t error_len) {
     Handle* h = (Handle*)handle;
     return guarded(error, error_len, [&] {
         tf::ensure(count >= 1 && passes >= 1, "profile needs inputs and passes");
         std::vector<std::unique_ptr<tf::Event>> events;
-        for (int i = 0; i < 5 * passes; ++i) events.push_back(std::make_unique<tf::Event>(true));
+        for (int i = 0; i < 7 * passes; ++i) events.push_back(std::make_unique<tf::Event>(true));
         const size_t n = h->rows * (size_t)h->native->geometry().hidden;
         try {
             for (int pass = 0; pass < passes; ++pass) {
-                hipEvent_t raw[5];
-                for (int i = 0; i < 5; ++i) raw[i] = events[5 * pass + i]->raw();
-                h->native->marks(raw);
+                hipEvent_t raw[7];
+                for (int i = 0; i < 7; ++i) raw[i] = events[7 * pass + i]->raw();
+                h->native->marks(raw, exact ? 7 : 5);
                 h->layer->run(*h->workspace, inputs[pass % count], n, *h->tokens, *h->stream);
             }
         } catch (...) { h->native->marks(nullptr); throw; }
         h->native->marks(nullptr);
         h->stream->synchronize();
-        double sum[5] = {0, 0, 0, 0, 0};
+        // [0 .. 3]: front-end, FC1 + SwiGLU, FC2, sum (launch to launch); [4]: first mark to last; [5]: the FC1 + SwiGLU kernel alone
+        double sum[6] = {0, 0, 0, 0, 0, 0};
         for (int pass = 0; pass < passes; ++pass) {
-            for (int i = 0; i < 4; ++i) sum[i] += events[5 * pass + i + 1]->elapsed_since(*events[5 * pass + i]);
-            sum[4] += events[5 * pass + 4]->elapsed_since(*events[5 * pass]);
+            for (int i = 0; i < 4; ++i) sum[i] += events[7 * pass + i + 1]->elapsed_since(*events[7 * pass + i]);
+            sum[4] += events[7 * pass + 4]->elapsed_since(*events[7 * pass]);
+            if (exact) sum[5] += events[7 * pass + 6]->elapsed_since(*events[7 * pass + 5]);
         }
-        for (int i = 0; i < 5; ++i) milliseconds[i] = (float)(sum[i] / passes);
+        for (int i = 0; i < 6; ++i) milliseconds[i] = (float)(sum[i] / passes);
     });
 }
 // Paired owners: a second LayerFfn over the same prepared layer and the pooled workspace.  Runs owner A (the handle's layer,

@@ -44,8 +44,8 @@ Native::~Native() {
     if (ctx_ && close_) close_(ctx_);
     if (lib_) dlclose(lib_);
 }
-void Native::marks(hipEvent_t* events) const {
-    ensure(marks_(ctx_, (void* const*)events, events ? 5 : 0) == 0, "profiling marks rejected");
+void Native::marks(hipEvent_t* events, size_t count) const {
+    ensure(marks_(ctx_, (void* const*)events, events ? count : 0) == 0, "profiling marks rejected");
 }
 void Native::codec_encode(uint64_t routed, uint64_t scales, uint64_t shared, uint64_t packed, int rows, int k, hipStream_t s) const {
     ensure(encode_((const uint8_t*)routed, (const uint8_t*)scales, (const uint8_t*)shared, (uint8_t*)packed, rows, k, s) == 0, "packed MoE encode launch");   // src/ffn.rs:856-858

@@ -39,7 +39,7 @@ public:
     void primitive(int index, const uint64_t* pointers, size_t np, const int32_t* scalars, size_t ns, hipStream_t s, const char* what) const;
     int64_t scratch_bytes(int index, int rows) const;
     // five events recorded around the launches of the dynamic entries (null: off)
-    void marks(hipEvent_t* events) const;
+    void marks(hipEvent_t* events, size_t count = 5) const;      // 5: between the launches; 7: + the FC1 kernel's own begin / end
     // the wire row "dual_quant_rows_v1" (src/ffn.rs:805-811 RowTransport's functions)
     void codec_encode(uint64_t routed, uint64_t scales, uint64_t shared, uint64_t packed, int rows, int k, hipStream_t s) const;
     void codec_decode(uint64_t packed, uint64_t shared, uint64_t row_scales, uint64_t mma_scales, int rows, int k, hipStream_t s) const;

@@ -22,7 +22,7 @@ void* tfh_layer_create(const char*, const ca_geometry*, int, const void* const*,
 void tfh_layer_destroy(void*);
 int tfh_layer_set_tokens(void*, const int64_t*, int, const int32_t*, char*, size_t);
 int tfh_layer_run(void*, uint64_t, char*, size_t);
-int tfh_layer_profile_marks(void*, const uint64_t*, int, int, float*, char*, size_t);
+int tfh_layer_profile_marks(void*, const uint64_t*, int, int, int, float*, char*, size_t);
 long long tfh_layer_tap(void*, const char*, void*, size_t, char*, size_t);
 }
 
@@ -106,9 +106,9 @@ int main(int argc, char** argv) {
     const double fc1_bytes = tiles * (2.0 * I * H / 2 + 2.0 * I * H / 32) + (early_shared ? 0.0 : 2.0 * S * H) + rows * (2.0 * H + K * I * 2 + 2.0 * S);
     const double fc2_bytes = tiles * (1.0 * H * I / 2 + 1.0 * H * I / 32) + 1.0 * H * S + rows * (K * I * 2 + K * H * 2 + 2.0 * S + 2.0 * H);
     std::printf("{\"tiles\": %.3f, \"fc1_algorithmic_bytes\": %.0f, \"fc2_algorithmic_bytes\": %.0f}\n", tiles, fc1_bytes, fc2_bytes);
-    float ms[5] = {0, 0, 0, 0, 0};
+    float ms[6] = {0, 0, 0, 0, 0, 0};
     if (rows <= 64) {
-        if (tfh_layer_profile_marks(layer, inputs.data(), batches, passes, ms, error, sizeof error)) { std::fprintf(stderr, "profile: %s\n", error); return 1; }
+        if (tfh_layer_profile_marks(layer, inputs.data(), batches, passes, 0, ms, error, sizeof error)) { std::fprintf(stderr, "profile: %s\n", error); return 1; }
     } else {       // many rows: another schedule (no marks); the passes are there for the profiler
         for (int i = 0; i < passes; ++i)
             if (tfh_layer_run(layer, inputs[i % batches], error, sizeof error)) { std::fprintf(stderr, "run: %s\n", error); return 1; }
