@@ -449,7 +449,11 @@ __global__ void __launch_bounds__(64 * WAVES, WAVES == 4 ? 2 : 1) tf_phase1_stre
     const long long r_items = routed.w ? (long long)plan.tiles * (routed.inter / 16) : 0;
     const long long s_units = shared.w ? (long long)tf_tiles(shared) * (shared.inter / 16) * 2 : 0;
     const long long total = r_items + s_units;
-    const long long lo = total * blockIdx.x / gridDim.x, hi = total * (blockIdx.x + 1) / gridDim.x;
+    // equal shares for as many workgroups as fill whole rounds: with every workgroup of the grid taking floor or ceil of
+    // total / grid items, the last round runs on a part of the chip that is too small to keep the memory system busy
+    const long long rounds = (total + gridDim.x - 1) / gridDim.x, active = rounds > 0 ? (total + rounds - 1) / rounds : 0;
+    if ((long long)blockIdx.x >= active) return;
+    const long long lo = total * blockIdx.x / active, hi = total * (blockIdx.x + 1) / active;
     if (lo < r_items) tf_fc1_items<false, KSR, WAVES>(routed, (int)lo, (int)(hi < r_items ? hi : r_items), red, plan);
     if (hi > r_items) {
         const long long a = (lo > r_items ? lo - r_items : 0), b = hi - r_items;
