@@ -84,6 +84,8 @@ def test_argument_validation_needs_no_device():
     assert lib.ca_shared_swiglu(0, None, None, None) == -1 and lib.ca_ffn_add(70000, None, None, None, None) == -1
     assert lib.ca_moe_nibble_permute(None, 16, 0, None) == -1
     assert lib.ca_primitives_launch(None, 0, None, 0, None, 0, None) == -1
+    # the profiling marks take none, five (between the launches) or seven events (+ the FC1 kernel's own start / completion)
+    assert lib.ca_primitives_marks(None, None, 0) == -1
     grid = (ctypes.c_uint32 * 3)(1, 1, 1)
     assert lib.ca_kernel_launch(b"no_such_kernel", grid, grid, 0, (ctypes.c_void_p * 1)(), None) == -3
 

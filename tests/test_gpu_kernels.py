@@ -242,6 +242,12 @@ def test_error_conventions():
     assert native.primitives_launch(ctx, 2, [None, None, None], [1, 0, 0]) == -1
     bad = geometry(1000, 16, 2, 512, 512)
     assert lib.ca_ffn_configure(ctypes.byref(bad)) == -4
+    # profiling marks: none, five or seven events
+    dummy = (ctypes.c_void_p * 7)(*[1] * 7)
+    assert lib.ca_primitives_marks(ctypes.c_void_p(ctx), dummy, 6) == -1
+    dummy[6] = None
+    assert lib.ca_primitives_marks(ctypes.c_void_p(ctx), dummy, 7) == -1
+    assert lib.ca_primitives_marks(ctypes.c_void_p(ctx), None, 0) == 0
     with pytest.raises(RuntimeError):
         native.launch("no_such_kernel", 1, 64, [])
 
