@@ -129,6 +129,9 @@ def main():
                     help="benchmark: sigmoid scores, renormalised, 128-wide activation blocks, 128 x 128 shared weight blocks (the headline); "
                          "reference: the reference's own numerics (sqrt-softplus x 1.5, 32-wide blocks, 32 x 32, image-token bias)")
     ap.add_argument("--no-cpu-baseline", action="store_true")
+    ap.add_argument("--overlap", type=int, default=None, choices=[0, 1],
+                    help="many rows: the shared expert on a second stream beside the routed experts (the reference's dual-stream schedule, "
+                         "src/ffn.rs:1000-1040) or after them on the same stream; default: the layer's own choice")
     ap.add_argument("--copy-probe", action="store_true", help="append four 256 MiB device copies (counter calibration)")
     ap.add_argument("--profile-steps", type=int, default=64, help="eager passes with per-kernel HIP events for the roofline")
     args = ap.parse_args()
@@ -158,7 +161,7 @@ def main():
     if args.config == "c5":      # expert popularity ~ rank^-1.1: the busiest experts take more than ten times the mean load
         ops.bias = synth.zipf_bias(g.experts, 1.1, 0.06, device="cuda")
     xs = make_inputs(synth, args.config, cfg, "cuda", batches)
-    layer = host.Layer(g, ops, cfg["rows"])
+    layer = host.Layer(g, ops, cfg["rows"]) if args.overlap is None else host.Layer(g, ops, cfg["rows"], overlap=bool(args.overlap))
     layer.set_tokens()
     layer.keep_intermediate(False)      # many rows: FC2 reads the FP8 codes; the BF16 copy is a tap the tests ask for
     setup_s = time.time() - t0
