@@ -240,6 +240,8 @@ def bf16_ulp_distance(got_u16, want_u16, accumulation=1e-4):
     """Largest |got - want| in units of the allowance 2^-7 |want| (one BF16 rounding step) + `accumulation` * max |want|
     (FP32 / matrix-core accumulation-order noise of a dot product, which does not shrink with the result)."""
     gv, wv = bf(got_u16), bf(want_u16)
+    if wv.size == 0:          # nothing to compare (no live route)
+        return 0.0
     allowance = np.abs(wv) * 2.0 ** -7 + accumulation * np.abs(wv).max() + 1e-300
     return float((np.abs(gv - wv) / allowance).max())
 
@@ -251,5 +253,7 @@ def bf(a):
 def error_stats(got_u16, want_u16):
     """(max relative error against the reference's largest magnitude per row, mean absolute error)."""
     g, w = bf(got_u16), bf(want_u16)
+    if w.size == 0:
+        return 0.0, 0.0
     scale = np.abs(w).max() + 1e-30
     return float(np.abs(g - w).max() / scale), float(np.abs(g - w).mean())

@@ -56,6 +56,15 @@ def test_one_live_row_of_a_wider_owner():
     assert (taps["ids"][1:] == -1).all() and not taps["weights"][1:].any()
 
 
+@pytest.mark.parametrize("rows", [8, 40, 130])
+def test_no_live_row(rows):
+    # live = 0 (src/ffn.rs:121-126 admits it): no route is active, the plan has no tile, the expert launches have no item; the
+    # routed output is zero and the layer output is the shared expert's rows past the live prefix as the oracle defines them
+    taps, _ = run_case(rows, 1024, 16, 2, 512, 512, "reference", live=0)
+    assert np.all(taps["ids"] < 0) or np.all(taps["ids"] >= 16)
+    assert not np.any(taps["routed"] & 0x7fff)
+
+
 def test_many_rows_with_a_live_prefix_and_padding_rows():
     rows = 200
     padding = [-1] * rows
