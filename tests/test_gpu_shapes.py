@@ -40,6 +40,8 @@ def run_case(rows, hidden, experts, topk, inter, shared, mode, live=None, paddin
     (64, 1024, 32, 4, 512, 512, "reference"),       # the last row count of the streaming path
     (65, 1024, 32, 4, 512, 512, "benchmark"),       # the first of the grouped-GEMM path
     (130, 2048, 16, 2, 1024, 1024, "reference"),    # a second, partly filled row tile; K 1024 in FC2
+    (64, 1024, 8, 8, 512, 512, "benchmark"),        # every row to every expert: four full 16-row tiles an expert, 512 routes in the one-block plan
+    (200, 1024, 8, 8, 512, 512, "reference"),       # the same at many rows: two 128-row tiles an expert, the second partly filled
     (6, 5120, 32, 6, 2560, 2560, "reference"),      # the reference's token width (src/ffn.rs:65-66): eight-wave FC1 launch, five k-steps a wave
     (40, 5120, 64, 6, 1536, 512, "benchmark"),      # the same with three row tiles; K 1536 in FC2 (three k-steps a wave: scale words straddled)
     (130, 5120, 32, 2, 1024, 512, "reference"),     # many rows at that width: 160 activation scale bytes a row, staged in two passes
