@@ -124,3 +124,20 @@ def test_prequantized_shared_input(overlap):
         layer.lib.tfh_layer_run_quantized.argtypes = None
         layer._check(layer.lib.tfh_layer_run_quantized(layer.h, ctypes.c_uint64(x.cuda().data_ptr()), ctypes.c_uint64(0), ctypes.c_uint64(0), layer._err, 512))
     layer.close()
+
+
+def test_verify_rows_permutation_equivariance_through_the_folded_entry():
+    # the 32 rows of the verify configuration in another order: every row's routes, routed sum and layer output are the same
+    # bits (the rows share expert tiles in another arrangement, the shared expert's row tiles hold other rows)
+    g, ops, x, rows = make("c3", "benchmark", "cuda")
+    layer = host.Layer(g, ops, rows)
+    layer.set_tokens()
+    layer.run(x)
+    first = layer.taps()
+    perm = torch.randperm(rows, generator=torch.Generator().manual_seed(7))
+    layer.run(x[perm.cuda()].contiguous())
+    second = layer.taps()
+    layer.close()
+    order = perm.numpy()
+    for name in ["ids", "weights", "xq", "xs", "route_out", "routed", "shared_down", "out"]:
+        assert np.array_equal(np.ascontiguousarray(second[name]).view(np.uint8), np.ascontiguousarray(first[name][order]).view(np.uint8)), name

@@ -66,6 +66,28 @@ def test_full_size_prefill(config):
     layer.close()
 
 
+def test_full_size_row_permutation_equivariance():
+    # a property that needs no oracle and covers every row of the largest configuration: a token row's result depends on that
+    # row alone (its logits, routes, codes, every expert product and the ordered sum), so permuting the 16,384 rows of the batch
+    # must permute ids, routing weights and the layer output bit for bit, although every expert tile then holds other rows in
+    # another order
+    c = CONFIGS["c5"]
+    g = geometry(c["hidden"], c["experts"], c["topk"], c["inter"], c["shared"], "benchmark")
+    ops = synth.LayerOperands(g, "c5", device="cuda")
+    ops.bias = synth.zipf_bias(g.experts, 1.1, 0.06, device="cuda")
+    rows = c["rows"]
+    x = synth.activations("c5", rows, g.hidden, device="cuda")
+    perm = torch.randperm(rows, generator=torch.Generator().manual_seed(41)).cuda()
+    layer = GpuLayer(g, ops, rows)
+    layer.run(x)
+    first = {k: getattr(layer, k).clone() for k in ("ids", "weights", "routed", "out", "shared_down")}
+    layer.run(x[perm].contiguous())
+    for k, v in first.items():
+        assert torch.equal(getattr(layer, k), v[perm]), k
+    assert int(layer.tile_base[-1]) > 0
+    layer.close()
+
+
 def subset(taps, sample, g, rows):
     return {k: taps[k][sample] for k in ["logits", "ids", "weights", "xq", "xs", "xq_min", "xs_min", "route_out", "routed", "shared_up",
                                          "shared_act", "shared_aq", "shared_as", "shared_down", "out"]}
