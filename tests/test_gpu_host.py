@@ -96,6 +96,10 @@ def test_paired_owners_pool_into_one_launch():
     out_a, out_b = layer.pair_run(xa_d, tokens_a, live_a, xb_d, tokens_b, live_b)
     assert np.array_equal(out_a[:live_a], alone[0][:live_a]), "owner A differs from its own run"
     assert np.array_equal(out_b[:live_b], alone[1][:live_b]), "owner B differs from its own run"
+    # the shared expert once over the pooled rows (the reference pools the owners' shared up-projection, src/paired_ffn.rs:91-102):
+    # the same bits again
+    pool_a, pool_b = layer.pair_run(xa_d, tokens_a, live_a, xb_d, tokens_b, live_b, pool_shared=True)
+    assert np.array_equal(pool_a[:live_a], alone[0][:live_a]) and np.array_equal(pool_b[:live_b], alone[1][:live_b]), "pooled shared expert"
     # and against the oracle, like any other schedule
     from helpers import error_stats, oracle_layer
     want = oracle_layer(g, ops, xb, tokens_b, live_b)["out"]

@@ -38,7 +38,7 @@ def load():
         lib.tfh_layer_profile_step.argtypes = [vp, ctypes.c_uint64, ctypes.POINTER(ctypes.c_float), cp, sz]
         lib.tfh_layer_profile_marks.argtypes = [vp, ctypes.POINTER(ctypes.c_uint64), ctypes.c_int, ctypes.c_int, ctypes.c_int, ctypes.POINTER(ctypes.c_float), cp, sz]
         lib.tfh_layer_pair_run.argtypes = [vp, ctypes.c_uint64, ctypes.POINTER(ctypes.c_int64), ctypes.c_int, ctypes.c_uint64, ctypes.POINTER(ctypes.c_int64),
-                                           ctypes.c_int, vp, vp, cp, sz]
+                                           ctypes.c_int, ctypes.c_int, vp, vp, cp, sz]
         lib.tfh_layer_tap.restype = ctypes.c_longlong
         lib.tfh_layer_tap.argtypes = [vp, cp, vp, sz, cp, sz]
         lib.tfh_layer_census.argtypes = [vp, vp, cp, sz]
@@ -167,13 +167,14 @@ class Layer:
         self._check(self.lib.tfh_layer_profile_marks(self.h, ptrs, len(xs), passes, int(exact), ms, self._err, 512))
         return list(ms)
 
-    def pair_run(self, xa, tokens_a, live_a, xb, tokens_b, live_b):
-        """Two owners of this layer through the pooled launch (Paired::run): returns both owners' outputs [rows][hidden] (BF16 bits)."""
+    def pair_run(self, xa, tokens_a, live_a, xb, tokens_b, live_b, pool_shared=False):
+        """Two owners of this layer through the pooled launch (Paired::run): returns both owners' outputs [rows][hidden] (BF16 bits).
+        `pool_shared`: the shared expert runs once over the pooled rows instead of once per owner."""
         ia = (ctypes.c_int64 * self.rows)(*[int(t) for t in tokens_a])
         ib = (ctypes.c_int64 * self.rows)(*[int(t) for t in tokens_b])
         oa = np.empty((self.rows, self.g.hidden), np.uint16)
         ob = np.empty((self.rows, self.g.hidden), np.uint16)
-        self._check(self.lib.tfh_layer_pair_run(self.h, xa.data_ptr(), ia, live_a, xb.data_ptr(), ib, live_b,
+        self._check(self.lib.tfh_layer_pair_run(self.h, xa.data_ptr(), ia, live_a, xb.data_ptr(), ib, live_b, int(pool_shared),
                                                 oa.ctypes.data_as(ctypes.c_void_p), ob.ctypes.data_as(ctypes.c_void_p), self._err, 512))
         return oa, ob
 

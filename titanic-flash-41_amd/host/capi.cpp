@@ -20,6 +20,7 @@ struct Handle {
     tf::LayerFfn::Options options;
     // a second owner of the same layer and the pool both owners run through (src/paired_ffn.rs)
     std::unique_ptr<tf::LayerFfn> layer_b;
+    std::unique_ptr<tf::LayerFfn> layer_pool;       // 2 x rows: the shared expert over both owners' pooled rows
     std::unique_ptr<tf::TokenRows> tokens_b;
     std::unique_ptr<tf::Paired> paired;
 };
@@ -268,9 +269,9 @@ int tfh_layer_profile_marks(void* handle, const uint64_t* inputs, int count, int
 }
 // Paired owners: a second LayerFfn over the same prepared layer and the pooled workspace.  Runs owner A (the handle's layer,
 // input `a_input`, token ids / live count as given) and owner B through Paired::run and copies both owners' layer outputs
-// ([rows][hidden] BF16 each) to the host.
+// ([rows][hidden] BF16 each) to the host.  `pool_shared` != 0: the shared expert runs once over the pooled rows.
 int tfh_layer_pair_run(void* handle, uint64_t a_input, const int64_t* a_ids, int a_live, uint64_t b_input, const int64_t* b_ids, int b_live,
-                       uint16_t* a_output, uint16_t* b_output, char* error, size_t error_len) {
+                       int pool_shared, uint16_t* a_output, uint16_t* b_output, char* error, size_t error_len) {
     Handle* h = (Handle*)handle;
     return guarded(error, error_len, [&] {
         if (!h->paired) {
@@ -281,7 +282,8 @@ int tfh_layer_pair_run(void* handle, uint64_t a_input, const int64_t* a_ids, int
         }
         h->tokens->update(a_ids, h->rows, (size_t)a_live);
         h->tokens_b->update(b_ids, h->rows, (size_t)b_live);
-        h->paired->run(*h->layer, a_input, *h->tokens, *h->layer_b, b_input, *h->tokens_b, *h->stream);
+        if (pool_shared && !h->layer_pool) h->layer_pool = std::make_unique<tf::LayerFfn>(h->native, h->weights, h->prepared, 2 * h->rows, h->options);
+        h->paired->run(*h->layer, a_input, *h->tokens, *h->layer_b, b_input, *h->tokens_b, *h->stream, pool_shared ? h->layer_pool.get() : nullptr);
         h->stream->synchronize();
         h->layer->output().download(a_output, h->layer->output().len());
         h->layer_b->output().download(b_output, h->layer_b->output().len());

@@ -593,13 +593,14 @@ void LayerFfn::sum_shared(const Workspace& workspace, size_t live_rows, const St
 // ---- Paired ------------------------------------------------------------------------------------------------------------------
 Paired::Paired(std::shared_ptr<const Native> native, size_t owner_rows)
     : native_(native), rows_(owner_rows), workspace_(native, 2 * owner_rows), shared_scratch_{Workspace(native, owner_rows), Workspace(native, owner_rows)},
+      shared_scratch_pool_(native, 2 * owner_rows),
       input_(2 * owner_rows * native->geometry().hidden), ids_(2 * owner_rows * native->geometry().topk),
       routing_(2 * owner_rows * native->geometry().topk) {
     ensure(owner_rows >= 1 && 2 * owner_rows <= 64, "paired owners pool into one few-row launch");
     input_.zero(); ids_.zero(); routing_.zero();                                                               // src/paired_ffn.rs:21-23
 }
 void Paired::run(LayerFfn& a, uint64_t a_input, const TokenRows& a_tokens, LayerFfn& b, uint64_t b_input, const TokenRows& b_tokens,
-                 const Stream& stream) {                                                                       // :65-120
+                 const Stream& stream, LayerFfn* pool) {                                                       // :65-120
     const ca_geometry& g = native_->geometry();
     const size_t a_live = a_tokens.active_rows(), b_live = b_tokens.active_rows(), H = g.hidden, K = g.topk;
     ensure(a.rows() == rows_ && b.rows() == rows_ && a_live >= 1 && a_live <= rows_ && b_live >= 1 && b_live <= rows_ && a_input && b_input &&
@@ -615,6 +616,14 @@ void Paired::run(LayerFfn& a, uint64_t a_input, const TokenRows& a_tokens, Layer
         check(hipMemcpyAsync((void*)(routing_.ptr() + o.offset * K * 4), (const void*)o.ffn->router().routing().ptr(), o.live * K * 4, hipMemcpyDeviceToDevice, stream.raw()), "pool weights");
     }
     workspace_.run_live(a.expert(), input_.ptr(), input_.len(), ids_, routing_, a_live + b_live, stream);      // :91
+    if (pool != nullptr) {                                                                                     // :91-102: the shared expert once, over the pooled rows
+        ensure(pool->rows() == 2 * rows_ && a.expert().same_layer_weights(pool->expert()), "pooled shared expert needs a layer of both owners' rows");
+        pool->run_shared(shared_scratch_pool_, input_.ptr(), stream);
+        for (const Owner& o : owners)
+            native_->ffn_add((int)o.live, workspace_.output().ptr() + o.offset * H * 2, pool->shared_down().ptr() + o.offset * H * 2, o.ffn->output().ptr(),
+                             stream.raw());
+        return;
+    }
     for (int i = 0; i < 2; ++i) {                                                                              // :108-115: every owner's shared expert on its own rows
         const Owner& o = owners[i];
         o.ffn->run_shared(shared_scratch_[i], o.input, stream);

@@ -292,8 +292,11 @@ private:
 class Paired {
 public:
     Paired(std::shared_ptr<const Native> native, size_t owner_rows);
+    // `pool` (may be null): a LayerFfn of the same layer for 2 x owner_rows rows.  With it the shared expert runs once over the
+    // pooled rows (its weights stream once for both owners; the reference pools the owners' shared up-projection,
+    // src/paired_ffn.rs:91-102, src/fp8_paired.rs:15-60) instead of once per owner; a row's result is the same bits either way.
     void run(LayerFfn& a, uint64_t a_input, const TokenRows& a_tokens, LayerFfn& b, uint64_t b_input, const TokenRows& b_tokens,
-             const Stream& stream);
+             const Stream& stream, LayerFfn* pool = nullptr);
     const Workspace& workspace() const { return workspace_; }
     const Buffer<int32_t>& ids() const { return ids_; }
 private:
@@ -301,6 +304,7 @@ private:
     size_t rows_;
     Workspace workspace_;
     Workspace shared_scratch_[2];      // the owners' shared-branch quantizer scratch
+    Workspace shared_scratch_pool_;    // the same for the pooled rows
     Buffer<uint16_t> input_;
     Buffer<int32_t> ids_;
     Buffer<float> routing_;
