@@ -55,29 +55,6 @@ __device__ __forceinline__ void tf_load_a(ATile<KSMAX>& t, const uint8_t* codes,
     }
 }
 
-// The same from global memory that other workgroups of this launch have published (device-scope loads).
-template <int KS, int KSMAX = KS>
-__device__ __forceinline__ void tf_load_a_acquire(ATile<KSMAX>& t, const uint8_t* codes, const uint8_t* scales, long long row, int k,
-                                                  int act_block, int ks_first, int lane) {
-    const int g = lane >> 4;
-#pragma unroll
-    for (int q = 0; q < (KS + 3) / 4; ++q) t.scale[q] = 0x7f7f7f7fu;
-#pragma unroll
-    for (int s = 0; s < KS; ++s) {
-        const int ks = ks_first + s;
-        if (row >= 0) {
-            const uint8_t* base = codes + row * k + ks * 128 + 16 * g;
-            const u4v lo = tf_acquire_u4v(reinterpret_cast<const u4v*>(base));
-            const u4v hi = tf_acquire_u4v(reinterpret_cast<const u4v*>(base + 64));
-            t.a[s] = v8i{(int)lo[0], (int)lo[1], (int)lo[2], (int)lo[3], (int)hi[0], (int)hi[1], (int)hi[2], (int)hi[3]};
-            const uint32_t byte = __hip_atomic_load(scales + row * (k / act_block) + (ks * 128 + 32 * g) / act_block, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
-            t.scale[s >> 2] = (t.scale[s >> 2] & ~(0xffu << (8 * (s & 3)))) | (byte << (8 * (s & 3)));
-        } else {
-            t.a[s] = v8i{0, 0, 0, 0, 0, 0, 0, 0};
-        }
-    }
-}
-
 // One pipeline unit of streamed weights for this wave: N 16-byte loads a lane (N KiB a wave).
 //   FP4 (routed): TILES weight tiles of 16 rows, KS k-steps each: d[t * KS + s].
 //   FP8 (shared): TILES / 2 weight tiles, each k-step as two 16-byte planes: d[(t * KS + s) * 2 + half].
@@ -522,8 +499,18 @@ __device__ __forceinline__ void tf_front_shared_item(const StreamArgs& p, const 
         const int rows = min(16, all_row_count - 16 * tile);                // of this tile
         ATile<KS> a;
         if (HANDOFF && ready) {
-            tf_load_a_acquire<KS>(a, p.a_codes + (size_t)tile * 16 * k, p.a_scales + (size_t)tile * 16 * (k / p.act_block),
-                                  (lane & 15) < rows ? (lane & 15) : -1, k, p.act_block, ks_first, lane);
+            // the tile's codes and scales, published by the quantizer blocks, through LDS: consecutive lanes take consecutive
+            // 8-byte pieces (device-scope loads come from beyond this XCD's L2; as A-fragment gathers, 8 bytes from 64 places
+            // an instruction, they took 20 us a block).  The previous tile's operand left LDS before that tile's barrier below.
+            const unsigned long long* codes = reinterpret_cast<const unsigned long long*>(p.a_codes + (size_t)tile * 16 * k);
+            const uint32_t* scale_words = reinterpret_cast<const uint32_t*>(p.a_scales + (size_t)tile * 16 * (k / p.act_block));
+            const int pieces = rows * (k >> 3), words = rows * (k / p.act_block) >> 2;         // k / act_block is a multiple of 4
+            for (int q = threadIdx.x; q < pieces; q += blockDim.x)
+                reinterpret_cast<unsigned long long*>(s_codes)[q] = __hip_atomic_load(codes + q, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+            for (int q = threadIdx.x; q < words; q += blockDim.x)
+                reinterpret_cast<uint32_t*>(s_scales)[q] = __hip_atomic_load(scale_words + q, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+            __syncthreads();
+            tf_load_a<KS>(a, s_codes, s_scales, (lane & 15) < rows ? (lane & 15) : -1, k, p.act_block, ks_first, lane);
         } else {
             // (the previous tile's operand left LDS before that tile's barrier below)
             const uint16_t* input = all_rows + (size_t)tile * 16 * k;
