@@ -206,7 +206,7 @@ def main():
     shared_fc1_bytes = 2 * S * H + (2 * S // BN) * (H // BK) + rows * (H + H // B) + rows * S * 2
     shared_fc2_bytes = H * S + (H // BN) * (S // BK) + rows * S * 2 + rows * H * 2
     # owners of at most eight rows: the shared expert's first projection streams inside the front-end launch, not in this one
-    early_shared = rows <= 64 and H <= 4096
+    early_shared = rows <= 64 and H <= 5120
     phase1_bytes = fc1_bytes + (0 if wide or early_shared else shared_fc1_bytes)
     phase2_bytes = fc2_bytes + (0 if wide else shared_fc2_bytes)
     fc1_ms = float(parts[2])

@@ -171,11 +171,11 @@ int launch_dynamic(const Context& c, bool route, const uint64_t* p, const int32_
             // per group of four rows: one expert a wave, eight waves a block (four for owners of at most eight rows)
             const int row_groups = (owner + 3) / 4;
             int logit_blocks = gate ? row_groups * (row_groups > 2 ? (g.experts + 7) / 8 : (g.experts + 3) / 4) : 0;
-            // hidden <= 4,096: the shared expert's first projection streams in this launch, beside the front-end's chain of
+            // hidden <= 5,120: the shared expert's first projection streams in this launch, beside the front-end's chain of
             // dependent steps, instead of lengthening the routed experts' first launch
             const int shared_blocks = g.shared_intermediate / 16;          // one item (16 columns, every row tile) a block
             const int dense_logit_blocks = row_groups * ((g.experts + 7) / 8);
-            const bool early_shared = sa.w != nullptr && gate && g.hidden <= 4096 && (phases & 3) == 3;
+            const bool early_shared = sa.w != nullptr && gate && g.hidden <= TF_FRONT_SHARED_MAX_K && (g.hidden <= 4096 || g.hidden % 1024 == 0) && (phases & 3) == 3;
             if (early_shared) {
                 logit_blocks = dense_logit_blocks;
                 ca_moe_route_frontend_shared<<<quant_blocks + 1 + logit_blocks + shared_blocks, 512, 0, s>>>(

@@ -453,7 +453,7 @@ __global__ void __launch_bounds__(256, 2) tf_phase2_stream(const StreamArgs rout
     if (hi > r_items) tf_fc2_items<true, KSS>(shared, (int)(lo > r_items ? lo - r_items : 0), (int)(hi - r_items), red, dyn, dyn + 16 * (size_t)kmax, plan);
 }
 
-// The experts' front-end with the shared expert's first projection in the same launch (few-row owners, hidden <= 4,096).
+// The experts' front-end with the shared expert's first projection in the same launch (few-row owners, hidden <= 5,120).
 // The front-end proper keeps a handful of workgroups busy for its whole length (gate product, routing, plan: a chain of
 // dependent steps) while the rest of the chip idles, or idles again once the logit blocks are done; the shared expert does
 // not depend on the routing, so its up / gate weights (two thirds of its bytes) stream here instead of inside the routed
@@ -469,9 +469,9 @@ __device__ __forceinline__ void tf_front_shared_item(const StreamArgs& p, const 
     const int k = p.k, per_row = k >> 3, group_lanes = p.act_block >> 3;
     const int per_tile = p.inter / 16, tiles = (all_row_count + 15) >> 4;
     uint8_t* s_codes = s_pool;                                        // [rows][k]             (at most 64 KiB)
-    uint8_t* s_scales = s_pool + 16 * 4096;                           // [rows][k / act_block] (at most 2 KiB)
+    uint8_t* s_scales = s_pool + 16 * TF_FRONT_SHARED_MAX_K;          // [rows][k / act_block]
     // [row tile parity][gate / up][wave][i][lane]: 2 x 8 KiB; consecutive row tiles alternate, so one barrier a tile is enough
-    float (*red)[2][4][4][64] = reinterpret_cast<float (*)[2][4][4][64]>(s_pool + 16 * 4096 + 2048);
+    float (*red)[2][4][4][64] = reinterpret_cast<float (*)[2][4][4][64]>(s_pool + 16 * TF_FRONT_SHARED_MAX_K + 16 * (TF_FRONT_SHARED_MAX_K / 32));
     const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6, half = wave >> 2, quarter = wave & 3, ks_first = quarter * KS;
     // `quant_blocks` > 0: the launch's quantizer blocks publish the rows' codes (shared flavour) and count themselves in; this
     // block waits for all of them (a bounded wait: they have lower block ids, none of them waits for anything) and reads its
@@ -599,6 +599,7 @@ extern "C" __global__ void __launch_bounds__(512) ca_moe_route_frontend_shared(
                 case 3072: tf_front_shared_item<6, true>(shared, input, rows, s_pool, block, sync, quant_blocks, shared_blocks); break;
                 case 3584: tf_front_shared_item<7, true>(shared, input, rows, s_pool, block, sync, quant_blocks, shared_blocks); break;
                 case 4096: tf_front_shared_item<8, true>(shared, input, rows, s_pool, block, sync, quant_blocks, shared_blocks); break;
+                case 5120: tf_front_shared_item<10, true>(shared, input, rows, s_pool, block, sync, quant_blocks, shared_blocks); break;
                 default: break;
             }
         } else {
@@ -611,6 +612,7 @@ extern "C" __global__ void __launch_bounds__(512) ca_moe_route_frontend_shared(
                 case 3072: tf_front_shared_item<6, false>(shared, input, rows, s_pool, block, sync, 0, shared_blocks); break;
                 case 3584: tf_front_shared_item<7, false>(shared, input, rows, s_pool, block, sync, 0, shared_blocks); break;
                 case 4096: tf_front_shared_item<8, false>(shared, input, rows, s_pool, block, sync, 0, shared_blocks); break;
+                case 5120: tf_front_shared_item<10, false>(shared, input, rows, s_pool, block, sync, 0, shared_blocks); break;
                 default: break;
             }
         }

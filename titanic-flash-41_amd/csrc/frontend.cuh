@@ -158,7 +158,9 @@ extern "C" __global__ void __launch_bounds__(512) ca_moe_frontend(
 // blocks of this small grid are resident together.
 #define TF_SYNC_QUANT_DONE 17             // arrival words (128 bytes apart) of the launch that also runs the shared expert's first projection:
 #define TF_SYNC_SHARED_PASSED 18          // quantizer blocks that are done; item blocks that have read the quantizer's output
-#define TF_FRONT_POOL_BYTES 83968          // 82 KiB: the shared expert's item blocks hold a 16-row tile's codes (64 KiB), scales (2) and partial sums (16)
+#define TF_FRONT_SHARED_MAX_K 5120         // widest token row whose shared up / gate projection runs inside the front-end launch
+// the shared expert's item blocks hold a 16-row tile's codes, its scales (32-wide blocks at most) and two sets of partial sums
+#define TF_FRONT_POOL_BYTES (16 * TF_FRONT_SHARED_MAX_K + 16 * (TF_FRONT_SHARED_MAX_K / 32) + 16384)
 // `grid_blocks`: the blocks of the launch that belong to the front-end (block ids [0, grid_blocks)); `s_pool`: TF_FRONT_POOL_BYTES
 // of LDS (logit blocks: the token rows; block 0 of owners of at most eight rows: logits, biases, token ids, live count).
 __device__ __forceinline__ void tf_route_frontend(

@@ -102,7 +102,7 @@ int main(int argc, char** argv) {
     // the rows' codes, intermediates and outputs
     const double K = g.topk;
     // owners of at most eight rows: the shared expert's up / gate weights stream in the front-end launch, not in the FC1 launch
-    const bool early_shared = rows <= 64 && H <= 4096;
+    const bool early_shared = rows <= 64 && H <= 5120;
     const double fc1_bytes = tiles * (2.0 * I * H / 2 + 2.0 * I * H / 32) + (early_shared ? 0.0 : 2.0 * S * H) + rows * (2.0 * H + K * I * 2 + 2.0 * S);
     const double fc2_bytes = tiles * (1.0 * H * I / 2 + 1.0 * H * I / 32) + 1.0 * H * S + rows * (K * I * 2 + K * H * 2 + 2.0 * S + 2.0 * H);
     std::printf("{\"tiles\": %.3f, \"fc1_algorithmic_bytes\": %.0f, \"fc2_algorithmic_bytes\": %.0f}\n", tiles, fc1_bytes, fc2_bytes);
