@@ -48,6 +48,7 @@ def run_case(rows, hidden, experts, topk, inter, shared, mode, live=None, paddin
     (5, 1536, 16, 2, 3072, 3584, "benchmark"),      # three, six and seven k-steps a wave
     (70, 6144, 16, 2, 512, 512, "reference"),       # many rows, K 6,144
     (3, 8192, 8, 2, 1024, 1024, "benchmark"),       # the widest token row
+    (130, 8192, 8, 2, 512, 512, "reference"),       # the same at many rows: 256 activation scale bytes a row, the table's capacity
 ])
 def test_shape(rows, hidden, experts, topk, inter, shared, mode):
     run_case(rows, hidden, experts, topk, inter, shared, mode)
