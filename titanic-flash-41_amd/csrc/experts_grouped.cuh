@@ -1,0 +1,456 @@
+// Many-row (prefill) routed-expert projections: grouped GEMM with both operands streamed into LDS by the memory system.
+//
+// One task = one unit of an expert's physical rows (BM = 128: one plan tile; BM = 256: two consecutive plan tiles of the
+// same expert) x one column group (FC1: 128 intermediate columns = 128 "up" + 128 "gate" weight rows; FC2: 256 output
+// columns).  A workgroup of eight waves (two a SIMD) keeps a BM x 256 accumulator: wave (wm, wn) holds token rows
+// [wm BM/4, +BM/4) against weight rows [128 wn, +128) of the group, i.e. BM/64 x 8 products of
+// v_mfma_scale_f32_16x16x128_f8f6f4 a k-step of 128.
+//
+// No operand of the main loop passes through vector registers on its way in: token codes (E4M3, gathered through the
+// permutation map), their UE8M0 scales, the prepared FP4 weights and their scales are written into LDS by
+// global_load_lds (16 or 4 bytes a lane, a wave's 64 lanes land at consecutive LDS addresses), LEAD k-steps ahead of
+// their use, in a ring of LEAD + 1 stages.  The loads are issued from inline assembly, so the compiler's own wait
+// insertion does not know them (it would wait for every load in flight before each LDS read); the kernel counts them
+// itself: loads complete in issue order, every wave issues the same number of them in every k-step, and the wait at the
+// top of a k-step allows exactly the loads issued after that k-step's own to stay in flight.  One barrier a k-step
+// then makes every wave's share of the stage visible to all and frees the stage that was read a k-step ago.
+//
+// Token tile in LDS: row-major, 128 bytes a row and k-step, the 16-byte pieces of a row permuted by a function of the
+// row so that the eight lanes that copy one row read one whole 128-byte line of global memory while the sixteen rows a
+// matrix-instruction fragment reads at once fall into different banks.  Weights in LDS: as prepared (1 KiB a 16-row
+// weight tile and k-step in fragment order).
+//
+// Workgroups are persistent; workgroup b runs on XCD b % 8 and takes a contiguous eighth of the units, all column
+// groups of a unit at about the same time on neighbouring CUs of that XCD: a unit's token rows and an expert's weights
+// reach an XCD's L2 once while its workgroups pass.  The next task's first operands are requested before the current
+// task's epilogue (SwiGLU + FP8 requantization, or routing weight + scatter), which needs no registers for them.
+//
+// Reference semantics (contract level): the two phase kernels of the reference's dynamic MoE node
+// (src/moe.rs:1098-1289; runtime/kernels/moe-runtime-*/manifest.json precision string).
+#pragma once
+#include "experts_gemm.cuh"
+
+// Lane l of the wave copies 16 (4) bytes from global address base + offset (a scalar base, the lane's own 32-bit byte
+// offset) to LDS byte address lds_base + 16 l (4 l).
+__device__ __forceinline__ void tf_dma16(const uint8_t* base, uint32_t offset, uint32_t lds_base) {
+    asm volatile("s_mov_b32 m0, %2\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %0, %1" ::"v"(offset), "s"(base), "s"(lds_base) : "memory");
+}
+__device__ __forceinline__ void tf_dma4(const uint8_t* base, uint32_t offset, uint32_t lds_base) {
+    asm volatile("s_mov_b32 m0, %2\n\ts_nop 0\n\tglobal_load_lds_dword %0, %1" ::"v"(offset), "s"(base), "s"(lds_base) : "memory");
+}
+template <int N>
+__device__ __forceinline__ void tf_wait_vm() { asm volatile("s_waitcnt vmcnt(%0)" ::"n"(N) : "memory"); }
+// Workgroup barrier that orders LDS accesses only (no wait for loads from global memory in flight).
+__device__ __forceinline__ void tf_lds_barrier() {
+    asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory");
+    __builtin_amdgcn_s_barrier();
+    asm volatile("" ::: "memory");
+}
+__device__ __forceinline__ uint32_t tf_lds_addr(const void* p) {
+    return (uint32_t)(size_t)(const __attribute__((address_space(3))) uint8_t*)p;
+}
+// acc += weights (FP4, first operand) x tokens (FP8, second operand) with the accumulator held in place (written as
+// assembly: the compiler's own form of this instruction writes a fresh destination for every product, and 128 accumulator
+// registers a lane then no longer fit beside the operands).  SW / ST: which byte of the weight / token scale registers
+// applies.  Lane (g, r) of the result holds weight rows 4 g .. 4 g + 3 of the 16-row weight tile for token row r of the
+// fragment.  Hazards the compiler does not see: results are read by vector instructions only after tf_mfma_settle().
+template <int SW, int ST>
+__device__ __forceinline__ void tf_mfma_weights_first(v4f& acc, const u4v& weights, const v8i& tokens, uint32_t scale_w, uint32_t scale_t) {
+    asm volatile("v_mfma_scale_f32_16x16x128_f8f6f4 %0, %1, %2, %0, %3, %4 op_sel:[%5,%6,0] op_sel_hi:[%7,%8,0] cbsz:4"
+                 : "+v"(acc) : "v"(weights), "v"(tokens), "v"(scale_w), "v"(scale_t), "n"(SW & 1), "n"(ST & 1), "n"(SW >> 1), "n"(ST >> 1));
+}
+// The matrix pipeline's last results have reached the registers (the longest product takes 8 passes of 4 cycles; 32 idle
+// cycles follow the last product before any of these eight accumulators is read).
+__device__ __forceinline__ void tf_mfma_settle(v4f (&acc)[8]) {
+    asm volatile("s_nop 15\n\ts_nop 15"
+                 : "+v"(acc[0]), "+v"(acc[1]), "+v"(acc[2]), "+v"(acc[3]), "+v"(acc[4]), "+v"(acc[5]), "+v"(acc[6]), "+v"(acc[7]));
+}
+// Requests that may still be in flight at the top of k-step `u` of an unrolled round of four: those issued in the LEAD - 1
+// k-steps before it.  Every k-step issues DATA requests, k-step 1 of a round two more (the next round's weight scales).
+// Requests the count does not know (the next tasks' permutation map, stores) only make the wait stricter: it lets the N
+// youngest stay in flight, and whatever is younger than the k-step's own requests may.
+template <int LEAD, int DATA>
+constexpr int tf_loads_behind(int u) {
+    int n = 0;
+    for (int j = 1; j < LEAD; ++j) n += DATA + (((u - j) & 3) == 1 ? 2 : 0);
+    return n;
+}
+
+template <int MODE, int BM, bool WORDS>
+__global__ void __launch_bounds__(512) tf_grouped_gemm(const GemmArgs p) {
+    constexpr bool FC1 = MODE == TF_GEMM_FC1_ROUTED;
+    constexpr int NS = BM == 256 ? 3 : 4, LEAD = NS - 1;
+    constexpr int NA = BM / 64;              // 16-byte pieces of the token tile a thread requests a k-step
+    constexpr int NF = BM / 64;              // 16-row fragments of a wave (BM / 4 rows)
+    constexpr int WROWS = BM / 4;
+    constexpr int DATA = NA + 1 + 2;         // requests a wave issues a k-step: token pieces, token scales, two weight tiles
+    constexpr int A_STAGE = BM * 128, B_STAGE = 16 * 1024;
+    constexpr int ROW_WAVES = BM / 64;       // waves whose 64 lanes cover the tile's rows once; the other waves repeat them
+    __shared__ __attribute__((aligned(1024))) uint8_t s_a[NS * A_STAGE];
+    __shared__ __attribute__((aligned(1024))) uint8_t s_b[NS * B_STAGE];
+    __shared__ __attribute__((aligned(256))) uint32_t s_asc[NS][BM];
+    __shared__ __attribute__((aligned(256))) uint32_t s_bsc[16 * 64];
+    __shared__ __attribute__((aligned(256))) int32_t s_src[3][BM];   // the permutation map's entry (route index) of each tile row, for three tasks in turn
+    __shared__ __attribute__((aligned(256))) float s_wgt[3][BM];     // FC2: routing weight of each tile row; FC1: row maxima of the two column halves
+    __shared__ uint16_t s_ubase[BM == 256 ? 514 : 2], s_tbase[BM == 256 ? 514 : 2];
+    __shared__ int32_t s_part[8];
+
+    const int tid = threadIdx.x, lane = tid & 63, wave = __builtin_amdgcn_readfirstlane(tid >> 6);
+    const int wm = wave >> 1, wn = wave & 1, g = lane >> 4, r16 = lane & 15;
+    const int KS = p.k / 128, scales_row = p.k / p.act_block;
+    const int groups = FC1 ? p.inter / 128 : p.hidden / 256;
+    const int total_tiles = p.expert_tile_base[p.experts];
+    int units = total_tiles;
+    if constexpr (BM == 256) {
+        // units of two plan tiles: per expert ceil(tiles / 2); exclusive prefix over the experts (one thread an expert)
+        const int e = tid;
+        int tb = 0, tn = 0;
+        if (e < p.experts) { tb = p.expert_tile_base[e]; tn = p.expert_tile_base[e + 1]; }
+        const int mine = (tn - tb + 1) >> 1;
+        int prefix = mine;
+#pragma unroll
+        for (int o = 1; o < 64; o <<= 1) {
+            const int below = __shfl_up(prefix, o);
+            if (lane >= o) prefix += below;
+        }
+        if (lane == 63) s_part[wave] = prefix;
+        __syncthreads();
+        for (int w = 0; w < wave; ++w) prefix += s_part[w];
+        if (e < p.experts) { s_ubase[e + 1] = (uint16_t)prefix; s_tbase[e] = (uint16_t)tb; }
+        if (e == p.experts - 1) s_tbase[e + 1] = (uint16_t)tn;
+        if (e == 0) s_ubase[0] = 0;
+        __syncthreads();
+        units = s_ubase[p.experts];
+    }
+    const int xcd = blockIdx.x & 7, local = blockIdx.x >> 3, local_count = gridDim.x >> 3;
+    const int u_lo = (int)((long long)units * xcd / 8), u_hi = (int)((long long)units * (xcd + 1) / 8);
+    const int my_tasks = (u_hi - u_lo) * groups;
+    if (local >= my_tasks) return;
+
+    // What a task needs from the plan is requested two tasks ahead, and not through vector registers either (a load the
+    // compiler knows of makes it wait for every load in flight, the ring's requests included, before the loaded register's
+    // next use): the tile rows' entries of the permutation map (and their routing weights) go to an LDS slot like every other
+    // operand; the task's scalars (tile, expert, valid rows) are scalar loads.
+    struct TaskRef { int ng, first_tile, rows, expert; };      // the same in every lane
+    auto scalar_load = [](const int32_t* at) {
+        int32_t v;
+        asm volatile("s_load_dword %0, %1, 0x0\n\ts_waitcnt lgkmcnt(0)" : "=s"(v) : "s"(at) : "memory");
+        return v;
+    };
+    const uint32_t lds_src = tf_lds_addr(&s_src[0][0]), lds_wgt = tf_lds_addr(&s_wgt[0][0]);
+    int walk = 0;                            // BM == 256: the expert of the last unit looked up (units are asked for in ascending order)
+    auto fetch = [&](int q, int slot) {
+        TaskRef r;
+        const int un = q / groups, unit = u_lo + un;
+        r.ng = q - un * groups;
+        if constexpr (BM == 256) {
+            while (__builtin_amdgcn_readfirstlane((int)s_ubase[walk + 1]) <= unit) ++walk;       // s_ubase[walk] <= unit < s_ubase[walk + 1]
+            const int k2 = unit - __builtin_amdgcn_readfirstlane((int)s_ubase[walk]);
+            const int tb = __builtin_amdgcn_readfirstlane((int)s_tbase[walk]), tn = __builtin_amdgcn_readfirstlane((int)s_tbase[walk + 1]);
+            r.expert = walk;
+            r.first_tile = tb + 2 * k2;
+            r.rows = min(BM, (tn - tb - 1) * 128 + scalar_load(p.task_valid_rows + (size_t)(tn - 1) * p.groups) - 256 * k2);
+        } else {
+            r.first_tile = unit;
+            r.expert = scalar_load(p.task_expert + (size_t)unit * p.groups);
+            r.rows = scalar_load(p.task_valid_rows + (size_t)unit * p.groups);
+        }
+        const uint32_t at = (uint32_t)min(r.first_tile * 128 + ((wave & (ROW_WAVES - 1)) * 64 + lane), total_tiles * 128 - 1) * 4u;
+        tf_dma4(reinterpret_cast<const uint8_t*>(p.token_map), at, lds_src + slot * (BM * 4) + (wave & (ROW_WAVES - 1)) * 256);
+        if constexpr (!FC1) tf_dma4(reinterpret_cast<const uint8_t*>(p.token_weights), at, lds_wgt + slot * (BM * 4) + (wave & (ROW_WAVES - 1)) * 256);
+        return r;
+    };
+
+    // ---- request state: where this thread's pieces of a k-step come from, for the current task and the one after -----------
+    // Every request is a scalar base (operand array + the k-step's offset, or the expert's weight tile) plus the lane's own
+    // 32-bit byte offset, which stays the same for a whole task.
+    struct Source {
+        uint32_t a_off[NA], asc_off;
+        const uint8_t* b_base[2];
+        const uint8_t* bsc_base[2];
+    };
+    const uint32_t lds_a = tf_lds_addr(s_a), lds_b = tf_lds_addr(s_b), lds_asc = tf_lds_addr(&s_asc[0][0]), lds_bsc = tf_lds_addr(s_bsc);
+    // The task's slot has landed and is visible (a wait for the requests and a barrier lie between its request and this).
+    auto install = [&](Source& src, const TaskRef& task, int slot) {
+        const int ng = task.ng, first_tile = task.first_tile, expert = task.expert, rows = task.rows;
+        auto source_row = [&](int row) -> uint32_t {         // rows past the valid ones request the first row's bytes again
+            if constexpr (FC1) return (uint32_t)(s_src[slot][row < rows ? row : 0] / p.topk);
+            else return (uint32_t)(first_tile * 128 + (row < rows ? row : 0));
+        };
+#pragma unroll
+        for (int c = 0; c < NA; ++c) {
+            const int row = (wave * NA + c) * 8 + (lane >> 3);
+            const int piece = (lane & 7) ^ ((row & 7) ^ ((row >> 3) & 1));
+            src.a_off[c] = source_row(row) * (uint32_t)p.k + piece * 16;
+        }
+        src.asc_off = source_row((wave & (ROW_WAVES - 1)) * 64 + lane) * (uint32_t)scales_row;
+        const uint8_t* w = p.w + (size_t)expert * p.w_expert_stride;
+        const uint8_t* ws = p.ws + (size_t)expert * p.ws_expert_stride;
+#pragma unroll
+        for (int c = 0; c < 2; ++c) {
+            const int T = wave * 2 + c;
+            const int ntile = FC1 ? (T < 8 ? ng * 8 + T : p.inter / 16 + ng * 8 + T - 8) : ng * 16 + T;
+            src.b_base[c] = w + (size_t)ntile * KS * 1024;
+            src.bsc_base[c] = ws + (size_t)ntile * (p.k / 512) * 256;
+        }
+    };
+    const uint32_t lane16 = lane * 16, lane4 = lane * 4;
+    // Request `op` of k-step `ks` of a task into ring stage `stage`: ops [0, NA): token pieces, NA: token scales, NA + 1, NA + 2:
+    // weight tiles; ops DATA, DATA + 1: the weight scales of round `ks / 4` (four k-steps a word).
+    auto issue_op = [&](const Source& src, int op, int ks, int stage) {
+        if (op < NA) tf_dma16(p.a_codes + (size_t)ks * 128, src.a_off[op], lds_a + stage * A_STAGE + (wave * NA + op) * 1024);
+        else if (op == NA) tf_dma4(p.a_scales + (WORDS ? (ks >> 2) * 4 : ks * 4), src.asc_off, lds_asc + stage * (BM * 4) + (wave & (ROW_WAVES - 1)) * 256);
+        else if (op < DATA) tf_dma16(src.b_base[op - NA - 1] + (size_t)ks * 1024, lane16, lds_b + stage * B_STAGE + (wave * 2 + op - NA - 1) * 1024);
+        else tf_dma4(src.bsc_base[op - DATA] + (size_t)(ks >> 2) * 256, lane4, lds_bsc + (wave * 2 + op - DATA) * 256);
+    };
+
+    // ---- this lane's fragment addresses ----------------------------------------------------------------------------------
+    const int swz = (r16 & 7) ^ (r16 >> 3);
+    const int a_lo = (wm * WROWS + r16) * 128 + ((g ^ swz) << 4), a_hi = a_lo ^ 64;     // + 2,048 a fragment
+    // weight tiles of the wave within a stage: FC1: four "up" tiles 4 wn + t, then the four "gate" tiles 8 + 4 wn + t of the same
+    // columns; FC2: tiles 8 wn + t.  One base a wave plus a constant a tile.
+    const int b_first = FC1 ? wn * 4 : wn * 8;
+    auto b_step = [](int t) constexpr { return FC1 ? (t < 4 ? t : 8 + t - 4) : t; };
+
+    // ---- the first task's first k-steps, and the second task's slot ------------------------------------------------------------
+    Source now, then;
+    TaskRef cur = fetch(local, 0);
+    tf_wait_vm<0>();
+    tf_lds_barrier();
+    install(now, cur, 0);
+#pragma unroll
+    for (int c = 0; c < 2; ++c) issue_op(now, DATA + c, 0, 0);
+#pragma unroll
+    for (int d = 0; d < LEAD; ++d)
+#pragma unroll
+        for (int op = 0; op < DATA; ++op) issue_op(now, op, d, d);
+    TaskRef nxt = fetch(min(local + local_count, my_tasks - 1), 1);
+    tf_wait_vm<0>();
+    int cs = 0, ps = LEAD;                  // stage read in the current k-step; stage the k-step LEAD ahead is written to
+    int slot = 0, slot_next = 1, slot_after = 2;
+    for (int q = local; q < my_tasks; q += local_count) {
+        const int rows = cur.rows, first_tile = cur.first_tile, ng = cur.ng;
+        const int nf = max(0, min(NF, (rows - wm * WROWS + 15) >> 4));     // fragments of this wave with valid rows
+        TaskRef after = nxt;
+
+        // One task, compiled for 0, NF / 2 or NF fragments of the wave so that no product sits under a branch and the
+        // accumulators are as many as the wave needs; every wave issues the same requests and passes the same barriers
+        // whatever its count.
+        auto run_task = [&](auto frags_constant) {
+            constexpr int FR = decltype(frags_constant)::value, FRA = FR > 0 ? FR : 1;
+            v4f acc[FRA][8];
+#pragma unroll
+            for (int f = 0; f < FRA; ++f)
+#pragma unroll
+                for (int t = 0; t < 8; ++t) acc[f][t] = v4f{0.f, 0.f, 0.f, 0.f};
+            uint32_t bsc[8];
+#pragma unroll
+            for (int t = 0; t < 8; ++t) bsc[t] = 0;
+            // One k-step.  FIRST / LAST: in the task's first / last round of four.  The requests of k-step ks + LEAD (the next
+            // task's first k-steps in the last round: the ring runs on across tasks) are issued between the fragments' products,
+            // so that their address arithmetic runs under the matrix pipeline.
+            auto k_step = [&](auto u_constant, auto first_constant, auto last_constant, int ks) {
+                constexpr int u = decltype(u_constant)::value;
+                constexpr bool FIRST = decltype(first_constant)::value, LAST = decltype(last_constant)::value;
+                // the task's first LEAD k-steps landed before the previous task's stores went out (below)
+                if constexpr (!FIRST || u >= LEAD) tf_wait_vm<tf_loads_behind<LEAD, DATA>(u)>();
+                __builtin_amdgcn_s_barrier();
+                asm volatile("" ::: "memory");
+                if constexpr (FIRST && u == 0) install(then, nxt, slot_next);
+                constexpr bool OVER = LAST && u + LEAD >= 4;           // the requests belong to the next task
+                const int ks_ahead = OVER ? u + LEAD - 4 : ks + LEAD;
+                const Source& from = OVER ? then : now;
+                constexpr int OPS = DATA + (u == 1 ? 2 : 0);           // k-step 1 of a round: the next round's weight scales first
+                auto issue_range = [&](int lo, int hi) {
+#pragma unroll
+                    for (int i = lo; i < hi; ++i) {
+                        if (u == 1 && i < 2) issue_op(LAST ? then : now, DATA + i, LAST ? 0 : ks + 3, 0);
+                        else issue_op(from, i - (u == 1 ? 2 : 0), ks_ahead, ps);
+                    }
+                };
+                if constexpr (FR == 0) issue_range(0, OPS);
+                if constexpr (FR > 0) {
+                    const uint8_t* sa = s_a + cs * A_STAGE;
+                    const uint8_t* sb = s_b + cs * B_STAGE + b_first * 1024 + lane16;
+                    const uint32_t* sc = &s_asc[cs][wm * WROWS + r16];
+                    u4v bf[8];
+#pragma unroll
+                    for (int t = 0; t < 8; ++t) bf[t] = *reinterpret_cast<const u4v*>(sb + b_step(t) * 1024);
+                    if constexpr (u == 0) {
+#pragma unroll
+                        for (int t = 0; t < 8; ++t) bsc[t] = s_bsc[b_first * 64 + lane + b_step(t) * 64];
+                    }
+                    // fragment f + 1 leaves LDS while fragment f is multiplied: two register sets
+                    u4v lo[2], hi[2];
+                    uint32_t word[2];
+                    lo[0] = *reinterpret_cast<const u4v*>(sa + a_lo);
+                    hi[0] = *reinterpret_cast<const u4v*>(sa + a_hi);
+                    word[0] = sc[0];
+#pragma unroll
+                    for (int f = 0; f < FR; ++f) {
+                        if (f + 1 < FR) {
+                            lo[(f + 1) & 1] = *reinterpret_cast<const u4v*>(sa + a_lo + (f + 1) * 2048);
+                            hi[(f + 1) & 1] = *reinterpret_cast<const u4v*>(sa + a_hi + (f + 1) * 2048);
+                            word[(f + 1) & 1] = sc[(f + 1) * 16];
+                        }
+                        const u4v l = lo[f & 1], h = hi[f & 1];
+                        const uint32_t sca = WORDS ? word[f & 1] : word[f & 1] >> (8 * g);
+                        constexpr int SEL = WORDS ? u : 0;
+                        const v8i av = v8i{(int)l[0], (int)l[1], (int)l[2], (int)l[3], (int)h[0], (int)h[1], (int)h[2], (int)h[3]};
+#pragma unroll
+                        for (int t = 0; t < 8; ++t) tf_mfma_weights_first<u, SEL>(acc[f][t], bf[t], av, bsc[t], sca);
+                        issue_range(OPS * f / FR, OPS * (f + 1) / FR);
+                        __builtin_amdgcn_sched_barrier(0);       // keeps fragment f + 2's reads behind these products: two register sets
+                    }
+                }
+                cs = cs + 1 == NS ? 0 : cs + 1;
+                ps = ps + 1 == NS ? 0 : ps + 1;
+                // the plan's entries for the task after the next: a chain of dependent scalar steps, taken by the two waves of a
+                // SIMD in different k-steps so that one of them always has products to issue
+                if constexpr (FIRST && (u == 1 || u == 2)) {
+                    if ((wave < 4) == (u == 1)) after = fetch(min(q + 2 * local_count, my_tasks - 1), slot_after);
+                }
+            };
+            auto round = [&](auto first_constant, auto last_constant, int ks0) {
+                k_step(std::integral_constant<int, 0>{}, first_constant, last_constant, ks0);
+                k_step(std::integral_constant<int, 1>{}, first_constant, last_constant, ks0 + 1);
+                k_step(std::integral_constant<int, 2>{}, first_constant, last_constant, ks0 + 2);
+                k_step(std::integral_constant<int, 3>{}, first_constant, last_constant, ks0 + 3);
+            };
+            if (KS == 4) round(std::true_type{}, std::true_type{}, 0);
+            else {
+                round(std::true_type{}, std::false_type{}, 0);
+                for (int ks0 = 4; ks0 < KS - 4; ks0 += 4) round(std::false_type{}, std::false_type{}, ks0);
+                round(std::false_type{}, std::true_type{}, KS - 4);
+            }
+#pragma unroll
+            for (int f = 0; f < FR; ++f) tf_mfma_settle(acc[f]);
+
+            // ---- epilogue: values first, then a wait for every request in flight (the next task's first k-steps, long landed
+            // by now: its first LEAD k-steps then wait for nothing, in particular not for the stores below), then the stores ---
+            // Lane (g, r16) of product (f, t) holds tile row wm WROWS + 16 f + r16 and the four consecutive columns 4 g + i of
+            // weight tile t.
+            if constexpr (FC1) {
+                // t < 4: "up" tiles, t >= 4: the "gate" tiles of the same columns 64 wn + 16 (t % 4) + 4 g + i of the group
+                float hv[FRA][4][4];
+                float amax[FRA][2];
+                uint32_t codes[FRA][4], exponent[FRA][2];
+                float (*s_max)[BM] = s_wgt;          // [wn][row]: FC1 keeps no routing weights here
+#pragma unroll
+                for (int f = 0; f < FR; ++f) {
+#pragma unroll
+                    for (int j = 0; j < 4; ++j)
+#pragma unroll
+                        for (int i = 0; i < 4; ++i) {
+                            const float gv = fminf(acc[f][4 + j][i], p.limit), uv = fminf(p.limit, fmaxf(-p.limit, acc[f][j][i]));
+                            hv[f][j][i] = tf_bf16(tf_to_bf16(__fmul_rn(__fmul_rn(gv, tf_logistic_fast(gv)), uv)));
+                        }
+#pragma unroll
+                    for (int b = 0; b < 2; ++b) {
+                        float m = 0.f;
+#pragma unroll
+                        for (int j = 2 * b; j < 2 * b + 2; ++j)
+#pragma unroll
+                            for (int i = 0; i < 4; ++i) m = fmaxf(m, fabsf(hv[f][j][i]));
+                        m = fmaxf(m, __shfl_xor(m, 16));
+                        amax[f][b] = fmaxf(m, __shfl_xor(m, 32));       // over the 32 columns of weight tiles 2 b, 2 b + 1
+                    }
+                }
+                if constexpr (WORDS) {               // one scale a row and 128 columns: both column halves (waves wn = 0, 1)
+#pragma unroll
+                    for (int f = 0; f < FR; ++f) if (g == 0) s_max[wn][wm * WROWS + 16 * f + r16] = fmaxf(amax[f][0], amax[f][1]);
+                    tf_lds_barrier();
+#pragma unroll
+                    for (int f = 0; f < FR; ++f) {
+                        const int row = wm * WROWS + 16 * f + r16;
+                        amax[f][0] = amax[f][1] = fmaxf(s_max[0][row], s_max[1][row]);
+                    }
+                }
+#pragma unroll
+                for (int f = 0; f < FR; ++f)
+#pragma unroll
+                    for (int b = 0; b < 2; ++b) {
+                        exponent[f][b] = tf_block_exponent(amax[f][b]);
+                        const float inv = tf_block_inverse(exponent[f][b]);
+#pragma unroll
+                        for (int j = 2 * b; j < 2 * b + 2; ++j)
+                            codes[f][j] = tf_pack_e4m3(__fmul_rn(hv[f][j][0], inv), __fmul_rn(hv[f][j][1], inv), __fmul_rn(hv[f][j][2], inv), __fmul_rn(hv[f][j][3], inv));
+                    }
+                tf_wait_vm<0>();
+#pragma unroll
+                for (int f = 0; f < FR; ++f) {
+                    const int row = wm * WROWS + 16 * f + r16;
+                    if (row < rows) {
+                        const size_t phys = (size_t)first_tile * 128 + row;
+#pragma unroll
+                        for (int j = 0; j < 4; ++j) {
+                            const int col = ng * 128 + wn * 64 + j * 16 + 4 * g;
+                            *reinterpret_cast<uint32_t*>(p.h_codes + phys * p.inter + col) = codes[f][j];
+                            if (p.h_bf16 != nullptr)
+                                *reinterpret_cast<u2v*>(p.h_bf16 + phys * p.inter + col) = u2v{tf_pack_bf16(hv[f][j][0], hv[f][j][1]), tf_pack_bf16(hv[f][j][2], hv[f][j][3])};
+                        }
+                        if (g == 0) {
+                            if constexpr (WORDS) { if (wn == 0) p.h_scales[phys * (p.inter / 128) + ng] = (uint8_t)exponent[f][0]; }
+                            else {
+                                p.h_scales[phys * (p.inter / 32) + ng * 4 + wn * 2] = (uint8_t)exponent[f][0];
+                                p.h_scales[phys * (p.inter / 32) + ng * 4 + wn * 2 + 1] = (uint8_t)exponent[f][1];
+                            }
+                        }
+                    }
+                }
+            } else {
+                // output columns 256 ng + 128 wn + 16 t + 4 g + i of the row's route, scaled by its routing weight
+                u2v packed[FRA][8];
+                size_t out_at[FRA];
+#pragma unroll
+                for (int f = 0; f < FR; ++f) {
+                    const int row = min(wm * WROWS + 16 * f + r16, BM - 1);
+                    const float share = s_wgt[slot][row];
+                    out_at[f] = (size_t)s_src[slot][row] * p.hidden + ng * 256 + wn * 128 + 4 * g;
+#pragma unroll
+                    for (int t = 0; t < 8; ++t)
+                        packed[f][t] = u2v{tf_pack_bf16(__fmul_rn(acc[f][t][0], share), __fmul_rn(acc[f][t][1], share)),
+                                           tf_pack_bf16(__fmul_rn(acc[f][t][2], share), __fmul_rn(acc[f][t][3], share))};
+                }
+                tf_wait_vm<0>();
+#pragma unroll
+                for (int f = 0; f < FR; ++f)
+                    if (wm * WROWS + 16 * f + r16 < rows) {
+#pragma unroll
+                        for (int t = 0; t < 8; ++t) *reinterpret_cast<u2v*>(p.out + out_at[f] + 16 * t) = packed[f][t];
+                    }
+            }
+            if constexpr (FR == 0) tf_wait_vm<0>();
+        };
+        if (nf > NF / 2) run_task(std::integral_constant<int, NF>{});
+        else if (nf > 0) run_task(std::integral_constant<int, NF / 2>{});
+        else run_task(std::integral_constant<int, 0>{});
+        cur = nxt;
+        nxt = after;
+        now = then;
+        const int done = slot;
+        slot = slot_next; slot_next = slot_after; slot_after = done;
+    }
+}
+
+// Shapes the streamed grouped GEMM takes: contraction lengths that are multiples of 512, at most 512 experts (one thread an
+// expert in the unit prefix), whole column groups.
+inline bool tf_grouped_shape_ok(const GemmArgs& a, bool fc1) {
+    return a.k >= 512 && a.k % 512 == 0 && (a.act_block == 32 || a.act_block == 128) && a.experts <= 512 &&
+           (fc1 ? (a.inter >= 128 && a.inter % 128 == 0) : (a.hidden >= 256 && a.hidden % 256 == 0));
+}
+// `routes`: rows x top-k of the launch; experts with about two plan tiles or more on average run 256-row units.
+template <int MODE>
+inline int tf_launch_grouped(const GemmArgs& a, long long routes, int cus, hipStream_t s) {
+    if (!tf_grouped_shape_ok(a, MODE == TF_GEMM_FC1_ROUTED)) return -4;
+    const int grid = tf_gemm_grid(cus);
+    const bool big = routes >= 192ll * a.experts, words = a.act_block == 128;
+    if (big) {
+        if (words) tf_grouped_gemm<MODE, 256, true><<<grid, 512, 0, s>>>(a);
+        else tf_grouped_gemm<MODE, 256, false><<<grid, 512, 0, s>>>(a);
+    } else {
+        if (words) tf_grouped_gemm<MODE, 128, true><<<grid, 512, 0, s>>>(a);
+        else tf_grouped_gemm<MODE, 128, false><<<grid, 512, 0, s>>>(a);
+    }
+    return (int)hipGetLastError();
+}
