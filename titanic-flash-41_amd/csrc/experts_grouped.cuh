@@ -210,6 +210,7 @@ __global__ void __launch_bounds__(512) tf_grouped_gemm(const GemmArgs p) {
     // weight tiles of the wave within a stage: FC1: four "up" tiles 4 wn + t, then the four "gate" tiles 8 + 4 wn + t of the same
     // columns; FC2: tiles 8 wn + t.  One base a wave plus a constant a tile.
     const int b_first = FC1 ? wn * 4 : wn * 8;
+    const int issue_slot = (wave + (wave >> 2) * 2) & 3;          // waves w and w + 4 share a SIMD: slots s and s + 2
     auto b_step = [](int t) constexpr { return FC1 ? (t < 4 ? t : 8 + t - 4) : t; };
 
     // ---- the first task's first k-steps, and the second task's slot ------------------------------------------------------------
@@ -299,7 +300,10 @@ __global__ void __launch_bounds__(512) tf_grouped_gemm(const GemmArgs p) {
                         const v8i av = v8i{(int)l[0], (int)l[1], (int)l[2], (int)l[3], (int)h[0], (int)h[1], (int)h[2], (int)h[3]};
 #pragma unroll
                         for (int t = 0; t < 8; ++t) tf_mfma_weights_first<u, SEL>(acc[f][t], bf[t], av, bsc[t], sca);
-                        issue_range(OPS * f / FR, OPS * (f + 1) / FR);
+                        // this wave's requests of the k-step, all behind one fragment's products and a different fragment for the
+                        // two waves of a SIMD and for neighbouring SIMDs: a request holds its wave until the address unit takes it,
+                        // and eight waves requesting at once hold each other while no product is issued
+                        if (f == issue_slot % FR) issue_range(0, OPS);
                         __builtin_amdgcn_sched_barrier(0);       // keeps fragment f + 2's reads behind these products: two register sets
                     }
                 }
