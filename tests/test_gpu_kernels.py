@@ -203,8 +203,11 @@ def test_prepared_layouts_codes_and_permutation_round_trip():
     assert np.array_equal(np_of(d).view(np.uint32), w32)
     assert native.load().ca_moe_nibble_permute(native.ptr(d), 6, 0, None) == -1
     # one-bit scale code on the prepared scale bytes + GPU self check + census
+    # matrix 0, 1: the commonest byte is the base; matrix 2: the byte below the commonest is more common than the byte above and
+    # becomes the base (kernels/expert_scale_codes.cuh:49-51)
     matrices, columns = 3, k // 32
-    prepared = np.stack([oracle.stream_scales(rng.choice(np.array([119, 119, 119, 120, 120, 117], np.uint8), (n, columns)), n, k) for _ in range(matrices)])
+    mixes = [[119, 119, 119, 120, 120, 117], [119, 119, 119, 120, 120, 117], [120, 120, 120, 119, 119, 117]]
+    prepared = np.stack([oracle.stream_scales(rng.choice(np.array(mixes[m], np.uint8), (n, columns)), n, k) for m in range(matrices)])
     units = (n // 128) * (columns // 4)
     code = torch.zeros(matrices * units * 16, dtype=torch.int32, device="cuda")
     flags = torch.zeros(matrices * units * 4, dtype=torch.int32, device="cuda")
@@ -219,6 +222,7 @@ def test_prepared_layouts_codes_and_permutation_round_trip():
     wc, wf, wb = oracle.scale_code1(prepared, matrices, n, columns)
     assert np.array_equal(np_of(code).view(np.uint32), wc) and np.array_equal(np_of(flags).view(np.uint32), wf)
     assert np.array_equal(np_of(bases).view(np.uint32), wb) and int(error.item()) == 0
+    assert [int(v) & 255 for v in wb] == [119, 119, 119]
     err, raw_rows = oracle.scale_code1_check(prepared, wc, wf, wb, matrices, n, columns)
     assert err == 0 and raw_rows == int(counts.item()) and raw_rows > 0
     # four-bit row deltas

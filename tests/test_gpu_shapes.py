@@ -49,6 +49,11 @@ def run_case(rows, hidden, experts, topk, inter, shared, mode, live=None, paddin
     (70, 6144, 16, 2, 512, 512, "reference"),       # many rows, K 6,144
     (3, 8192, 8, 2, 1024, 1024, "benchmark"),       # the widest token row
     (130, 8192, 8, 2, 512, 512, "reference"),       # the same at many rows: 256 activation scale bytes a row, the table's capacity
+    (4, 512, 512, 2, 512, 512, "reference"),        # as many experts as the plan block has threads: the tile total is written by the last expert's thread
+    (600, 512, 512, 2, 512, 512, "benchmark"),      # the same through the many-route plan kernels
+    (1100, 1024, 8, 2, 512, 512, "benchmark"),      # two plan tiles an expert and more: the grouped GEMM's 256-row units; FC2 with one round of k-steps
+    (1100, 1024, 8, 2, 512, 512, "reference"),      # the same with 32-wide activation blocks
+    (700, 2048, 4, 1, 1024, 512, "benchmark"),      # 256-row units whose last unit of an expert is a single, partly filled plan tile
 ])
 def test_shape(rows, hidden, experts, topk, inter, shared, mode):
     run_case(rows, hidden, experts, topk, inter, shared, mode)

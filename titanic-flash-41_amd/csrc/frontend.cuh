@@ -97,8 +97,9 @@ __device__ __forceinline__ void tf_plan_block(const int32_t* ids, const float* w
     __syncthreads();
     int base = prefix - tiles;
     for (int w = 0; w < wave; ++w) base += s_wave[w];
-    if (t <= experts) expert_tile_base[t] = base;
+    if (t == experts - 1) expert_tile_base[experts] = base + tiles;      // the total: written by the last expert's thread (experts may equal blockDim.x)
     if (t < experts) {
+        expert_tile_base[t] = base;
         s_base[t] = base;
         for (int k = 0; k < tiles; ++k) {
             const int valid = min(tile_m, count - k * tile_m);
@@ -392,7 +393,8 @@ extern "C" __global__ void __launch_bounds__(512) ca_plan_tiles(int32_t experts,
     __syncthreads();
     int base = prefix - tiles;
     for (int w = 0; w < wave; ++w) base += s_wave[w];
-    if (t <= experts) expert_tile_base[t] = base;
+    if (t == experts - 1) expert_tile_base[experts] = base + tiles;      // the total: written by the last expert's thread (experts may equal blockDim.x)
+    if (t < experts) expert_tile_base[t] = base;
     if (t < experts)
         for (int k = 0; k < tiles; ++k) {
             const int valid = min(tile_m, count - k * tile_m);

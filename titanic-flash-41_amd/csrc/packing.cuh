@@ -41,105 +41,151 @@ extern "C" __global__ void ca_dense_compact_fp8(const u4v* source, u4v* out, int
     const size_t at = (((size_t)(r / 16) * (k / 128) + ks) * 2 + half) * 64 + g * 16 + r % 16;
     if (inverse) out[i] = source[at]; else out[at] = source[i];
 }
-// Reversible nibble interleave inside each 32-bit word: [e0..e7] -> [e0,e4,e1,e5,e2,e6,e3,e7].
+// Reversible nibble interleave inside each 32-bit word: [e0..e7] -> [e0,e4,e1,e5,e2,e6,e3,e7] (the format of
+// kernels/moe_nibble_layout_probe.cu:9-12).  Forward: the low half's four nibbles spread to the even nibble positions, the
+// high half's to the odd ones (two shift-and-mask steps a half); inverse: the even and the odd nibbles squeezed back.
+__device__ __forceinline__ uint32_t tf_spread_nibbles(uint32_t h) {          // 0x0000dcba -> 0x0d0c0b0a
+    h = (h | (h << 8)) & 0x00ff00ffu;
+    return (h | (h << 4)) & 0x0f0f0f0fu;
+}
+__device__ __forceinline__ uint32_t tf_squeeze_nibbles(uint32_t v) {         // 0x0d0c0b0a -> 0x0000dcba
+    v = (v | (v >> 4)) & 0x00ff00ffu;
+    return (v | (v >> 8)) & 0x0000ffffu;
+}
 extern "C" __global__ void ca_moe_nibble_permute_words(uint32_t* words, unsigned long long count, int inverse) {
     for (unsigned long long i = (unsigned long long)blockIdx.x * blockDim.x + threadIdx.x; i < count;
          i += (unsigned long long)gridDim.x * blockDim.x) {
         const uint32_t x = words[i];
-        uint32_t y = 0;
-#pragma unroll
-        for (int j = 0; j < 8; ++j) {
-            const int source = (j & 1) * 4 + (j >> 1);
-            if (inverse) y |= ((x >> (j * 4)) & 15u) << (source * 4);
-            else y |= ((x >> (source * 4)) & 15u) << (j * 4);
-        }
-        words[i] = y;
+        words[i] = inverse ? tf_squeeze_nibbles(x & 0x0f0f0f0fu) | (tf_squeeze_nibbles((x >> 4) & 0x0f0f0f0fu) << 16)
+                           : tf_spread_nibbles(x & 0xffffu) | (tf_spread_nibbles(x >> 16) << 4);
     }
 }
 
-// One-bit scale code.  Input: prepared scale bytes of one matrix per block, as units of 128 row words of `width` bytes
-// ([128-row tile][4-column slice][row][width]).  Output per matrix: base word b * 0x01010101 (b = the commonest byte, or
-// the one below it when that is more common than the one above); per unit 16 code words (bit 4 (r % 8) + j of word
-// r / 8 = byte j of row r minus b) and 4 flag words (bit r % 32 of word r / 32: row r holds a byte outside {b, b + 1}).
-__device__ __forceinline__ int sc1_tiles(int n) { return (n + 127) / 128; }
-__device__ __forceinline__ int sc1_slices(int columns) { return (columns + 3) / 4; }
-extern "C" __global__ void ca_expert_scale_code1(const uint8_t* scales, uint32_t* code, uint32_t* flags, uint32_t* bases,
-                                                 int n, int columns) {
-    __shared__ unsigned hist[256];
-    __shared__ int chosen;
-    const int matrix = blockIdx.x, tiles = sc1_tiles(n), slices = sc1_slices(columns);
-    const uint8_t* s = scales + (size_t)matrix * n * columns;
-    for (int i = threadIdx.x; i < 256; i += blockDim.x) hist[i] = 0;
-    __syncthreads();
-    for (int i = threadIdx.x; i < n * columns; i += blockDim.x) atomicAdd(&hist[s[i]], 1u);
-    __syncthreads();
-    if (threadIdx.x == 0) {
-        int c = 0;
-        for (int v = 1; v < 256; v++) if (hist[v] > hist[c]) c = v;
-        const int b = (c > 0 && (c == 255 || hist[c - 1] > hist[c + 1])) ? c - 1 : c;
-        chosen = b;
-        bases[matrix] = (uint32_t)b * 0x01010101u;
+// One-bit scale code (format: kernels/expert_scale_codes.cuh:29-36, word offsets src/config.rs:1365-1375).  Input: the
+// scale bytes of one matrix per workgroup, as units of 128 row words of `width` bytes ([128-row tile][4-column slice][row]
+// [width]).  Output per matrix: the base word b * 0x01010101 (b = the commonest byte, or the byte below it when that one is
+// more common than the byte above); per unit 16 code words (bit 4 (r % 8) + j of word r / 8: byte j of row r is b + 1) and
+// 4 flag words (bit r % 32 of word r / 32: row r holds a byte outside {b, b + 1} and stays raw).
+// One workgroup of four waves a matrix.  The byte counts are taken a wave of bytes at a time by matching: the lanes that
+// hold the same byte as the first lane still open are counted with one ballot and closed together (scale bytes take a
+// handful of values, so a wave's 64 bytes close in two or three rounds); the 256 counts are then ranked by all 256 threads
+// at once (largest count, lowest byte on a tie, as one packed key).  A wave then codes a unit at a time, 64 rows a pass: a
+// row's four bits meet the seven other rows of its code word through three lane exchanges, and a pass's raw rows are one
+// ballot, which is the flag word pair.
+__device__ __forceinline__ uint32_t tf_unit_row_word(const uint8_t* unit, int row, int width) {
+    uint32_t w = 0;
+    for (int j = 0; j < width; ++j) w |= (uint32_t)unit[row * width + j] << (8 * j);
+    return w;
+}
+// bit j: byte j of `word` equals `above` (= b + 1); `raw`: some byte of the row's `width` is neither b nor b + 1
+__device__ __forceinline__ uint32_t tf_row_bits(uint32_t word, int width, uint32_t b, bool& raw) {
+    uint32_t bits = 0;
+    raw = false;
+    for (int j = 0; j < width; ++j) {
+        const uint32_t v = (word >> (8 * j)) & 255u;
+        bits |= (uint32_t)(v == b + 1) << j;
+        raw = raw || (v != b && v != b + 1);
     }
-    __syncthreads();
-    const unsigned b = (unsigned)chosen;
-    const size_t units = (size_t)tiles * slices;
-    uint32_t* c = code + (size_t)matrix * units * 16;
-    uint32_t* f = flags + (size_t)matrix * units * 4;
-    for (size_t g = threadIdx.x; g < units * 4; g += blockDim.x) {
-        const int unit = (int)(g / 4), group = (int)(g % 4), tile = unit / slices, slice = unit % slices;
-        const int nr = min(128, n - tile * 128), width = min(4, columns - slice * 4);
-        const uint8_t* u = s + (size_t)tile * 128 * columns + (size_t)slice * nr * 4;
-        uint32_t words[4] = {0, 0, 0, 0}, flag = 0;
-        for (int i = 0; i < 32; i++) {
-            const int r = group * 32 + i;
-            if (r >= nr) continue;
-            unsigned nibble = 0;
-            bool raw = false;
-            for (int j = 0; j < width; j++) {
-                const unsigned v = u[r * width + j];
-                if (v == b) continue;
-                if (v == b + 1) { nibble |= 1u << j; continue; }
-                raw = true;
-            }
-            if (raw) { flag |= 1u << i; continue; }
-            words[i / 8] |= nibble << (4 * (i % 8));
+    return bits;
+}
+extern "C" __global__ void __launch_bounds__(256) ca_expert_scale_code1(const uint8_t* scales, uint32_t* code, uint32_t* flags, uint32_t* bases,
+                                                                        int n, int columns) {
+    __shared__ uint32_t s_count[4][256];          // a table a wave
+    __shared__ uint32_t s_best[4];
+    __shared__ uint32_t s_total[256];
+    const int t = threadIdx.x, lane = t & 63, wave = t >> 6, waves = blockDim.x >> 6;
+    const int matrix = blockIdx.x, tiles = (n + 127) / 128, slices = (columns + 3) / 4;
+    const uint8_t* bytes = scales + (size_t)matrix * n * columns;
+    const int total = n * columns;
+    for (int i = lane; i < 256; i += 64) s_count[wave][i] = 0;
+    __builtin_amdgcn_wave_barrier();
+    for (int first = wave * 64; first < total; first += waves * 64) {
+        const int at = first + lane;
+        const int value = at < total ? bytes[at] : -1;
+        unsigned long long open = __ballot(value >= 0);
+        while (open) {
+            const int leader = __ffsll((long long)open) - 1;
+            const int which = __shfl(value, leader);
+            const unsigned long long same = __ballot(value == which);
+            if (lane == leader) s_count[wave][which] += (uint32_t)__popcll(same);
+            open &= ~same;
         }
-        for (int w = 0; w < 4; w++) c[(size_t)unit * 16 + group * 4 + w] = words[w];
-        f[(size_t)unit * 4 + group] = flag;
+    }
+    __syncthreads();
+    // thread v ranks byte v: key = count << 8 | (255 - v), so the largest key is the largest count and, on a tie, the lowest byte
+    uint32_t mine = 0;
+    if (t < 256) {
+        for (int w = 0; w < waves; ++w) mine += s_count[w][t];
+        s_total[t] = mine;
+    }
+    uint32_t key = t < 256 ? (mine << 8) | (uint32_t)(255 - t) : 0u;
+#pragma unroll
+    for (int o = 32; o > 0; o >>= 1) key = max(key, (uint32_t)__shfl_xor((int)key, o));
+    if (lane == 0) s_best[wave] = key;
+    __syncthreads();
+    for (int w = 0; w < waves; ++w) key = max(key, s_best[w]);
+    const int commonest = 255 - (int)(key & 255u);
+    const bool below = commonest > 0 && (commonest == 255 || s_total[commonest - 1] > s_total[commonest + 1]);
+    const uint32_t b = (uint32_t)(below ? commonest - 1 : commonest);
+    if (t == 0) bases[matrix] = b * 0x01010101u;
+    const int units = tiles * slices;
+    uint32_t* unit_code = code + (size_t)matrix * units * 16;
+    uint32_t* unit_flags = flags + (size_t)matrix * units * 4;
+    for (int unit = wave; unit < units; unit += waves) {
+        const int tile = unit / slices, slice = unit - tile * slices;
+        const int rows = min(128, n - tile * 128), width = min(4, columns - slice * 4);
+        const uint8_t* u = bytes + (size_t)tile * 128 * columns + (size_t)slice * rows * 4;
+        for (int pass = 0; pass < 2; ++pass) {
+            const int r = pass * 64 + lane;
+            bool raw = false;
+            uint32_t bits = 0;
+            if (r < rows) bits = tf_row_bits(tf_unit_row_word(u, r, width), width, b, raw);
+            const unsigned long long raw_rows = __ballot(raw);
+            uint32_t word = raw ? 0u : bits << (4 * (lane & 7));
+            word |= (uint32_t)__shfl_xor((int)word, 1);
+            word |= (uint32_t)__shfl_xor((int)word, 2);
+            word |= (uint32_t)__shfl_xor((int)word, 4);
+            if ((lane & 7) == 0) unit_code[(size_t)unit * 16 + pass * 8 + (lane >> 3)] = word;
+            if (lane < 2) unit_flags[(size_t)unit * 4 + pass * 2 + lane] = (uint32_t)(raw_rows >> (32 * lane));
+        }
     }
 }
-// Decode check: word = flagged ? raw : ((nibble * 0x00204081) & 0x01010101) + base, masked to the width.  Error bit 1: a
-// coded row decodes wrong; bit 2: a flagged row is fully on {b, b + 1}.
-extern "C" __global__ void ca_expert_scale_code1_check(const uint8_t* scales, const uint32_t* code, const uint32_t* flags,
-                                                       const uint32_t* bases, uint32_t* error, int n, int columns) {
-    const int matrix = blockIdx.y, tiles = sc1_tiles(n), slices = sc1_slices(columns);
+// The decode the kernels apply, checked against every row word: word = raw row ? the row's bytes : ((four bits * 0x00204081)
+// & 0x01010101) + base, masked to the width.  Error bit 1: a coded row decodes wrong; bit 2: a raw row lies wholly on
+// {b, b + 1} (the coder never leaves such a row raw).  A wave checks 64 rows of a unit (grid.x * blockDim.x >= units * 128,
+// grid.y = matrices) and reports once, from its ballots.
+extern "C" __global__ void __launch_bounds__(256) ca_expert_scale_code1_check(const uint8_t* scales, const uint32_t* code, const uint32_t* flags,
+                                                                              const uint32_t* bases, uint32_t* error, int n, int columns) {
+    const int lane = threadIdx.x & 63, matrix = blockIdx.y, tiles = (n + 127) / 128, slices = (columns + 3) / 4;
     const size_t units = (size_t)tiles * slices;
-    const size_t row_id = (size_t)blockIdx.x * blockDim.x + threadIdx.x;
-    if (row_id >= units * 128) return;
-    const int unit = (int)(row_id / 128), r = (int)(row_id % 128), tile = unit / slices, slice = unit % slices;
-    const int nr = min(128, n - tile * 128), width = min(4, columns - slice * 4);
-    if (r >= nr) return;
-    const uint8_t* u = scales + (size_t)matrix * n * columns + (size_t)tile * 128 * columns + (size_t)slice * nr * 4 + (size_t)r * width;
-    uint32_t raw = 0;
-    for (int j = 0; j < width; j++) raw |= (uint32_t)u[j] << (8 * j);
-    const uint32_t mask = width == 4 ? 0xffffffffu : (1u << (8 * width)) - 1u;
-    const uint32_t flag = (flags[((size_t)matrix * units + unit) * 4 + r / 32] >> (r % 32)) & 1u;
-    const uint32_t word = code[((size_t)matrix * units + unit) * 16 + r / 8];
-    const uint32_t nibble = (word >> (4 * (r % 8))) & 15u;
-    const uint32_t decoded = (((nibble * 0x00204081u) & 0x01010101u) + bases[matrix]) & mask;
-    if (!flag && decoded != raw) atomicOr(error, 1u);
-    if (flag) {
-        const uint32_t b = bases[matrix] & 255u;
-        bool on = true;
-        for (int j = 0; j < width; j++) { const uint32_t v = (raw >> (8 * j)) & 255u; on = on && (v == b || v == b + 1); }
-        if (on) atomicOr(error, 2u);
+    const size_t half_unit = ((size_t)blockIdx.x * blockDim.x + threadIdx.x) >> 6;          // 64 rows
+    if (half_unit >= units * 2) return;
+    const int unit = (int)(half_unit >> 1), r = (int)(half_unit & 1) * 64 + lane, tile = unit / slices, slice = unit - tile * slices;
+    const int rows = min(128, n - tile * 128), width = min(4, columns - slice * 4);
+    const uint32_t base = bases[matrix], b = base & 255u;
+    bool wrong = false, idle_raw = false;
+    if (r < rows) {
+        const uint8_t* u = scales + (size_t)matrix * n * columns + (size_t)tile * 128 * columns + (size_t)slice * rows * 4;
+        const uint32_t held = tf_unit_row_word(u, r, width);
+        const uint32_t mask = width == 4 ? 0xffffffffu : (1u << (8 * width)) - 1u;
+        const size_t at = (size_t)matrix * units + unit;
+        const bool is_raw = (flags[at * 4 + (r >> 5)] >> (r & 31)) & 1u;
+        const uint32_t four = (code[at * 16 + (r >> 3)] >> (4 * (r & 7))) & 15u;
+        bool off_pair;
+        (void)tf_row_bits(held, width, b, off_pair);
+        wrong = !is_raw && ((((four * 0x00204081u) & 0x01010101u) + base) & mask) != held;
+        idle_raw = is_raw && !off_pair;
     }
+    const uint32_t found = (__ballot(wrong) ? 1u : 0u) | (__ballot(idle_raw) ? 2u : 0u);
+    if (found && lane == 0) atomicOr(error, found);
 }
-extern "C" __global__ void ca_expert_scale_code1_census(const uint32_t* flags, unsigned long long* counts, size_t words) {
+// Raw rows of a coded layer (set flag bits), for the load report: a wave adds its words' bit counts and reports once.
+extern "C" __global__ void __launch_bounds__(256) ca_expert_scale_code1_census(const uint32_t* flags, unsigned long long* counts, size_t words) {
     const size_t i = (size_t)blockIdx.x * blockDim.x + threadIdx.x;
-    if (i >= words) return;
-    const unsigned bits = __popc(flags[i]);
-    if (bits) atomicAdd(counts, (unsigned long long)bits);
+    int bits = i < words ? __popc(flags[i]) : 0;
+#pragma unroll
+    for (int o = 32; o > 0; o >>= 1) bits += __shfl_xor(bits, o);
+    if (bits && (threadIdx.x & 63) == 0) atomicAdd(counts, (unsigned long long)bits);
 }
 // Four-bit row deltas of row-major scale matrices [n][columns]: header byte 4, per-row base at 16 + row, then nibble pairs
 // (a - lo) | (b - lo) << 4, rows of a 128-row tile interleaved two bytes at a time.  Fails closed (error bit 1) when a
