@@ -11,7 +11,8 @@
  * so calls can be captured into a HIP graph.  All pointers are device pointers unless stated otherwise.
  *
  * Shapes are not compiled in: ca_ffn_configure() sets the process geometry used by the fixed-signature entry points,
- * and ca_primitives_open() snapshots it into the context it returns.
+ * and ca_primitives_open() snapshots it into the context it returns; ca_primitives_open_geometry() and the *_in functions
+ * keep a geometry per context, so that layers of different geometries live side by side in one process.
  */
 #ifndef TITANIC_MOE_H
 #define TITANIC_MOE_H
@@ -47,6 +48,13 @@ int ca_shared_swiglu(int rows, const void* input, void* output, void* stream);
 int ca_ffn_add(int rows, const void* routed, const void* shared, void* out, void* stream);
 /* Additive: the gate product for any row count (rows > 16 use the matrix-core kernel, whose summation order differs). */
 int ca_router_logits_wide(int rows, const void* x, const void* w, void* out, void* stream);
+/* Additive: the same four functions with the geometry of a context of ca_primitives_open_geometry instead of the process
+ * geometry, for hosts that keep layers of several geometries in one process (the reference's 384-expert target and
+ * 128-expert drafter, src/layer_id.rs:39-47).  -1 for a null context. */
+int ca_router_logits_in(void* context, int rows, const void* x, const void* w, void* out, void* stream);
+int ca_router_logits_wide_in(void* context, int rows, const void* x, const void* w, void* out, void* stream);
+int ca_shared_swiglu_in(void* context, int rows, const void* input, void* output, void* stream);
+int ca_ffn_add_in(void* context, int rows, const void* routed, const void* shared, void* out, void* stream);
 
 /* ---- kernels the reference resolves by name from a code module (src/cuda.rs:199-226 Module::function + launch) -- */
 /* Launches the `extern "C" __global__` kernel `name` with the reference's launch tuple ([grid;3], [block;3], dynamic
@@ -77,6 +85,9 @@ int ca_pack_bf16(const void* input, uint8_t* packed, int rows, int k, void* stre
 /* ---- operator ABI (src/primitives.rs:45-60, 91-182; bridge.cc) ------------------------------------------------- */
 int32_t ca_primitives_abi(void);                /* returns 1 */
 void* ca_primitives_open(int32_t* status);      /* host handle; snapshots the process geometry and the device's CU count */
+/* Additive: a handle with a geometry of its own; the process geometry is neither read nor written.  -1 null, -4 unsupported. */
+void* ca_primitives_open_geometry(const ca_geometry* geometry, int32_t* status);
+int32_t ca_primitives_geometry(void* context, ca_geometry* out);      /* additive: the handle's geometry */
 void ca_primitives_close(void* context);
 /* Entries, pointer and scalar lists: titanic-flash-41_amd/contracts/bindings.json (same schema as the reference's). */
 int32_t ca_primitives_launch(void* context, int32_t index, const uint64_t* pointers, size_t pointer_count,
@@ -95,6 +106,13 @@ int64_t ca_primitives_scratch_bytes(void* context, int32_t index, int32_t rows);
  * count 0 turns it off.  Not for use while the stream is being captured.  0, or -1 for a null context / event or a count
  * other than 0, 5 or 7. */
 int32_t ca_primitives_marks(void* context, void* const* events, size_t count);
+
+/* No counterpart in the reference (its front-end has no waits inside a launch).  The front-end launch of entries 1 and 9 hands
+ * data from some of its workgroups to others; every such wait is bounded by `limit` polls (default 262,144), after which the
+ * waiter does the work it waited for itself and marks the `sync_ptr` region: later launches then take that path at once
+ * (same results) until the host has zeroed the region again.  limit 0: no hand-off is ever waited for.  0, or -1 for a null
+ * context or a negative limit. */
+int32_t ca_primitives_spin_limit(void* context, int32_t limit);
 
 #ifdef __cplusplus
 }

@@ -90,6 +90,30 @@ def test_argument_validation_needs_no_device():
     assert lib.ca_kernel_launch(b"no_such_kernel", grid, grid, 0, (ctypes.c_void_p * 1)(), None) == -3
 
 
+def test_contexts_carry_their_geometry_and_the_library_is_pinned(tmp_path):
+    import shutil
+    lib = native.load()
+    st = ctypes.c_int32(7)
+    assert not lib.ca_primitives_open_geometry(None, ctypes.byref(st)) and st.value == -1
+    bad = native.Geometry(1000, 16, 2, 512, 512, 0, 1.0, 128, 128, 128, -1, 10.0)
+    assert not lib.ca_primitives_open_geometry(ctypes.byref(bad), ctypes.byref(st)) and st.value == -4
+    assert lib.ca_router_logits_in(None, 1, None, None, None, None) == -1 and lib.ca_ffn_add_in(None, 1, None, None, None, None) == -1
+    assert lib.ca_shared_swiglu_in(None, 1, None, None, None) == -1 and lib.ca_primitives_spin_limit(None, 1) == -1
+    assert lib.ca_primitives_geometry(None, None) == -1
+    # the host mirror refuses a kernel library whose SHA-256 differs from the manifest beside it (src/ffn.rs:70-74), before loading it
+    shutil.copy(native.KERNEL_LIB, tmp_path / "libtitanic_moe_hip.so")
+    (tmp_path / "manifest.json").write_text(json.dumps({"library_sha256": "0" * 64}))
+    host_lib = pkg.host.load()
+    err = ctypes.create_string_buffer(256)
+    g = native.Geometry(1024, 16, 2, 512, 512, 0, 1.0, 128, 128, 128, -1, 10.0)
+    handle = host_lib.tfh_layer_create(str(tmp_path / "libtitanic_moe_hip.so").encode(), ctypes.byref(g), 4, (ctypes.c_void_p * 11)(), 0, 1, 1, 1, 0, 1, 1, err, 256)
+    assert not handle and b"hash mismatch" in err.value
+    # the manifest the build wrote pins the library that is loaded
+    manifest = json.load(open(os.path.join(os.path.dirname(native.KERNEL_LIB), "manifest.json")))
+    import hashlib
+    assert manifest["library_sha256"] == hashlib.sha256(open(native.KERNEL_LIB, "rb").read()).hexdigest()
+
+
 def test_host_library_loads_and_reports_a_missing_kernel_library():
     host = pkg.host
     lib = host.load()

@@ -4,6 +4,7 @@
   titanic_moe_gfx950.hsaco   the same kernels as a code object for hosts that load modules by name
   libtitanic_ffn_host.so     the C++ host mirror of the reference's Rust FFN operators (needs only the HIP runtime)
   tf_layer_probe             stand-alone driver of the layer for profilers (no Python in the process)
+  manifest.json              SHA-256 of the libraries just built; the host mirror refuses a kernel library that differs from it
 """
 import os
 import subprocess
@@ -16,6 +17,7 @@ KERNEL_LIB = os.path.join(HERE, "libtitanic_moe_hip.so")
 CODE_OBJECT = os.path.join(HERE, "titanic_moe_gfx950.hsaco")
 HOST_LIB = os.path.join(HERE, "libtitanic_ffn_host.so")
 PROBE = os.path.join(HERE, "tf_layer_probe")
+MANIFEST = os.path.join(HERE, "manifest.json")
 
 # -ffp-contract=off: bit-exact steps are written as explicit fma / mul / add.  Packed FP32 instructions stay off.
 DEVICE_FLAGS = ["-O3", "--offload-arch=gfx950", "-std=c++17", "-ffp-contract=off", "-Xclang", "-target-feature", "-Xclang",
@@ -53,8 +55,36 @@ def build_probe():
     return PROBE
 
 
+def write_manifest():
+    """manifest.json beside the libraries: what the host mirror pins the kernel library with (the reference pins every native
+    artifact by SHA-256 in its manifests and refuses another: src/ffn.rs:70-74, src/primitives.rs:75-79)."""
+    import hashlib
+    import json
+
+    def digest(path):
+        return hashlib.sha256(open(path, "rb").read()).hexdigest() if os.path.exists(path) else None
+    manifest = {"schema": 1, "architecture": "gfx950", "abi": 1, "library": os.path.basename(KERNEL_LIB), "library_sha256": digest(KERNEL_LIB),
+                "code_object": os.path.basename(CODE_OBJECT), "code_object_sha256": digest(CODE_OBJECT),
+                "host_library": os.path.basename(HOST_LIB), "host_library_sha256": digest(HOST_LIB)}
+    with open(MANIFEST, "w") as f:
+        json.dump(manifest, f, indent=1)
+        f.write("\n")
+    return MANIFEST
+
+
+def write_pinned_contracts():
+    """The operator contracts with the hash of the library just built (contracts/pinned/, beside the committed ones, whose
+    hash fields are null because no library is committed)."""
+    import importlib
+    contracts = importlib.import_module("titanic-flash-41_amd.contracts")
+    contracts.main(os.path.join(HERE, "contracts", "pinned"), KERNEL_LIB)
+
+
 def build():
-    return build_kernels(), build_host(), build_probe()
+    built = build_kernels(), build_host(), build_probe()
+    write_manifest()
+    write_pinned_contracts()
+    return built
 
 
 if __name__ == "__main__":

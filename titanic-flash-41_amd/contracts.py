@@ -109,14 +109,15 @@ def native_contract(g, library):
 BENCHMARK_GEOMETRY = dict(hidden=4096, experts=256, topk=6, intermediate=2048, shared_intermediate=2048, act_block=128, swiglu_limit=10.0)
 
 
-def main():
-    native = importlib.import_module("titanic-flash-41_amd.native")
-    os.makedirs(OUT, exist_ok=True)
-    lib = os.environ.get("TITANIC_MOE_PIN_LIBRARY") and native.KERNEL_LIB   # pin the hash only when packaging a built library
-    json.dump(bindings(lib), open(os.path.join(OUT, "bindings.json"), "w"), indent=1)
-    json.dump(native_contract(BENCHMARK_GEOMETRY, lib), open(os.path.join(OUT, "native.json"), "w"), indent=1)
+def main(out=OUT, library=None):
+    """Writes the contracts to `out`; `library`: the built kernel library whose SHA-256 they pin (None: the hash fields stay
+    null, as in the committed copies, since no library is committed)."""
+    os.makedirs(out, exist_ok=True)
+    lib = library
+    json.dump(bindings(lib), open(os.path.join(out, "bindings.json"), "w"), indent=1)
+    json.dump(native_contract(BENCHMARK_GEOMETRY, lib), open(os.path.join(out, "native.json"), "w"), indent=1)
     for rows in (4, 32, 4096):
-        json.dump(runtime_contract(BENCHMARK_GEOMETRY, rows, lib), open(os.path.join(OUT, "runtime-contract-m%d.json" % rows), "w"), indent=1)
+        json.dump(runtime_contract(BENCHMARK_GEOMETRY, rows, lib), open(os.path.join(out, "runtime-contract-m%d.json" % rows), "w"), indent=1)
 
 
 if __name__ == "__main__":

@@ -38,6 +38,7 @@ struct Context {
     hipEvent_t marks[7];   // profiling aid: see ca_primitives_marks
     bool marking;
     bool kernel_marks;     // marks[5], marks[6]: begin and end of the FC1 + SwiGLU kernel itself
+    int spin_limit;        // polls a wait inside the front-end launch may take before the waiter does the work itself
 };
 
 // Records mark `i` on the launch stream when the caller asked for marks (never while a stream is captured: the caller's duty).
@@ -185,7 +186,7 @@ int launch_dynamic(const Context& c, bool route, const uint64_t* p, const int32_
                     (const float*)p[P_BIAS], (const float*)p[P_BIAS_ALT], (const long long*)p[P_TOKENS], (const int32_t*)p[P_LIVE],
                     (const int32_t*)p[P_PADDING], rows, g.topk, g.experts, g.hidden, groups, tile_m, owner, g.act_block,
                     (uint8_t*)p[P_PACKED_MIN], (uint8_t*)p[P_SCALES_MIN], g.scoring, g.route_scale, (long long)g.alt_token,
-                    (const uint16_t*)p[P_GATE_W], (uint32_t*)p[P_SYNC], logit_blocks, sa, shared_blocks);
+                    (const uint16_t*)p[P_GATE_W], (uint32_t*)p[P_SYNC], logit_blocks, sa, shared_blocks, c.spin_limit);
                 sa.w = nullptr;            // done: the routed experts' first launch runs without it
             } else
             ca_moe_route_frontend<<<quant_blocks + 1 + logit_blocks, 512, 0, s>>>(
@@ -194,7 +195,7 @@ int launch_dynamic(const Context& c, bool route, const uint64_t* p, const int32_
                 (const float*)p[P_BIAS], (const float*)p[P_BIAS_ALT], (const long long*)p[P_TOKENS], (const int32_t*)p[P_LIVE],
                 (const int32_t*)p[P_PADDING], rows, g.topk, g.experts, g.hidden, groups, tile_m, owner, g.act_block,
                 (uint8_t*)p[P_PACKED_MIN], (uint8_t*)p[P_SCALES_MIN], g.scoring, g.route_scale, (long long)g.alt_token,
-                (const uint16_t*)p[P_GATE_W], (uint32_t*)p[P_SYNC], logit_blocks);
+                (const uint16_t*)p[P_GATE_W], (uint32_t*)p[P_SYNC], logit_blocks, c.spin_limit);
         } else {
             ca_moe_frontend<<<quant_blocks, 512, 0, s>>>(
                 x, ids, weights, (uint8_t*)p[P_PACKED], (uint8_t*)p[P_SCALES], (int32_t*)p[P_TOKEN_MAP], (float*)p[P_TOKEN_WEIGHTS],
@@ -312,11 +313,16 @@ int launch_dense(const Context& c, const uint64_t* p, const int32_t* sc, hipStre
     for (int i = 0; i < 5; ++i) if (!p[i]) return -1;
     if (m < 1 || n < 64 || n % 64 || !supported_hidden(k)) return -1;
     if (m <= TF_STREAM_MAX_ROWS) {
-        StreamArgs a{};
+        // few rows (src/fp8_linear.rs:883-897 launches this entry at 6 rows): the streaming kernel of the shared expert's first
+        // projection, whose BF16 projections before the activation are this product; the activation itself is not stored.
+        // Its items pair weight tile j with tile n / 32 + j, so n is a multiple of 32 (of 64 here).
+        StreamArgs a{}, none{};
         a.a_codes = (const uint8_t*)p[0]; a.a_scales = (const uint8_t*)p[1];
         a.w = (const uint8_t*)p[2]; a.ws = (const uint8_t*)p[3]; a.bn = c.g.shared_bn; a.bk = c.g.shared_bk;
-        a.dense_rows = m; a.k = k; a.hidden = n; a.act_block = c.g.act_block; a.out = (uint16_t*)p[4];
-        return -4;   // few-row dense products run inside ffn.shared_expert
+        a.dense_rows = m; a.k = k; a.inter = n / 2; a.hidden = k; a.act_block = c.g.act_block; a.limit = c.g.swiglu_limit;
+        a.out = nullptr; a.tap = (uint16_t*)p[4];
+        if (c.cus <= 0) return (int)hipErrorNoDevice;
+        return launch_phase1(none, a, c.stream_wgs, s);
     }
     GemmArgs a{};
     a.a_codes = (const uint8_t*)p[0]; a.a_scales = (const uint8_t*)p[1];
@@ -400,34 +406,52 @@ int ca_ffn_geometry(ca_geometry* out) {
     *out = g_geometry;
     return 0;
 }
-int ca_router_logits(int rows, const void* x, const void* w, void* out, void* stream) {
+// The four functions of the reference's libcanada_ffn.so keep its signatures, which carry no shapes: they take the process
+// geometry of ca_ffn_configure.  A host that keeps layers of several geometries in one process (the reference's 384-expert
+// target and 128-expert drafter, src/layer_id.rs:39-47) calls the *_in variants, which take the geometry of a context.
+namespace {
+int router_logits_of(const ca_geometry& g, int rows, const void* x, const void* w, void* out, void* stream) {
     if (rows < 1 || rows > 16 || !x || !w || !out) return -1;
-    ca_router_logits_rows<<<g_geometry.experts, 64, 0, (hipStream_t)stream>>>((const uint16_t*)x, (const uint16_t*)w, (float*)out, rows,
-                                                                              g_geometry.hidden, g_geometry.experts);
+    ca_router_logits_rows<<<g.experts, 64, 0, (hipStream_t)stream>>>((const uint16_t*)x, (const uint16_t*)w, (float*)out, rows, g.hidden, g.experts);
     return launch_status();
 }
-int ca_router_logits_wide(int rows, const void* x, const void* w, void* out, void* stream) {
+int router_logits_wide_of(const ca_geometry& g, int rows, const void* x, const void* w, void* out, void* stream) {
     if (rows < 1 || !x || !w || !out) return -1;
-    if (rows <= 16) return ca_router_logits(rows, x, w, out, stream);
-    if (g_geometry.hidden % 64) return -4;
-    const dim3 grid((rows + 127) / 128, (g_geometry.experts + 255) / 256);
-    ca_router_logits_mfma<<<grid, 512, 0, (hipStream_t)stream>>>((const uint16_t*)x, (const uint16_t*)w, (float*)out, rows,
-                                                                 g_geometry.hidden, g_geometry.experts);
+    if (rows <= 16) return router_logits_of(g, rows, x, w, out, stream);
+    if (g.hidden % 64) return -4;
+    const dim3 grid((rows + 127) / 128, (g.experts + 255) / 256);
+    ca_router_logits_mfma<<<grid, 512, 0, (hipStream_t)stream>>>((const uint16_t*)x, (const uint16_t*)w, (float*)out, rows, g.hidden, g.experts);
     return launch_status();
 }
-int ca_shared_swiglu(int rows, const void* input, void* output, void* stream) {
+int shared_swiglu_of(const ca_geometry& g, int rows, const void* input, void* output, void* stream) {
     if (rows < 1 || rows > 65536 || !input || !output) return -1;
-    const long long items = (long long)rows * (g_geometry.shared_intermediate >> 3);
-    ca_shared_swiglu_rows<<<(int)((items + 255) / 256), 256, 0, (hipStream_t)stream>>>(
-        (const uint16_t*)input, (uint16_t*)output, rows, g_geometry.shared_intermediate, g_geometry.swiglu_limit);
+    const long long items = (long long)rows * (g.shared_intermediate >> 3);
+    ca_shared_swiglu_rows<<<(int)((items + 255) / 256), 256, 0, (hipStream_t)stream>>>((const uint16_t*)input, (uint16_t*)output, rows,
+                                                                                       g.shared_intermediate, g.swiglu_limit);
     return launch_status();
 }
-int ca_ffn_add(int rows, const void* routed, const void* shared, void* out, void* stream) {
+int ffn_add_of(const ca_geometry& g, int rows, const void* routed, const void* shared, void* out, void* stream) {
     if (rows < 1 || rows > 65536 || !routed || !shared || !out) return -1;
-    const long long n8 = (long long)rows * (g_geometry.hidden >> 3);
-    ca_ffn_add_rows<<<(int)((n8 + 255) / 256), 256, 0, (hipStream_t)stream>>>((const uint16_t*)routed, (const uint16_t*)shared,
-                                                                              (uint16_t*)out, n8);
+    const long long n8 = (long long)rows * (g.hidden >> 3);
+    ca_ffn_add_rows<<<(int)((n8 + 255) / 256), 256, 0, (hipStream_t)stream>>>((const uint16_t*)routed, (const uint16_t*)shared, (uint16_t*)out, n8);
     return launch_status();
+}
+}  // namespace
+int ca_router_logits(int rows, const void* x, const void* w, void* out, void* stream) { return router_logits_of(g_geometry, rows, x, w, out, stream); }
+int ca_router_logits_wide(int rows, const void* x, const void* w, void* out, void* stream) { return router_logits_wide_of(g_geometry, rows, x, w, out, stream); }
+int ca_shared_swiglu(int rows, const void* input, void* output, void* stream) { return shared_swiglu_of(g_geometry, rows, input, output, stream); }
+int ca_ffn_add(int rows, const void* routed, const void* shared, void* out, void* stream) { return ffn_add_of(g_geometry, rows, routed, shared, out, stream); }
+int ca_router_logits_in(void* context, int rows, const void* x, const void* w, void* out, void* stream) {
+    return context ? router_logits_of(((const Context*)context)->g, rows, x, w, out, stream) : -1;
+}
+int ca_router_logits_wide_in(void* context, int rows, const void* x, const void* w, void* out, void* stream) {
+    return context ? router_logits_wide_of(((const Context*)context)->g, rows, x, w, out, stream) : -1;
+}
+int ca_shared_swiglu_in(void* context, int rows, const void* input, void* output, void* stream) {
+    return context ? shared_swiglu_of(((const Context*)context)->g, rows, input, output, stream) : -1;
+}
+int ca_ffn_add_in(void* context, int rows, const void* routed, const void* shared, void* out, void* stream) {
+    return context ? ffn_add_of(((const Context*)context)->g, rows, routed, shared, out, stream) : -1;
 }
 int ca_moe_nibble_permute(void* data, uint64_t bytes, int inverse, void* stream) {
     if (!data || bytes % 4 || (inverse != 0 && inverse != 1)) return -1;
@@ -472,21 +496,24 @@ int ca_kernel_launch(const char* name, const uint32_t grid[3], const uint32_t bl
 
 int32_t ca_primitives_abi(void) { return 1; }
 int32_t ca_primitives_entries(void) { return kEntryCount; }
-void* ca_primitives_open(int32_t* status) {
+void* ca_primitives_open_geometry(const ca_geometry* geometry, int32_t* status) {
     if (!status) return nullptr;
-    *status = check_geometry(g_geometry);
+    if (!geometry) { *status = -1; return nullptr; }
+    *status = check_geometry(*geometry);
     if (*status) return nullptr;
     int device = 0, cus = 0;
     hipError_t e = hipGetDevice(&device);
     if (e == hipSuccess) e = hipDeviceGetAttribute(&cus, hipDeviceAttributeMultiprocessorCount, device);
     if (e != hipSuccess) { *status = (int32_t)e; return nullptr; }
     Context* c = new Context{};
-    c->g = g_geometry; c->cus = cus; c->stream_wgs = cus * 2;
-    if (const char* v = std::getenv("TITANIC_MOE_STREAM_WGS_PER_CU")) {
-        const int n = std::atoi(v);
-        if (n >= 1 && n <= 8) c->stream_wgs = cus * n;
-    }
+    c->g = *geometry; c->cus = cus; c->stream_wgs = cus * 2; c->spin_limit = 1 << 18;
     return c;
+}
+void* ca_primitives_open(int32_t* status) { return ca_primitives_open_geometry(&g_geometry, status); }
+int32_t ca_primitives_geometry(void* context, ca_geometry* out) {
+    if (!context || !out) return -1;
+    *out = ((const Context*)context)->g;
+    return 0;
 }
 void ca_primitives_close(void* context) { delete (Context*)context; }
 int32_t ca_primitives_marks(void* context, void* const* events, size_t count) {
@@ -498,6 +525,11 @@ int32_t ca_primitives_marks(void* context, void* const* events, size_t count) {
         if (!events[i]) { c->marking = c->kernel_marks = false; return -1; }
         c->marks[i] = (hipEvent_t)events[i];
     }
+    return 0;
+}
+int32_t ca_primitives_spin_limit(void* context, int32_t limit) {
+    if (!context || limit < 0) return -1;
+    ((Context*)context)->spin_limit = limit;
     return 0;
 }
 int32_t ca_primitives_launch(void* context, int32_t index, const uint64_t* pointers, size_t np, const int32_t* scalars, size_t ns,

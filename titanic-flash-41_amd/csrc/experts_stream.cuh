@@ -296,7 +296,7 @@ __device__ __forceinline__ void tf_fc1_items(const StreamArgs& p, int item_first
                         const float u = fminf(p.limit, fmaxf(-p.limit, first));
                         value = __fmul_rn(__fmul_rn(g, tf_logistic(g)), u);
                     }
-                    p.out[row * p.inter + 16 * r.j + (lane & 15)] = tf_to_bf16(value);
+                    if (!FP8 || p.out != nullptr) p.out[row * p.inter + 16 * r.j + (lane & 15)] = tf_to_bf16(value);      // dense product alone: only the tap
                 }
             }
         }
@@ -465,7 +465,7 @@ __global__ void __launch_bounds__(256, 2) tf_phase2_stream(const StreamArgs rout
 // order, same activation).
 template <int KS, bool HANDOFF>
 __device__ __forceinline__ void tf_front_shared_item(const StreamArgs& p, const uint16_t* __restrict__ all_rows, int all_row_count, uint8_t* s_pool,
-                                                     int item, uint32_t* sync, int quant_blocks, int shared_blocks) {
+                                                     int item, uint32_t* sync, int quant_blocks, int shared_blocks, int spin_limit) {
     const int k = p.k, per_row = k >> 3, group_lanes = p.act_block >> 3;
     const int per_tile = p.inter / 16, tiles = (all_row_count + 15) >> 4;
     uint8_t* s_codes = s_pool;                                        // [rows][k]             (at most 64 KiB)
@@ -475,16 +475,20 @@ __device__ __forceinline__ void tf_front_shared_item(const StreamArgs& p, const 
     const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6, half = wave >> 2, quarter = wave & 3, ks_first = quarter * KS;
     // `quant_blocks` > 0: the launch's quantizer blocks publish the rows' codes (shared flavour) and count themselves in; this
     // block waits for all of them (a bounded wait: they have lower block ids, none of them waits for anything) and reads its
-    // operand from their output instead of quantizing every row again.  Should the bound expire it quantizes them itself.
+    // operand from their output instead of quantizing every row again.  Should the bound expire, or have expired in an earlier
+    // launch (the arrival word may then hold that launch's late arrivals), it quantizes them itself.
     // The wait comes before the first weight request: a workgroup barrier waits for every load in flight.
     bool ready = false;
     if constexpr (HANDOFF) {
         __shared__ int s_ready;
         if (threadIdx.x == 0) {
             int ok = 0;
-            for (int spin = 0; spin < (1 << 18); ++spin) {
-                if (__hip_atomic_load(sync + 32 * TF_SYNC_QUANT_DONE, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT) >= (uint32_t)quant_blocks) { ok = 1; break; }
-                __builtin_amdgcn_s_sleep(2);
+            if (tf_sync_trusted(sync)) {
+                for (int spin = 0; spin < spin_limit; ++spin) {
+                    if (__hip_atomic_load(sync + 32 * TF_SYNC_QUANT_DONE, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT) >= (uint32_t)quant_blocks) { ok = 1; break; }
+                    __builtin_amdgcn_s_sleep(2);
+                }
+                if (!ok) tf_sync_give_up(sync);
             }
             s_ready = ok;
         }
@@ -567,7 +571,7 @@ __device__ __forceinline__ void tf_front_shared_item(const StreamArgs& p, const 
     }
     // every wave's operands have been consumed (the last tile's barrier): the last item block to get here empties both arrival
     // words for the next launch
-    if (HANDOFF && threadIdx.x == 0 && atomicAdd(sync + 32 * TF_SYNC_SHARED_PASSED, 1u) == (uint32_t)(shared_blocks - 1)) {
+    if (HANDOFF && ready && threadIdx.x == 0 && atomicAdd(sync + 32 * TF_SYNC_SHARED_PASSED, 1u) == (uint32_t)(shared_blocks - 1)) {
         __hip_atomic_store(sync + 32 * TF_SYNC_QUANT_DONE, 0u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
         __hip_atomic_store(sync + 32 * TF_SYNC_SHARED_PASSED, 0u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
     }
@@ -580,7 +584,7 @@ extern "C" __global__ void __launch_bounds__(512) ca_moe_route_frontend_shared(
     const int32_t* padding, int32_t rows, int32_t topk, int32_t experts, int32_t cols, int32_t groups, int32_t tile_m,
     int32_t owner_rows, int32_t act_block, uint8_t* packed_min, uint8_t* scales_min, int32_t scoring,
     float route_scale, long long alt_token, const uint16_t* gate_w, uint32_t* sync, int32_t logit_blocks, const StreamArgs shared,
-    int32_t shared_blocks) {
+    int32_t shared_blocks, int32_t spin_limit) {
     __shared__ __attribute__((aligned(16))) uint8_t s_pool[TF_FRONT_POOL_BYTES];
     const int grid_blocks = (int)gridDim.x - shared_blocks;
     // more than one row tile: the item blocks take the rows' codes from the launch's quantizer blocks (one tile: they quantize the
@@ -591,28 +595,28 @@ extern "C" __global__ void __launch_bounds__(512) ca_moe_route_frontend_shared(
         const int quant_blocks = grid_blocks - logit_blocks - 1;
         if (handoff) {
             switch (shared.k) {
-                case 512: tf_front_shared_item<1, true>(shared, input, rows, s_pool, block, sync, quant_blocks, shared_blocks); break;
-                case 1024: tf_front_shared_item<2, true>(shared, input, rows, s_pool, block, sync, quant_blocks, shared_blocks); break;
-                case 1536: tf_front_shared_item<3, true>(shared, input, rows, s_pool, block, sync, quant_blocks, shared_blocks); break;
-                case 2048: tf_front_shared_item<4, true>(shared, input, rows, s_pool, block, sync, quant_blocks, shared_blocks); break;
-                case 2560: tf_front_shared_item<5, true>(shared, input, rows, s_pool, block, sync, quant_blocks, shared_blocks); break;
-                case 3072: tf_front_shared_item<6, true>(shared, input, rows, s_pool, block, sync, quant_blocks, shared_blocks); break;
-                case 3584: tf_front_shared_item<7, true>(shared, input, rows, s_pool, block, sync, quant_blocks, shared_blocks); break;
-                case 4096: tf_front_shared_item<8, true>(shared, input, rows, s_pool, block, sync, quant_blocks, shared_blocks); break;
-                case 5120: tf_front_shared_item<10, true>(shared, input, rows, s_pool, block, sync, quant_blocks, shared_blocks); break;
+                case 512: tf_front_shared_item<1, true>(shared, input, rows, s_pool, block, sync, quant_blocks, shared_blocks, spin_limit); break;
+                case 1024: tf_front_shared_item<2, true>(shared, input, rows, s_pool, block, sync, quant_blocks, shared_blocks, spin_limit); break;
+                case 1536: tf_front_shared_item<3, true>(shared, input, rows, s_pool, block, sync, quant_blocks, shared_blocks, spin_limit); break;
+                case 2048: tf_front_shared_item<4, true>(shared, input, rows, s_pool, block, sync, quant_blocks, shared_blocks, spin_limit); break;
+                case 2560: tf_front_shared_item<5, true>(shared, input, rows, s_pool, block, sync, quant_blocks, shared_blocks, spin_limit); break;
+                case 3072: tf_front_shared_item<6, true>(shared, input, rows, s_pool, block, sync, quant_blocks, shared_blocks, spin_limit); break;
+                case 3584: tf_front_shared_item<7, true>(shared, input, rows, s_pool, block, sync, quant_blocks, shared_blocks, spin_limit); break;
+                case 4096: tf_front_shared_item<8, true>(shared, input, rows, s_pool, block, sync, quant_blocks, shared_blocks, spin_limit); break;
+                case 5120: tf_front_shared_item<10, true>(shared, input, rows, s_pool, block, sync, quant_blocks, shared_blocks, spin_limit); break;
                 default: break;
             }
         } else {
             switch (shared.k) {
-                case 512: tf_front_shared_item<1, false>(shared, input, rows, s_pool, block, sync, 0, shared_blocks); break;
-                case 1024: tf_front_shared_item<2, false>(shared, input, rows, s_pool, block, sync, 0, shared_blocks); break;
-                case 1536: tf_front_shared_item<3, false>(shared, input, rows, s_pool, block, sync, 0, shared_blocks); break;
-                case 2048: tf_front_shared_item<4, false>(shared, input, rows, s_pool, block, sync, 0, shared_blocks); break;
-                case 2560: tf_front_shared_item<5, false>(shared, input, rows, s_pool, block, sync, 0, shared_blocks); break;
-                case 3072: tf_front_shared_item<6, false>(shared, input, rows, s_pool, block, sync, 0, shared_blocks); break;
-                case 3584: tf_front_shared_item<7, false>(shared, input, rows, s_pool, block, sync, 0, shared_blocks); break;
-                case 4096: tf_front_shared_item<8, false>(shared, input, rows, s_pool, block, sync, 0, shared_blocks); break;
-                case 5120: tf_front_shared_item<10, false>(shared, input, rows, s_pool, block, sync, 0, shared_blocks); break;
+                case 512: tf_front_shared_item<1, false>(shared, input, rows, s_pool, block, sync, 0, shared_blocks, spin_limit); break;
+                case 1024: tf_front_shared_item<2, false>(shared, input, rows, s_pool, block, sync, 0, shared_blocks, spin_limit); break;
+                case 1536: tf_front_shared_item<3, false>(shared, input, rows, s_pool, block, sync, 0, shared_blocks, spin_limit); break;
+                case 2048: tf_front_shared_item<4, false>(shared, input, rows, s_pool, block, sync, 0, shared_blocks, spin_limit); break;
+                case 2560: tf_front_shared_item<5, false>(shared, input, rows, s_pool, block, sync, 0, shared_blocks, spin_limit); break;
+                case 3072: tf_front_shared_item<6, false>(shared, input, rows, s_pool, block, sync, 0, shared_blocks, spin_limit); break;
+                case 3584: tf_front_shared_item<7, false>(shared, input, rows, s_pool, block, sync, 0, shared_blocks, spin_limit); break;
+                case 4096: tf_front_shared_item<8, false>(shared, input, rows, s_pool, block, sync, 0, shared_blocks, spin_limit); break;
+                case 5120: tf_front_shared_item<10, false>(shared, input, rows, s_pool, block, sync, 0, shared_blocks, spin_limit); break;
                 default: break;
             }
         }
@@ -620,6 +624,6 @@ extern "C" __global__ void __launch_bounds__(512) ca_moe_route_frontend_shared(
     }
     tf_route_frontend(input, ids, weights, packed, scales, token_map, token_weights, task_expert, task_valid_rows, expert_tile_base, logits, bias,
                       bias_alt, tokens, live, padding, rows, topk, experts, cols, groups, tile_m, owner_rows, act_block, packed_min, scales_min,
-                      scoring, route_scale, alt_token, gate_w, sync, logit_blocks, grid_blocks, s_pool, handoff);
+                      scoring, route_scale, alt_token, gate_w, sync, logit_blocks, grid_blocks, s_pool, spin_limit, handoff);
 }
 

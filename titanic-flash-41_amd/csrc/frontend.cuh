@@ -154,11 +154,23 @@ extern "C" __global__ void __launch_bounds__(512) ca_moe_frontend(
 // logits.  Owners of at most eight rows: the logits are handed to block 0 through a mailbox of one word a logit (`sync` +
 // 4 KiB: zero = empty; block 0 polls every word, takes the value and empties the word again), so neither side waits for a
 // store to complete or for a counter.  Larger owners: the blocks publish the logits and count themselves in at `sync`
-// (seventeen words, 128 bytes apart).  The whole `sync` region is zero before the first launch and every launch leaves it
-// zero.  Every wait is bounded: if the logits do not arrive block 0 computes them itself, so the kernel always ends.  All
-// blocks of this small grid are resident together.
+// (seventeen words, 128 bytes apart).  The whole `sync` region is zero before the first launch, and a launch whose waits all
+// end in time leaves it zero.  Every wait is bounded by `spin_limit` polls: the waiter then does the work it waited for itself
+// (block 0 forms the logits and routes every row; an item block quantizes its rows), so the kernel always ends, and sets the
+// word TF_SYNC_DIRTY, which is never cleared by a kernel: what the late producers still post stays in the region, so from
+// then on no launch trusts a hand-off (every waiter takes its own path at once, the results stay the same) until the host
+// has zeroed the region again.  The blocks a waiter waits for need not all be resident with it: workgroups are dispatched in
+// block order, the waited-for blocks wait for nothing themselves, and the blocks before them (quantizer blocks) end without
+// waiting, so they reach a CU while the waiter polls; the bound covers whatever breaks that assumption.
 #define TF_SYNC_QUANT_DONE 17             // arrival words (128 bytes apart) of the launch that also runs the shared expert's first projection:
 #define TF_SYNC_SHARED_PASSED 18          // quantizer blocks that are done; item blocks that have read the quantizer's output
+#define TF_SYNC_DIRTY 19                  // a bounded wait has expired since the host last zeroed the region
+__device__ __forceinline__ bool tf_sync_trusted(const uint32_t* sync) {
+    return __hip_atomic_load(sync + 32 * TF_SYNC_DIRTY, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT) == 0u;
+}
+__device__ __forceinline__ void tf_sync_give_up(uint32_t* sync) {
+    __hip_atomic_store(sync + 32 * TF_SYNC_DIRTY, 1u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+}
 #define TF_FRONT_SHARED_MAX_K 5120         // widest token row whose shared up / gate projection runs inside the front-end launch
 // the shared expert's item blocks hold a 16-row tile's codes, its scales (32-wide blocks at most) and two sets of partial sums
 #define TF_FRONT_POOL_BYTES (16 * TF_FRONT_SHARED_MAX_K + 16 * (TF_FRONT_SHARED_MAX_K / 32) + 16384)
@@ -171,7 +183,7 @@ __device__ __forceinline__ void tf_route_frontend(
     const int32_t* padding, int32_t rows, int32_t topk, int32_t experts, int32_t cols, int32_t groups, int32_t tile_m,
     int32_t owner_rows, int32_t act_block, uint8_t* packed_min, uint8_t* scales_min, int32_t scoring,
     float route_scale, long long alt_token, const uint16_t* gate_w, uint32_t* sync, int32_t logit_blocks, int grid_blocks,
-    uint8_t* s_pool, bool publish_min = false) {
+    uint8_t* s_pool, int32_t spin_limit, bool publish_min = false) {
     __shared__ __attribute__((aligned(16))) int32_t s_ids[1024];
     __shared__ float s_weights[1024];
     const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6, waves = blockDim.x >> 6;
@@ -231,23 +243,26 @@ __device__ __forceinline__ void tf_route_frontend(
                 if (t < owner_rows && tokens != nullptr) my_token = tokens[t];
                 if (t == 0) my_live = live[0];
             }
-            if (threadIdx.x == 0) arrived = 1;
+            const bool trusted = tf_sync_trusted(sync);            // uniform: one word
+            if (threadIdx.x == 0) arrived = trusted ? 1 : 0;
             __syncthreads();
-            if (distributed) {
+            if (!trusted) {
+                // a wait has expired in some earlier launch: the region may hold that launch's words; nothing of it is read
+            } else if (distributed) {
                 if (threadIdx.x < 64) {
                     int ok = 0;
-                    for (int spin = 0; spin < (1 << 18); ++spin) {
+                    for (int spin = 0; spin < spin_limit; ++spin) {
                         if (__hip_atomic_load(routed_groups, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT) >= (uint32_t)row_groups) { ok = 1; break; }
                         __builtin_amdgcn_s_sleep(2);
                     }
-                    if (lane == 0) __hip_atomic_store(routed_groups, 0u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
-                    if (lane == 0 && !ok) arrived = 0;
+                    if (lane == 0 && ok) __hip_atomic_store(routed_groups, 0u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+                    if (lane == 0 && !ok) { arrived = 0; tf_sync_give_up(sync); }
                 }
             } else {
                 // every thread takes its words of the mailbox as they arrive and empties them for the next launch
                 for (int i = threadIdx.x; i < owner_rows * experts; i += blockDim.x) {
                     uint32_t word = 0;
-                    for (int spin = 0; spin < (1 << 18); ++spin) {
+                    for (int spin = 0; spin < spin_limit; ++spin) {
                         word = __hip_atomic_load(mailbox + i, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
                         if (word != 0u) break;
                         __builtin_amdgcn_s_sleep(1);
@@ -257,6 +272,7 @@ __device__ __forceinline__ void tf_route_frontend(
                         __hip_atomic_store(mailbox + i, 0u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
                     } else {
                         arrived = 0;
+                        tf_sync_give_up(sync);
                     }
                 }
                 if (t < experts) { s_bias[t] = my_bias; s_bias[512 + t] = my_alt; }
@@ -264,7 +280,7 @@ __device__ __forceinline__ void tf_route_frontend(
                 if (t == 0) *s_live = my_live;
             }
             __syncthreads();
-            if (!arrived) {              // the bound expired: this block forms the logits (and routes) itself, so the kernel always ends
+            if (!arrived) {              // a bound expired (now or in an earlier launch): this block forms the logits (and routes) itself
                 for (int e = wave; e < experts; e += waves) tf_logits_expert(input, gate_w, logits, owner_rows, cols, experts, e, lane);
                 tf_stores_done();
                 __syncthreads();
@@ -309,11 +325,11 @@ extern "C" __global__ void __launch_bounds__(512) ca_moe_route_frontend(
     float* logits, const float* bias, const float* bias_alt, const long long* tokens, const int32_t* live,
     const int32_t* padding, int32_t rows, int32_t topk, int32_t experts, int32_t cols, int32_t groups, int32_t tile_m,
     int32_t owner_rows, int32_t act_block, uint8_t* packed_min, uint8_t* scales_min, int32_t scoring,
-    float route_scale, long long alt_token, const uint16_t* gate_w, uint32_t* sync, int32_t logit_blocks) {
+    float route_scale, long long alt_token, const uint16_t* gate_w, uint32_t* sync, int32_t logit_blocks, int32_t spin_limit) {
     __shared__ __attribute__((aligned(16))) uint8_t s_pool[TF_FRONT_POOL_BYTES];
     tf_route_frontend(input, ids, weights, packed, scales, token_map, token_weights, task_expert, task_valid_rows, expert_tile_base, logits, bias,
                       bias_alt, tokens, live, padding, rows, topk, experts, cols, groups, tile_m, owner_rows, act_block, packed_min, scales_min,
-                      scoring, route_scale, alt_token, gate_w, sync, logit_blocks, (int)gridDim.x, s_pool);
+                      scoring, route_scale, alt_token, gate_w, sync, logit_blocks, (int)gridDim.x, s_pool, spin_limit);
 }
 // Row quantizer alone (any number of rows).
 extern "C" __global__ void __launch_bounds__(256) ca_quantize_rows(

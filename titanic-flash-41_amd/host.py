@@ -11,6 +11,7 @@ HERE = os.path.dirname(os.path.abspath(__file__))
 HOST_LIB = os.path.join(HERE, "libtitanic_ffn_host.so")
 _lib = None
 
+EXTRA_TAPS = {"sync": np.uint32}       # the front-end's hand-off region (not a layer tap: not in taps())
 TAPS = {"logits": np.float32, "ids": np.int32, "weights": np.float32, "xq": np.uint8, "xs": np.uint8, "xq_min": np.uint8,
         "xs_min": np.uint8, "h": np.uint16, "hq": np.uint8, "hs": np.uint8, "task_expert": np.int32, "task_valid": np.int32,
         "tile_base": np.int32, "token_map": np.int32, "token_weights": np.float32, "route_out": np.uint16, "routed": np.uint16,
@@ -178,9 +179,20 @@ class Layer:
                                                 oa.ctypes.data_as(ctypes.c_void_p), ob.ctypes.data_as(ctypes.c_void_p), self._err, 512))
         return oa, ob
 
+    def spin_limit(self, limit):
+        """Polls a wait inside the front-end launch may take before the waiter does the work itself (0: gives up at once)."""
+        self.lib.tfh_layer_spin_limit.argtypes = [ctypes.c_void_p, ctypes.c_int, ctypes.c_char_p, ctypes.c_size_t]
+        self._check(self.lib.tfh_layer_spin_limit(self.h, limit, self._err, 512))
+
+    def zero_sync(self):
+        """The host's reset of the front-end's hand-off region (after a wait has expired)."""
+        self.lib.tfh_layer_zero_sync.argtypes = [ctypes.c_void_p, ctypes.c_char_p, ctypes.c_size_t]
+        self._check(self.lib.tfh_layer_zero_sync(self.h, self._err, 512))
+
     def tap(self, name):
+        dtype = TAPS.get(name) or EXTRA_TAPS[name]
         size = self._check(self.lib.tfh_layer_tap(self.h, name.encode(), None, 0, self._err, 512))
-        out = np.empty(size // np.dtype(TAPS[name]).itemsize, TAPS[name])
+        out = np.empty(size // np.dtype(dtype).itemsize, dtype)
         self._check(self.lib.tfh_layer_tap(self.h, name.encode(), out.ctypes.data, size, self._err, 512))
         return out
 

@@ -109,6 +109,18 @@ void tfh_layer_destroy(void* handle) { delete (Handle*)handle; }
 // The geometry the layer runs with (the caller's, with the expert widths padded to multiples of 512): the widths of the taps.
 void tfh_layer_geometry(void* handle, ca_geometry* out) { *out = ((Handle*)handle)->native->geometry(); }
 // Many rows: drop (0) or keep (1) the BF16 tap of the routed intermediate.
+// Test hooks of the front-end's in-launch hand-offs: the bound of its waits, and the host's reset of the `sync` region.
+int tfh_layer_spin_limit(void* handle, int limit, char* error, size_t error_len) {
+    Handle* h = (Handle*)handle;
+    return guarded(error, error_len, [&] { h->native->spin_limit(limit); });
+}
+int tfh_layer_zero_sync(void* handle, char* error, size_t error_len) {
+    Handle* h = (Handle*)handle;
+    return guarded(error, error_len, [&] {
+        h->stream->synchronize();
+        tf::check(hipMemset((void*)h->workspace->at("sync_ptr"), 0, h->workspace->bytes_of("sync_ptr")), "zero sync region");
+    });
+}
 void tfh_layer_keep_intermediate(void* handle, int on) { ((Handle*)handle)->workspace->keep_intermediate(on != 0); }
 
 int tfh_layer_set_tokens(void* handle, const int64_t* ids, int live, const int32_t* padding, char* error, size_t error_len) {
@@ -314,7 +326,7 @@ long long tfh_layer_tap(void* handle, const char* name, void* out, size_t bytes,
                 {"xq", "packed_a_storage_ptr"}, {"xs", "scale_storage_ptr"}, {"xq_min", "shared_a_storage_ptr"}, {"xs_min", "shared_scale_storage_ptr"},
                 {"h", "intermediate_ptr"}, {"hq", "intermediate_codes_ptr"}, {"hs", "intermediate_scales_ptr"}, {"task_expert", "task_expert_ptr"},
                 {"task_valid", "task_valid_rows_ptr"}, {"tile_base", "expert_tile_base"}, {"token_map", "token_map_ptr"},
-                {"token_weights", "token_weights_ptr"}, {"route_out", "scatter_ptr"}};
+                {"token_weights", "token_weights_ptr"}, {"route_out", "scatter_ptr"}, {"sync", "sync_ptr"}};
             auto it = alias.find(n);
             tf::ensure(it != alias.end(), "unknown tap");
             buf(w.at(it->second), w.bytes_of(it->second));

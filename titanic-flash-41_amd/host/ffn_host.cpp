@@ -2,6 +2,9 @@
 #include "ffn_host.hpp"
 #include <dlfcn.h>
 #include <algorithm>
+#include <cstdio>
+#include <fstream>
+#include <vector>
 
 namespace tf {
 
@@ -13,20 +16,75 @@ F symbol(void* lib, const char* name) {
     return reinterpret_cast<F>(p);
 }
 size_t align256(size_t n) { return (n + 255) / 256 * 256; }
+
+// SHA-256 (FIPS 180-4) of a file, as lower-case hexadecimal; empty when the file cannot be read.
+std::string sha256_file(const std::string& path) {
+    static const uint32_t K[64] = {
+        0x428a2f98, 0x71374491, 0xb5c0fbcf, 0xe9b5dba5, 0x3956c25b, 0x59f111f1, 0x923f82a4, 0xab1c5ed5, 0xd807aa98, 0x12835b01, 0x243185be,
+        0x550c7dc3, 0x72be5d74, 0x80deb1fe, 0x9bdc06a7, 0xc19bf174, 0xe49b69c1, 0xefbe4786, 0x0fc19dc6, 0x240ca1cc, 0x2de92c6f, 0x4a7484aa,
+        0x5cb0a9dc, 0x76f988da, 0x983e5152, 0xa831c66d, 0xb00327c8, 0xbf597fc7, 0xc6e00bf3, 0xd5a79147, 0x06ca6351, 0x14292967, 0x27b70a85,
+        0x2e1b2138, 0x4d2c6dfc, 0x53380d13, 0x650a7354, 0x766a0abb, 0x81c2c92e, 0x92722c85, 0xa2bfe8a1, 0xa81a664b, 0xc24b8b70, 0xc76c51a3,
+        0xd192e819, 0xd6990624, 0xf40e3585, 0x106aa070, 0x19a4c116, 0x1e376c08, 0x2748774c, 0x34b0bcb5, 0x391c0cb3, 0x4ed8aa4a, 0x5b9cca4f,
+        0x682e6ff3, 0x748f82ee, 0x78a5636f, 0x84c87814, 0x8cc70208, 0x90befffa, 0xa4506ceb, 0xbef9a3f7, 0xc67178f2};
+    std::ifstream in(path, std::ios::binary);
+    if (!in) return std::string();
+    std::vector<uint8_t> data((std::istreambuf_iterator<char>(in)), std::istreambuf_iterator<char>());
+    const uint64_t bits = (uint64_t)data.size() * 8;
+    data.push_back(0x80);
+    while (data.size() % 64 != 56) data.push_back(0);
+    for (int i = 7; i >= 0; --i) data.push_back((uint8_t)(bits >> (8 * i)));
+    uint32_t h[8] = {0x6a09e667, 0xbb67ae85, 0x3c6ef372, 0xa54ff53a, 0x510e527f, 0x9b05688c, 0x1f83d9ab, 0x5be0cd19};
+    auto rotr = [](uint32_t v, int n) { return (v >> n) | (v << (32 - n)); };
+    for (size_t at = 0; at < data.size(); at += 64) {
+        uint32_t w[64];
+        for (int i = 0; i < 16; ++i) w[i] = (uint32_t)data[at + 4 * i] << 24 | (uint32_t)data[at + 4 * i + 1] << 16 | (uint32_t)data[at + 4 * i + 2] << 8 | data[at + 4 * i + 3];
+        for (int i = 16; i < 64; ++i)
+            w[i] = w[i - 16] + (rotr(w[i - 15], 7) ^ rotr(w[i - 15], 18) ^ (w[i - 15] >> 3)) + w[i - 7] + (rotr(w[i - 2], 17) ^ rotr(w[i - 2], 19) ^ (w[i - 2] >> 10));
+        uint32_t v[8];
+        for (int i = 0; i < 8; ++i) v[i] = h[i];
+        for (int i = 0; i < 64; ++i) {
+            const uint32_t t1 = v[7] + (rotr(v[4], 6) ^ rotr(v[4], 11) ^ rotr(v[4], 25)) + ((v[4] & v[5]) ^ (~v[4] & v[6])) + K[i] + w[i];
+            const uint32_t t2 = (rotr(v[0], 2) ^ rotr(v[0], 13) ^ rotr(v[0], 22)) + ((v[0] & v[1]) ^ (v[0] & v[2]) ^ (v[1] & v[2]));
+            v[7] = v[6]; v[6] = v[5]; v[5] = v[4]; v[4] = v[3] + t1; v[3] = v[2]; v[2] = v[1]; v[1] = v[0]; v[0] = t1 + t2;
+        }
+        for (int i = 0; i < 8; ++i) h[i] += v[i];
+    }
+    char hex[65];
+    for (int i = 0; i < 8; ++i) std::snprintf(hex + 8 * i, 9, "%08x", h[i]);
+    return std::string(hex, 64);
+}
+// The value of "library_sha256" in the manifest the build writes beside the library (manifest.json); empty when absent.
+std::string manifest_sha256(const std::string& library) {
+    const size_t slash = library.find_last_of('/');
+    std::ifstream in((slash == std::string::npos ? std::string() : library.substr(0, slash + 1)) + "manifest.json");
+    if (!in) return std::string();
+    const std::string text((std::istreambuf_iterator<char>(in)), std::istreambuf_iterator<char>());
+    const size_t key = text.find("\"library_sha256\"");
+    if (key == std::string::npos) return std::string();
+    const size_t open = text.find('"', text.find(':', key) + 1);
+    const size_t close = open == std::string::npos ? open : text.find('"', open + 1);
+    return close == std::string::npos ? std::string() : text.substr(open + 1, close - open - 1);
+}
 }  // namespace
+
+std::string library_sha256(const std::string& path) { return sha256_file(path); }
 
 // ---- Native ---------------------------------------------------------------------------------------------------------
 Native::Native(const std::string& library, const ca_geometry& geometry) : g_(geometry) {
+    // the library is the one the build's manifest pins (src/ffn.rs:70-74, src/primitives.rs:75-79: "hash mismatch")
+    const std::string pinned = manifest_sha256(library);
+    if (!pinned.empty() && pinned != sha256_file(library)) throw Error("FFN native library hash mismatch: " + library);
     lib_ = dlopen(library.c_str(), RTLD_NOW | RTLD_LOCAL);
     if (!lib_) throw Error(std::string("load kernel library: ") + dlerror());
     ensure(symbol<int (*)()>(lib_, "ca_ffn_abi")() == 1, "FFN native ABI mismatch");                    // src/ffn.rs:76-77
     ensure(symbol<int32_t (*)()>(lib_, "ca_primitives_abi")() == 1, "primitive entrypoint ABI mismatch"); // src/primitives.rs:104-108
-    const int configured = symbol<int (*)(const ca_geometry*)>(lib_, "ca_ffn_configure")(&g_);
-    if (configured != 0) throw Error("FFN native contract changed: geometry rejected (" + std::to_string(configured) + ")");
-    router_logits_ = symbol<decltype(router_logits_)>(lib_, "ca_router_logits");
-    router_logits_wide_ = symbol<decltype(router_logits_wide_)>(lib_, "ca_router_logits_wide");
-    shared_swiglu_ = symbol<decltype(shared_swiglu_)>(lib_, "ca_shared_swiglu");
-    ffn_add_ = symbol<decltype(ffn_add_)>(lib_, "ca_ffn_add");
+    // the geometry lives in this object's context, not in the library's process state: layers of different geometries
+    // (the reference's target and drafter, src/layer_id.rs:39-47) keep a Native each
+    router_logits_ = symbol<decltype(router_logits_)>(lib_, "ca_router_logits_in");
+    router_logits_wide_ = symbol<decltype(router_logits_wide_)>(lib_, "ca_router_logits_wide_in");
+    shared_swiglu_ = symbol<decltype(shared_swiglu_)>(lib_, "ca_shared_swiglu_in");
+    ffn_add_ = symbol<decltype(ffn_add_)>(lib_, "ca_ffn_add_in");
+    spin_limit_ = symbol<decltype(spin_limit_)>(lib_, "ca_primitives_spin_limit");
     kernel_launch_ = symbol<decltype(kernel_launch_)>(lib_, "ca_kernel_launch");
     close_ = symbol<decltype(close_)>(lib_, "ca_primitives_close");
     launch_ = symbol<decltype(launch_)>(lib_, "ca_primitives_launch");
@@ -37,7 +95,8 @@ Native::Native(const std::string& library, const ca_geometry& geometry) : g_(geo
     local_live_ = symbol<decltype(local_live_)>(lib_, "ca_local_live");
     pack_bf16_ = symbol<decltype(pack_bf16_)>(lib_, "ca_pack_bf16");
     int32_t status = 0;
-    ctx_ = symbol<void* (*)(int32_t*)>(lib_, "ca_primitives_open")(&status);
+    ctx_ = symbol<void* (*)(const ca_geometry*, int32_t*)>(lib_, "ca_primitives_open_geometry")(&g_, &status);
+    if (status == -4) throw Error("FFN native contract changed: geometry rejected (" + std::to_string(status) + ")");
     if (status != 0 || !ctx_) throw Error("initialize primitive library: " + std::to_string(status));   // src/primitives.rs:116-119
 }
 Native::~Native() {
@@ -60,17 +119,18 @@ void Native::codec_pack_bf16(uint64_t input, uint64_t packed, int rows, int k, h
     ensure(pack_bf16_((const void*)input, (uint8_t*)packed, rows, k, s) == 0, "fused packed MoE producer launch");                  // :849-850
 }
 void Native::router_logits(int rows, uint64_t x, uint64_t w, uint64_t out, hipStream_t s) const {
-    ensure(router_logits_(rows, (const void*)x, (const void*)w, (void*)out, s) == 0, "tiny router GPU launch failed");   // src/ffn.rs:352-363
+    ensure(router_logits_(ctx_, rows, (const void*)x, (const void*)w, (void*)out, s) == 0, "tiny router GPU launch failed");   // src/ffn.rs:352-363
 }
 void Native::router_logits_wide(int rows, uint64_t x, uint64_t w, uint64_t out, hipStream_t s) const {
-    ensure(router_logits_wide_(rows, (const void*)x, (const void*)w, (void*)out, s) == 0, "wide router GPU launch failed");
+    ensure(router_logits_wide_(ctx_, rows, (const void*)x, (const void*)w, (void*)out, s) == 0, "wide router GPU launch failed");
 }
 void Native::shared_swiglu(int rows, uint64_t in, uint64_t out, hipStream_t s) const {
-    ensure(shared_swiglu_(rows, (const void*)in, (void*)out, s) == 0, "shared SwiGLU launch failed");                    // src/ffn.rs:1108-1118
+    ensure(shared_swiglu_(ctx_, rows, (const void*)in, (void*)out, s) == 0, "shared SwiGLU launch failed");                    // src/ffn.rs:1108-1118
 }
 void Native::ffn_add(int rows, uint64_t routed, uint64_t shared, uint64_t out, hipStream_t s) const {
-    ensure(ffn_add_(rows, (const void*)routed, (const void*)shared, (void*)out, s) == 0, "FFN shared addition launch failed");   // src/ffn.rs:1071-1082
+    ensure(ffn_add_(ctx_, rows, (const void*)routed, (const void*)shared, (void*)out, s) == 0, "FFN shared addition launch failed");   // src/ffn.rs:1071-1082
 }
+void Native::spin_limit(int limit) const { ensure(spin_limit_(ctx_, limit) == 0, "spin limit rejected"); }
 void Native::launch(const char* name, uint32_t grid_x, uint32_t grid_y, uint32_t block, uint32_t shared, void** args, hipStream_t s) const {
     const uint32_t grid[3] = {grid_x, grid_y, 1}, blk[3] = {block, 1, 1};
     const int status = kernel_launch_(name, grid, blk, shared, args, s);

@@ -21,6 +21,9 @@
 
 namespace tf {
 
+// SHA-256 of a file as lower-case hexadecimal (empty: unreadable): what the build's manifest pins the kernel library with.
+std::string library_sha256(const std::string& path);
+
 // ---- loaded kernel library (src/ffn.rs:46-85 Native::open, src/primitives.rs:66-151 Primitives::open) --------------
 class Native {
 public:
@@ -40,6 +43,8 @@ public:
     int64_t scratch_bytes(int index, int rows) const;
     // five events recorded around the launches of the dynamic entries (null: off)
     void marks(hipEvent_t* events, size_t count = 5) const;      // 5: between the launches; 7: + the FC1 kernel's own begin / end
+    // polls a wait inside the front-end launch may take before the waiter does the work itself (0: no hand-off is waited for)
+    void spin_limit(int limit) const;
     // the wire row "dual_quant_rows_v1" (src/ffn.rs:805-811 RowTransport's functions)
     void codec_encode(uint64_t routed, uint64_t scales, uint64_t shared, uint64_t packed, int rows, int k, hipStream_t s) const;
     void codec_decode(uint64_t packed, uint64_t shared, uint64_t row_scales, uint64_t mma_scales, int rows, int k, hipStream_t s) const;
@@ -49,10 +54,11 @@ private:
     void* lib_ = nullptr;
     void* ctx_ = nullptr;
     ca_geometry g_;
-    int (*router_logits_)(int, const void*, const void*, void*, void*) = nullptr;
-    int (*router_logits_wide_)(int, const void*, const void*, void*, void*) = nullptr;
-    int (*shared_swiglu_)(int, const void*, void*, void*) = nullptr;
-    int (*ffn_add_)(int, const void*, const void*, void*, void*) = nullptr;
+    int (*router_logits_)(void*, int, const void*, const void*, void*, void*) = nullptr;
+    int (*router_logits_wide_)(void*, int, const void*, const void*, void*, void*) = nullptr;
+    int (*shared_swiglu_)(void*, int, const void*, void*, void*) = nullptr;
+    int (*ffn_add_)(void*, int, const void*, const void*, void*, void*) = nullptr;
+    int32_t (*spin_limit_)(void*, int32_t) = nullptr;
     int (*kernel_launch_)(const char*, const uint32_t*, const uint32_t*, uint32_t, void**, void*) = nullptr;
     void (*close_)(void*) = nullptr;
     int32_t (*launch_)(void*, int32_t, const uint64_t*, size_t, const int32_t*, size_t, void*) = nullptr;

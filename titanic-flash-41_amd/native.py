@@ -13,7 +13,8 @@ EXPORTS = ["ca_ffn_abi", "ca_ffn_configure", "ca_ffn_geometry", "ca_router_logit
            "ca_router_logits_wide", "ca_kernel_launch", "ca_kernel_count", "ca_kernel_name", "ca_moe_nibble_permute",
            "ca_primitives_abi", "ca_primitives_open", "ca_primitives_close", "ca_primitives_launch", "ca_primitives_launch2",
            "ca_primitives_entries", "ca_primitives_scratch_bytes", "ca_primitives_marks", "ca_encode", "ca_decode", "ca_local_live",
-           "ca_pack_bf16"]
+           "ca_pack_bf16", "ca_primitives_spin_limit", "ca_primitives_open_geometry", "ca_primitives_geometry", "ca_router_logits_in",
+           "ca_router_logits_wide_in", "ca_shared_swiglu_in", "ca_ffn_add_in"]
 
 
 class Geometry(ctypes.Structure):
@@ -65,6 +66,16 @@ def load():
     lib.ca_pack_bf16.argtypes = [vp, vp, ctypes.c_int, ctypes.c_int, vp]
     lib.ca_primitives_marks.restype = i32
     lib.ca_primitives_marks.argtypes = [vp, ctypes.POINTER(vp), ctypes.c_size_t]
+    lib.ca_primitives_spin_limit.restype = i32
+    lib.ca_primitives_spin_limit.argtypes = [vp, i32]
+    lib.ca_primitives_open_geometry.restype = vp
+    lib.ca_primitives_open_geometry.argtypes = [ctypes.POINTER(Geometry), i32p]
+    lib.ca_primitives_geometry.restype = i32
+    lib.ca_primitives_geometry.argtypes = [vp, ctypes.POINTER(Geometry)]
+    lib.ca_router_logits_in.argtypes = [vp, ctypes.c_int, vp, vp, vp, vp]
+    lib.ca_router_logits_wide_in.argtypes = [vp, ctypes.c_int, vp, vp, vp, vp]
+    lib.ca_shared_swiglu_in.argtypes = [vp, ctypes.c_int, vp, vp, vp]
+    lib.ca_ffn_add_in.argtypes = [vp, ctypes.c_int, vp, vp, vp, vp]
     _lib = lib
     return lib
 
