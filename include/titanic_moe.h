@@ -107,6 +107,19 @@ int64_t ca_primitives_scratch_bytes(void* context, int32_t index, int32_t rows);
  * other than 0, 5 or 7. */
 int32_t ca_primitives_marks(void* context, void* const* events, size_t count);
 
+/* No counterpart in the reference: for callers that cannot allocate device memory (code under HIP graph capture, tight
+ * serving loops, harnesses that forbid it).  The routed experts of entry 0 (`integration.tp_moe.dynamic`: plan, token
+ * quantization, FC1 + SwiGLU, FC2 x routing weight) for at most 64 rows, with every scratch region of that entry (token
+ * codes, plan tables, intermediate) in a static device array of the library instead of a caller's arena; the caller passes only
+ * inputs (token rows BF16 [rows][H], top-k ids and weights [rows][K], the prepared expert weights and scales) and the output
+ * (route outputs BF16 [rows][K][H], what entry 0 writes to its `scatter_ptr`).  Same kernels and bits as entry 0.  The array
+ * (ca_moe_dynamic_static_capacity() bytes, 16 MiB) exists once a device and keeps the last call's contents; calls that
+ * overlap on one device race.  Nothing is allocated, freed or synchronized.  0; -1 null / rows < 1 / a context opened on
+ * another device than the current one; -5 more than 64 rows or a geometry whose regions exceed the array; -4; or a hipError_t. */
+int32_t ca_moe_dynamic_static(void* context, const void* input, const int32_t* topk_ids, const float* topk_weights, const void* w13,
+                              const void* s13, const void* w2, const void* s2, void* route_output, int32_t rows, void* stream);
+int64_t ca_moe_dynamic_static_capacity(void);
+
 /* No counterpart in the reference (its front-end has no waits inside a launch).  The front-end launch of entries 1 and 9 hands
  * data from some of its workgroups to others; every such wait is bounded by `limit` polls (default 262,144), after which the
  * waiter does the work it waited for itself and marks the `sync_ptr` region: later launches then take that path at once

@@ -12,7 +12,16 @@
 #include <cstdlib>
 #include <cstring>
 
+// Scratch of ca_moe_dynamic_static: one array a device, held from the library's load to the end of the process.  In host code
+// the array's name stands for the symbol, not for device memory: its address on the current device is looked up once a device
+// (ca_primitives_open*), and only that address is ever handed to kernels.
+#define TF_STATIC_SCRATCH_BYTES (16u << 20)
+static __device__ __align__(256) unsigned char scratch[TF_STATIC_SCRATCH_BYTES];
+
 namespace {
+
+constexpr int kMaxDevices = 64;
+void* g_static_scratch[kMaxDevices] = {};
 
 ca_geometry g_geometry = {5120, 384, 6, 576, 576, 1, 1.5f, 32, 32, 32, 129264, 10.f};   // src/ffn.rs:65-66, 245-258
 
@@ -39,7 +48,37 @@ struct Context {
     bool marking;
     bool kernel_marks;     // marks[5], marks[6]: begin and end of the FC1 + SwiGLU kernel itself
     int spin_limit;        // polls a wait inside the front-end launch may take before the waiter does the work itself
+    int device;            // the device the context was opened on
+    uint8_t* static_scratch;   // that device's copy of `scratch`
 };
+
+// The regions of entry 0 / 1's scratch arena, in the runtime contract's order, each aligned to 256 bytes: token codes and
+// scales (routed flavour, shared flavour), intermediate (BF16, codes, scales), tile tables, row maps, route outputs,
+// wide-plan scratch, the front-end's sync region.
+struct DynLayout {
+    long long packed, scales, packed_min, scales_min, inter, inter_codes, inter_scales, task_expert, task_valid, tile_base, token_map,
+        token_weights, scatter, plan_scratch, sync, total;
+    int tile_m;
+    long long tiles;
+};
+DynLayout dyn_layout(const ca_geometry& g, int rows) {
+    DynLayout l{};
+    const long long pairs = (long long)rows * g.topk;
+    l.tile_m = rows <= TF_STREAM_MAX_ROWS ? 16 : TF_GEMM_TILE_M;
+    l.tiles = (pairs + l.tile_m - 1) / l.tile_m - 1 + (g.experts < pairs ? g.experts : pairs);
+    const long long padded = l.tiles * l.tile_m, H = g.hidden, I = g.intermediate, B = g.act_block;
+    long long at = 0;
+    auto add = [&](long long n) { const long long here = at; at += (n + 255) / 256 * 256; return here; };
+    l.packed = add(rows * H); l.scales = add(rows * H / B); l.packed_min = add(rows * H); l.scales_min = add(rows * H / B);
+    l.inter = add(padded * I * 2); l.inter_codes = add(padded * I); l.inter_scales = add(padded * I / B);
+    l.task_expert = add(l.tiles * 4); l.task_valid = add(l.tiles * 4); l.tile_base = add((g.experts + 1) * 4ll);
+    l.token_map = add(padded * 4); l.token_weights = add(padded * 4);
+    l.scatter = add(pairs * H * 2);
+    l.plan_scratch = add(((pairs + 63) / 64 * g.experts + pairs) * 4);
+    l.sync = add(TF_SYNC_BYTES);
+    l.total = at;
+    return l;
+}
 
 // Records mark `i` on the launch stream when the caller asked for marks (never while a stream is captured: the caller's duty).
 void mark(const Context& c, int i, hipStream_t s) {
@@ -505,8 +544,16 @@ void* ca_primitives_open_geometry(const ca_geometry* geometry, int32_t* status) 
     hipError_t e = hipGetDevice(&device);
     if (e == hipSuccess) e = hipDeviceGetAttribute(&cus, hipDeviceAttributeMultiprocessorCount, device);
     if (e != hipSuccess) { *status = (int32_t)e; return nullptr; }
+    if (device < 0 || device >= kMaxDevices) { *status = -1; return nullptr; }
+    if (!g_static_scratch[device]) {          // this device's copy of the static scratch array: looked up once, with the device current
+        void* at = nullptr;
+        e = hipGetSymbolAddress(&at, HIP_SYMBOL(scratch));
+        if (e != hipSuccess || !at) { *status = e != hipSuccess ? (int32_t)e : -1; return nullptr; }
+        g_static_scratch[device] = at;
+    }
     Context* c = new Context{};
     c->g = *geometry; c->cus = cus; c->stream_wgs = cus * 2; c->spin_limit = 1 << 18;
+    c->device = device; c->static_scratch = (uint8_t*)g_static_scratch[device];
     return c;
 }
 void* ca_primitives_open(int32_t* status) { return ca_primitives_open_geometry(&g_geometry, status); }
@@ -575,22 +622,31 @@ int32_t ca_primitives_launch2(void* context, int32_t index, const uint64_t* word
 }
 int64_t ca_primitives_scratch_bytes(void* context, int32_t index, int32_t rows) {
     if (!context || rows < 1 || (index != 0 && index != 1)) return -1;
-    const ca_geometry& g = ((const Context*)context)->g;
-    const long long pairs = (long long)rows * g.topk;
-    const int tile_m = rows <= TF_STREAM_MAX_ROWS ? 16 : TF_GEMM_TILE_M;
-    const long long tiles = (pairs + tile_m - 1) / tile_m - 1 + (g.experts < pairs ? g.experts : pairs), padded = tiles * tile_m;
-    long long bytes = 0;
-    auto add = [&](long long n) { bytes += (n + 255) / 256 * 256; };
-    const long long H = g.hidden, I = g.intermediate, B = g.act_block;
-    // the regions of the runtime contract, in its order, each aligned to 256 bytes: token codes and scales (routed flavour,
-    // shared flavour), intermediate (BF16, codes, scales), tile tables, row maps, route outputs, wide-plan scratch, the front-end's sync region
-    add(rows * H); add(rows * H / B); add(rows * H); add(rows * H / B);
-    add(padded * I * 2); add(padded * I); add(padded * I / B);
-    add(tiles * 4); add(tiles * 4); add((g.experts + 1) * 4ll); add(padded * 4); add(padded * 4);
-    add(pairs * H * 2);
-    add(((pairs + 63) / 64 * g.experts + pairs) * 4);
-    add(TF_SYNC_BYTES);
-    return bytes;
+    return dyn_layout(((const Context*)context)->g, rows).total;
+}
+int64_t ca_moe_dynamic_static_capacity(void) { return (int64_t)TF_STATIC_SCRATCH_BYTES; }
+int32_t ca_moe_dynamic_static(void* context, const void* input, const int32_t* topk_ids, const float* topk_weights, const void* w13,
+                              const void* s13, const void* w2, const void* s2, void* route_output, int32_t rows, void* stream) {
+    if (!context || !input || !topk_ids || !topk_weights || !w13 || !s13 || !w2 || !s2 || !route_output || rows < 1) return -1;
+    const Context& c = *(const Context*)context;
+    if (rows > TF_STREAM_MAX_ROWS) return -5;                  // few-row owners only: the many-row arena is far past the static array
+    const DynLayout l = dyn_layout(c.g, rows);
+    // everything but the route outputs, which the caller passes, lies in the static array
+    const long long needed = l.scatter;
+    if (needed > (long long)TF_STATIC_SCRATCH_BYTES || l.tiles > TF_LDS_TILES) return -5;
+    int device = -1;
+    if (hipGetDevice(&device) != hipSuccess || device != c.device || !c.static_scratch) return -1;      // the array of the context's device
+    const uint64_t base = (uint64_t)c.static_scratch;
+    uint64_t p[P_DYN_COUNT] = {};
+    p[P_A] = (uint64_t)input; p[P_IDS] = (uint64_t)topk_ids; p[P_WEIGHTS] = (uint64_t)topk_weights;
+    p[P_PACKED] = base + l.packed; p[P_SCALES] = base + l.scales; p[P_PACKED_MIN] = 0; p[P_SCALES_MIN] = 0;
+    p[P_INTER] = base + l.inter; p[P_INTER_CODES] = base + l.inter_codes; p[P_INTER_SCALES] = base + l.inter_scales;
+    p[P_TASK_EXPERT] = base + l.task_expert; p[P_TASK_VALID] = base + l.task_valid; p[P_TILE_BASE] = base + l.tile_base;
+    p[P_TOKEN_MAP] = base + l.token_map; p[P_TOKEN_WEIGHTS] = base + l.token_weights;
+    p[P_W13] = (uint64_t)w13; p[P_S13] = (uint64_t)s13; p[P_W2] = (uint64_t)w2; p[P_S2] = (uint64_t)s2;
+    p[P_SCATTER] = (uint64_t)route_output; p[P_PLAN_SCRATCH] = 0;
+    const int32_t sc[S_DYN_COUNT] = {rows, rows, (int32_t)(l.tiles * l.tile_m), (int32_t)l.tiles, l.tile_m, 1};
+    return launch_dynamic(c, false, p, sc, (hipStream_t)stream);
 }
 
 }  // extern "C"

@@ -14,7 +14,7 @@ EXPORTS = ["ca_ffn_abi", "ca_ffn_configure", "ca_ffn_geometry", "ca_router_logit
            "ca_primitives_abi", "ca_primitives_open", "ca_primitives_close", "ca_primitives_launch", "ca_primitives_launch2",
            "ca_primitives_entries", "ca_primitives_scratch_bytes", "ca_primitives_marks", "ca_encode", "ca_decode", "ca_local_live",
            "ca_pack_bf16", "ca_primitives_spin_limit", "ca_primitives_open_geometry", "ca_primitives_geometry", "ca_router_logits_in",
-           "ca_router_logits_wide_in", "ca_shared_swiglu_in", "ca_ffn_add_in"]
+           "ca_router_logits_wide_in", "ca_shared_swiglu_in", "ca_ffn_add_in", "ca_moe_dynamic_static", "ca_moe_dynamic_static_capacity"]
 
 
 class Geometry(ctypes.Structure):
@@ -72,6 +72,9 @@ def load():
     lib.ca_primitives_open_geometry.argtypes = [ctypes.POINTER(Geometry), i32p]
     lib.ca_primitives_geometry.restype = i32
     lib.ca_primitives_geometry.argtypes = [vp, ctypes.POINTER(Geometry)]
+    lib.ca_moe_dynamic_static.restype = i32
+    lib.ca_moe_dynamic_static.argtypes = [vp, vp, vp, vp, vp, vp, vp, vp, vp, i32, vp]
+    lib.ca_moe_dynamic_static_capacity.restype = ctypes.c_int64
     lib.ca_router_logits_in.argtypes = [vp, ctypes.c_int, vp, vp, vp, vp]
     lib.ca_router_logits_wide_in.argtypes = [vp, ctypes.c_int, vp, vp, vp, vp]
     lib.ca_shared_swiglu_in.argtypes = [vp, ctypes.c_int, vp, vp, vp]
