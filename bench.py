@@ -6,15 +6,25 @@
 A step is one pass of the whole layer (gate product, top-k + plan + token quantization, routed FC1 + SwiGLU, FC2, shared
 expert, ordered sum + shared addition) over one batch of synthetic token rows that is already resident in HBM, replayed
 as a captured HIP graph as the reference replays its layer (src/probe.rs:1527-1542).  Sixteen distinct input batches
-are cycled so every step routes to other experts and streams their weights from HBM, not from the last step's cache.
+(two at many rows) are cycled so every step routes to other experts and streams their weights from HBM, not from the last
+step's cache.  A graph holds one pass over each batch, so --steps and --warmup are rounded up to whole replays; the line
+says so and carries the numbers that ran.
 
-Prints one JSON line: whole-layer tokens/s, the roofline of the dominant kernel (FC1 + SwiGLU of the routed experts;
-algorithmic bytes over its average duration, measured with two HIP events that take the kernel's start and completion
-on its launch stream; many rows: events recorded around the launch), and the CPU baseline (the C oracle, a port of the reference semantics: the
-reference has no CPU path) timed on a bounded sample of the same workload.
+Prints ONE JSON line.  Without --config its top level is the decode step (c2, the configuration the metric is quoted on):
+whole-layer tokens/s, the roofline of the dominant kernel (FC1 + SwiGLU of the routed experts; algorithmic bytes over its
+average duration, measured with two HIP events that take the kernel's start and completion on its launch stream), and the
+CPU baseline (the C oracle, a port of the reference semantics: the reference has no CPU path) timed on a bounded sample of
+the same workload, with all threads and with one.  `configs` then holds the same measurement of the speculative-verify step
+(c3) and the two prefill chunks (c4, c5: bound by the matrix units, flops over the FC1 launch's duration between events
+recorded around it).  With --config only that configuration runs and is the top level.
+
+`roofline.traffic` is the measured HBM bytes a launch of the dominant kernel: the ratio of measured to algorithmic bytes
+that the committed counter file holds for the same workload (profiles/counters.json, written by
+`python -m titanic-flash-41_amd.counters`; its library hash and commit are copied into the line) times the algorithmic
+bytes of this run's launches; null where the file has no run of the workload.
 
 --copy-probe appends four plain device copies of 256 MiB after the timed region: a counter run (rocprofv3 --pmc
-FETCH_SIZE / WRITE_SIZE) then holds a kernel of known traffic to scale the counters by.
+FETCH_SIZE / WRITE_SIZE) of this program then holds a kernel of known traffic to scale the counters by.
 """
 import argparse
 import importlib
@@ -45,14 +55,8 @@ CONFIGS = {
     "r4096": dict(rows=4096, hidden=5120, experts=384, topk=6, inter=2304, shared=2304,
                   workload="the reference's layer, prefill chunk of 4096 tokens; H 5120, E 384, top-6, I 2304, 1 shared expert (I 2304)"),
 }
+HEADLINE, OTHERS = "c2", ["c3", "c4", "c5"]
 MFMA_FP8_PEAK_TFLOPS, MFMA_FP4_PEAK_TFLOPS = 5000.0, 10100.0
-# Measured HBM traffic of the dominant kernel over its algorithmic bytes, from the counter runs summarized under profiles/
-# (rocprofv3 --pmc FETCH_SIZE, then WRITE_SIZE, on tf_layer_probe: the same geometry, rows and schedule with random operands;
-# each counter scaled by its reading for a 256 MiB copy kernel).  The line's `traffic` is this ratio times the algorithmic
-# bytes of this run's launches; None where no counter run exists for the configuration.
-TRAFFIC_OVER_ALGORITHMIC = {"c2": 1.0003}
-# Many rows: HBM bytes a launch of the routed FC1 kernel, measured the same way at the same number of rows.
-WIDE_TRAFFIC_BYTES = {"c4": 3.24e9, "c5": 6.92e9}
 
 
 def make_inputs(synth, name, cfg, device, batches=BATCHES):
@@ -69,26 +73,48 @@ def make_inputs(synth, name, cfg, device, batches=BATCHES):
     return xs
 
 
-def cpu_baseline(pkg, g, ops, xs, taps_ids, budget_s=20.0):
-    """Times the C oracle (staged, active experts only) on host cores for a bounded number of steps."""
+def cpu_model():
+    try:
+        with open("/proc/cpuinfo") as f:
+            for line in f:
+                if line.lower().startswith("model name"):
+                    return line.split(":", 1)[1].strip()
+    except OSError:
+        pass
+    return "unknown"
+
+
+def cpu_baseline(pkg, g, ops, xs, taps_ids, budget_s=15.0, single_budget_s=8.0):
+    """Times the C oracle (staged, active experts only) on host cores for a bounded number of steps: with every thread the
+    process may use (at most 16), then with one thread (the scalar figure)."""
     sys.path.insert(0, os.path.join(ROOT, "tests"))
     import oracle
     import helpers
-    threads = len(os.sched_getaffinity(0)) if hasattr(os, "sched_getaffinity") else (os.cpu_count() or 1)
-    threads = max(1, min(threads, 16))
-    oracle.set_threads(threads)
+    allowed = len(os.sched_getaffinity(0)) if hasattr(os, "sched_getaffinity") else (os.cpu_count() or 1)
+    threads = max(1, min(allowed, 16))
     rows = xs[0].shape[0]
-    done, spent = 0, 0.0
-    while done < 4 * len(xs) and (done == 0 or spent + spent / done < budget_s):
-        x = xs[done % len(xs)]
-        # gather the operands the step touches outside the timed region (the oracle reads host memory)
-        small_ops = _HostSubset(ops, taps_ids[done % len(xs)], g)
-        t0 = time.perf_counter()
-        helpers.oracle_layer(g, small_ops, x.cpu())
-        spent += time.perf_counter() - t0
-        done += 1
-    return {"value": rows * done / spent, "unit": "tokens/s", "cores": threads, "kind": "port",
-            "sample": "%d steps of this workload (%d rows each), C oracle with %d OpenMP threads, %.1f s" % (done, rows, threads, spent)}
+
+    def timed(n_threads, budget):
+        oracle.set_threads(n_threads)
+        done, spent = 0, 0.0
+        while done < 4 * len(xs) and (done == 0 or spent + spent / done < budget):
+            x = xs[done % len(xs)]
+            # gather the operands the step touches outside the timed region (the oracle reads host memory)
+            small_ops = _HostSubset(ops, taps_ids[done % len(xs)], g)
+            t0 = time.perf_counter()
+            helpers.oracle_layer(g, small_ops, x.cpu())
+            spent += time.perf_counter() - t0
+            done += 1
+        return done, spent
+
+    done, spent = timed(threads, budget_s)
+    done1, spent1 = timed(1, single_budget_s)
+    oracle.set_threads(threads)
+    return {"value": rows * done / spent, "unit": "tokens/s", "cores": threads, "threads": threads, "kind": "port",
+            "nproc": os.cpu_count(), "cpus_allowed": allowed, "cpu_model": cpu_model(),
+            "sample": "%d steps of this workload (%d rows each), C oracle with %d OpenMP threads, %.1f s" % (done, rows, threads, spent),
+            "single_thread": {"value": rows * done1 / spent1, "unit": "tokens/s", "cores": 1,
+                              "sample": "%d steps of this workload, the same C oracle with one thread, %.1f s" % (done1, spent1)}}
 
 
 class _HostSubset:
@@ -119,49 +145,36 @@ class _Sparse:
         return self.data[torch.as_tensor([self.index[int(e)] for e in ids], dtype=torch.long)]
 
 
-def main():
-    ap = argparse.ArgumentParser()
-    ap.add_argument("--gpus", type=int, default=1)
-    ap.add_argument("--steps", type=int, default=2000)
-    ap.add_argument("--warmup", type=int, default=200)
-    ap.add_argument("--config", default="c2", choices=sorted(CONFIGS))
-    ap.add_argument("--numerics", default=None, choices=["benchmark", "reference"],
-                    help="benchmark: sigmoid scores, renormalised, 128-wide activation blocks, 128 x 128 shared weight blocks (the headline); "
-                         "reference: the reference's own numerics (sqrt-softplus x 1.5, 32-wide blocks, 32 x 32, image-token bias)")
-    ap.add_argument("--no-cpu-baseline", action="store_true")
-    ap.add_argument("--overlap", type=int, default=None, choices=[0, 1],
-                    help="many rows: the shared expert on a second stream beside the routed experts (the reference's dual-stream schedule, "
-                         "src/ffn.rs:1000-1040) or after them on the same stream; default: the layer's own choice")
-    ap.add_argument("--copy-probe", action="store_true", help="append four 256 MiB device copies (counter calibration)")
-    ap.add_argument("--profile-steps", type=int, default=64, help="eager passes with per-kernel HIP events for the roofline")
-    args = ap.parse_args()
-    if args.gpus != 1:
-        print("bench.py measures one GPU: the layer runs on a single MI355X (no sharding, no collectives); --gpus %d is not supported" % args.gpus,
-              file=sys.stderr)
-        sys.exit(2)
+def geometry_of(native, cfg, numerics):
+    if numerics == "benchmark":
+        return native.Geometry(cfg["hidden"], cfg["experts"], cfg["topk"], cfg["inter"], cfg["shared"], 0, 1.0, 128, 128, 128, -1, 10.0)
+    return native.Geometry(cfg["hidden"], cfg["experts"], cfg["topk"], cfg["inter"], cfg["shared"], 1, 1.5, 32, 32, 32, 129264, 10.0)
+
+
+def measure(pkg, name, numerics, steps, warmup, profile_steps, overlap, operands, counter_file, with_cpu):
+    """One configuration: the whole-layer rate by graph replay, the dominant kernel's duration by HIP events, the
+    algorithmic bytes and flops of the launches that ran.  Returns the record and what the CPU baseline needs."""
+    import copy
     import numpy as np
     import torch
-    pkg = importlib.import_module("titanic-flash-41_amd")
-    native, synth, host = pkg.native, pkg.synth, pkg.host
-    cfg = CONFIGS[args.config]
-    if args.numerics is None:
-        args.numerics = "reference" if args.config.startswith("r") else "benchmark"
-    if args.numerics == "benchmark":
-        g = native.Geometry(cfg["hidden"], cfg["experts"], cfg["topk"], cfg["inter"], cfg["shared"], 0, 1.0, 128, 128, 128, -1, 10.0)
-    else:
-        g = native.Geometry(cfg["hidden"], cfg["experts"], cfg["topk"], cfg["inter"], cfg["shared"], 1, 1.5, 32, 32, 32, 129264, 10.0)
+    native, synth, host, counters = pkg.native, pkg.synth, pkg.host, pkg.counters
+    cfg = CONFIGS[name]
+    g = geometry_of(native, cfg, numerics)
     B, BN, BK = g.act_block, g.shared_bn, g.shared_bk
-    torch.cuda.set_device(0)
     t0 = time.time()
     wide = cfg["rows"] > 64
     batches = 2 if wide else BATCHES
     if wide:
-        args.steps, args.warmup, args.profile_steps = min(args.steps, 200), min(args.warmup, 20), min(args.profile_steps, 8)
-    ops = synth.LayerOperands(g, args.config, device="cuda")
-    if args.config == "c5":      # expert popularity ~ rank^-1.1: the busiest experts take more than ten times the mean load
+        steps, warmup, profile_steps = min(steps, 200), min(warmup, 20), min(profile_steps, 8)
+    key = (cfg["hidden"], cfg["experts"], cfg["inter"], cfg["shared"], numerics)
+    if key not in operands:     # the benchmark configurations share one geometry: one set of synthetic weights serves them all
+        operands[key] = synth.LayerOperands(g, "bench/%d/%d" % (cfg["hidden"], cfg["experts"]), device="cuda")
+    ops = operands[key]
+    if name == "c5":      # expert popularity ~ rank^-1.1: the busiest experts take more than ten times the mean load
+        ops = copy.copy(ops)
         ops.bias = synth.zipf_bias(g.experts, 1.1, 0.06, device="cuda")
-    xs = make_inputs(synth, args.config, cfg, "cuda", batches)
-    layer = host.Layer(g, ops, cfg["rows"]) if args.overlap is None else host.Layer(g, ops, cfg["rows"], overlap=bool(args.overlap))
+    xs = make_inputs(synth, name, cfg, "cuda", batches)
+    layer = host.Layer(g, ops, cfg["rows"]) if overlap is None else host.Layer(g, ops, cfg["rows"], overlap=bool(overlap))
     layer.set_tokens()
     layer.keep_intermediate(False)      # many rows: FC2 reads the FP8 codes; the BF16 copy is a tap the tests ask for
     setup_s = time.time() - t0
@@ -169,12 +182,13 @@ def main():
     # per-kernel durations (HIP events on the launch stream) and the routing of every batch
     ids_per_batch, parts = [], np.zeros(7)
     tiles_per_batch = []
+    fc1_kernel = 0.0
     if wide:
         # many rows: one eager pass at a time, events around each part (router, front-end, FC1, FC2, shared expert, sum)
         for x in xs:                      # warm every batch once
             layer.profile_step(x)
         passes = 0
-        for i in range(args.profile_steps):
+        for i in range(profile_steps):
             x = xs[i % batches]
             parts += np.array(layer.profile_step(x))
             passes += 1
@@ -190,15 +204,22 @@ def main():
             ids_per_batch.append(layer.tap("ids").reshape(cfg["rows"], cfg["topk"]).copy())
             tiles_per_batch.append(int(layer.tap("tile_base")[-1]))
         layer.profile_marks(xs, batches)
-        front, fc1, fc2, total, whole, _ = layer.profile_marks(xs, max(args.profile_steps, batches) * 4)
-        fc1_kernel = layer.profile_marks(xs, max(args.profile_steps, batches) * 4, exact=True)[5]
+        front, fc1, fc2, total, whole, _ = layer.profile_marks(xs, max(profile_steps, batches) * 4)
+        fc1_kernel = layer.profile_marks(xs, max(profile_steps, batches) * 4, exact=True)[5]
         parts = np.array([0.0, front, fc1, fc2, 0.0, total, whole])
     H, I, S, E, K, rows = cfg["hidden"], cfg["inter"], cfg["shared"], cfg["experts"], cfg["topk"], cfg["rows"]
-    distinct = float(np.mean([len(set(ids.ravel().tolist())) for ids in ids_per_batch]))
+    distinct = float(np.mean([len(set(ids[ids >= 0].ravel().tolist())) for ids in ids_per_batch]))
     tiles = float(np.mean(tiles_per_batch))
-    # algorithmic bytes: every streamed tile of FC1 reads one expert's up + gate weights and scales once
-    fc1_bytes = tiles * (2 * I * H // 2 + 2 * I * H // 32) + rows * (H + H // B) + rows * K * I * 2
-    fc2_bytes = tiles * (H * I // 2 + H * I // 32) + rows * K * I * 2 + rows * K * H * 2
+    routes = float(np.mean([(ids >= 0).sum() for ids in ids_per_batch]))
+    if wide:
+        # grouped GEMM: every expert with rows streams its weights and scales once, every route reads its token's codes and
+        # scales once and writes FP8 codes and block scales of the intermediate (FC2: reads those, writes BF16 route outputs)
+        fc1_bytes = distinct * (2 * I * H // 2 + 2 * I * H // 32) + routes * (H + H / B) + routes * (I + I / B)
+        fc2_bytes = distinct * (H * I // 2 + H * I // 32) + routes * (I + I / B) + routes * H * 2
+    else:
+        # streaming launches: every 16-row tile reads one expert's up + gate weights and scales once
+        fc1_bytes = tiles * (2 * I * H // 2 + 2 * I * H // 32) + rows * (H + H // B) + rows * K * I * 2
+        fc2_bytes = tiles * (H * I // 2 + H * I // 32) + rows * K * I * 2 + rows * K * H * 2
     shared_bytes = 3 * H * S + rows * (H + 2 * S * 2 + S * 2 + H * 2)
     router_bytes = 2 * E * H + rows * H * 2
     step_bytes = fc1_bytes + fc2_bytes + shared_bytes + router_bytes + rows * (K + 2) * H * 2
@@ -214,59 +235,116 @@ def main():
     # between the marks before and after it also holds the gap to the previous launch, about 3 us)
     fc1_kernel_ms = float(fc1_kernel) if not wide and fc1_kernel > 0 else fc1_ms
     achieved = phase1_bytes / (fc1_kernel_ms * 1e-3) / 1e9
-    routes = float(np.mean([(ids >= 0).sum() for ids in ids_per_batch]))
     fc1_flops, fc2_flops = routes * 2 * (2 * I) * H, routes * 2 * H * I
     step_flops = fc1_flops + fc2_flops + rows * (6 * H * S + 2 * H * E)
     max_load = float(np.mean([np.bincount(ids[ids >= 0].ravel(), minlength=E).max() for ids in ids_per_batch]))
 
-    # whole-layer throughput: one graph holds a pass over each of the sixteen batches (as the reference's graph holds its forty
+    # whole-layer throughput: one graph holds a pass over each of the input batches (as the reference's graph holds its forty
     # layers' passes); a step is one pass, so steps and warmup are rounded up to whole replays
+    asked = (steps, warmup)
     graph = layer.capture(xs)
     torch.cuda.synchronize()
-    replays, warm = -(-args.steps // batches), -(-args.warmup // batches)
-    args.steps, args.warmup = replays * batches, warm * batches
+    replays, warm = -(-steps // batches), -(-warmup // batches)
+    steps, warmup = replays * batches, warm * batches
     ms = layer.time([graph], warm, replays)
     torch.cuda.synchronize()
-    ms_per_step = ms / args.steps
+    ms_per_step = ms / steps
     value = rows / (ms_per_step * 1e-3)
 
-    line = {
-        "metric": "MoE-layer tokens/s", "value": value, "unit": "tokens/s", "n_gpus": 1, "steps": args.steps, "warmup": args.warmup,
-        "ms_per_step": ms_per_step, "higher_is_better": True, "scaling": "weak", "vs_baseline": None,
-        "dtype": "fp4 (e2m1 weights, ue8m0 scales) x fp8 (e4m3 activations), f32 accumulate",
-        "data": "synthetic", "config": {"workload": args.config + ": " + cfg["workload"], "numerics": ("sigmoid top-k renormalised, 128-wide activation blocks" if args.numerics == "benchmark" else
-                                                     "reference numerics: sqrt-softplus scores x 1.5, 32-wide activation blocks, 32 x 32 shared weight blocks"),
-                                        "input_batches": batches, "distinct_experts_per_step": distinct, "schedule": "HIP graph replay (%d passes a graph)" % batches},
-        "roofline": ({"bound": "mfma", "kernel": "tf_gemm<fp4, FC1> (routed FC1 + SwiGLU + FP8 requantization)",
-                      "achieved": fc1_flops / (fc1_ms * 1e-3) / 1e12, "peak": MFMA_FP8_PEAK_TFLOPS, "unit": "TFLOP/s",
-                      "frac": fc1_flops / (fc1_ms * 1e-3) / 1e12 / MFMA_FP8_PEAK_TFLOPS,
-                      "frac_of_fp4_peak": fc1_flops / (fc1_ms * 1e-3) / 1e12 / MFMA_FP4_PEAK_TFLOPS,
-                      "operands": "A = FP8 E4M3 activations, B = FP4 E2M1 weights: issues at the FP8 rate (measured)",
-                      "traffic": WIDE_TRAFFIC_BYTES.get(args.config) if args.numerics == "benchmark" else None, "traffic_source": "rocprofv3 counters on tf_layer_probe at the same rows (profiles/)",
-                      "flops_per_launch": fc1_flops, "avg_launch_ms": fc1_ms, "weight_gbs": fc1_bytes / (fc1_ms * 1e-3) / 1e9} if wide else
-                     {"bound": "hbm", "kernel": ("tf_phase1_stream (FC1 + SwiGLU of the routed experts; the shared expert's first projection streams in the front-end launch)"
-                                                  if early_shared else "tf_phase1_stream (FC1 + SwiGLU of the routed experts and the shared expert in one launch)"),
-                      "achieved": achieved, "peak": HBM_PEAK_GBS, "unit": "GB/s", "frac": achieved / HBM_PEAK_GBS,
-                      "traffic": (TRAFFIC_OVER_ALGORITHMIC[args.config] * phase1_bytes
-                                  if args.config in TRAFFIC_OVER_ALGORITHMIC and args.numerics == "benchmark" else None),
-                      "bytes_per_launch": phase1_bytes, "avg_launch_ms": fc1_kernel_ms, "launch_to_launch_ms": fc1_ms,
-                      "timing": "HIP events bound to the kernel's start and completion (hipExtLaunchKernelGGL) on its launch stream, eager passes of the layer's schedule"}),
+    ratio = counters.traffic_ratio(counter_file, name) if numerics == "benchmark" else None
+    traffic_source = None
+    if ratio is not None:
+        traffic_source = {"file": "profiles/counters.json", "git": counter_file.get("git"), "library_sha256": counter_file.get("library_sha256"),
+                          "same_library_as_this_run": counter_file.get("library_sha256") == native.library_sha256(),
+                          "traffic_over_algorithmic": ratio}
+    if wide:
+        tflops = fc1_flops / (fc1_ms * 1e-3) / 1e12
+        roofline = {"bound": "mfma", "kernel": "tf_grouped_gemm<FC1> (routed FC1 + SwiGLU + FP8 requantization)",
+                    "achieved": tflops, "peak": MFMA_FP8_PEAK_TFLOPS, "unit": "TFLOP/s", "frac": tflops / MFMA_FP8_PEAK_TFLOPS,
+                    "frac_of_fp4_peak": tflops / MFMA_FP4_PEAK_TFLOPS,
+                    "operands": "A = FP8 E4M3 activations, B = FP4 E2M1 weights: issues at the FP8 rate (measured)",
+                    "traffic": ratio * fc1_bytes if ratio is not None else None, "traffic_source": traffic_source,
+                    "bytes_or_flops_per_launch": fc1_flops, "per_launch_unit": "flop", "algorithmic_bytes_per_launch": fc1_bytes,
+                    "avg_launch_ms": fc1_ms, "weight_gbs": fc1_bytes / (fc1_ms * 1e-3) / 1e9,
+                    "timing": "HIP events recorded around the launch on its stream, eager passes of the layer's schedule"}
+    else:
+        roofline = {"bound": "hbm", "kernel": ("tf_phase1_stream (FC1 + SwiGLU of the routed experts; the shared expert's first projection streams in the front-end launch)"
+                                               if early_shared else "tf_phase1_stream (FC1 + SwiGLU of the routed experts and the shared expert in one launch)"),
+                    "achieved": achieved, "peak": HBM_PEAK_GBS, "unit": "GB/s", "frac": achieved / HBM_PEAK_GBS,
+                    "traffic": ratio * phase1_bytes if ratio is not None else None, "traffic_source": traffic_source,
+                    "bytes_or_flops_per_launch": phase1_bytes, "per_launch_unit": "byte", "avg_launch_ms": fc1_kernel_ms, "launch_to_launch_ms": fc1_ms,
+                    "timing": "HIP events bound to the kernel's start and completion (hipExtLaunchKernelGGL) on its launch stream, eager passes of the layer's schedule"}
+    record = {
+        "value": value, "unit": "tokens/s", "steps": steps, "warmup": warmup, "ms_per_step": ms_per_step,
+        "steps_note": "asked for %d steps after %d warm-up steps; rounded up to whole replays of the %d-pass graph" % (asked[0], asked[1], batches),
+        "config": {"workload": name + ": " + cfg["workload"],
+                   "numerics": ("sigmoid top-k renormalised, 128-wide activation blocks" if numerics == "benchmark" else
+                                "reference numerics: sqrt-softplus scores x 1.5, 32-wide activation blocks, 32 x 32 shared weight blocks"),
+                   "input_batches": batches, "distinct_experts_per_step": distinct, "schedule": "HIP graph replay (%d passes a graph)" % batches},
+        "roofline": roofline,
         "step_tflops": step_flops / (ms_per_step * 1e-3) / 1e12, "busiest_expert_rows": max_load, "phys_tiles": tiles,
         "step_bytes": step_bytes, "step_gbs": step_bytes / (ms_per_step * 1e-3) / 1e9, "step_hbm_frac": step_bytes / (ms_per_step * 1e-3) / 1e9 / HBM_PEAK_GBS,
         "kernel_ms": {"router": float(parts[0]), "front_end": float(parts[1]), "fc1_swiglu": fc1_ms, "fc2": float(parts[3]),
                       "shared_expert": float(parts[4]), "sum_shared": float(parts[5]), "eager_pass": float(parts[6])},
         "kernel_gbs": {"fc2": phase2_bytes / (float(parts[3]) * 1e-3) / 1e9},
+        "kernel_tflops": {"fc2": fc2_flops / (float(parts[3]) * 1e-3) / 1e12},
         "setup_s": setup_s,
     }
-    if not args.no_cpu_baseline:
-        line["cpu_baseline"] = cpu_baseline(pkg, g, ops, xs, ids_per_batch)
+    if with_cpu:
+        record["cpu_baseline"] = cpu_baseline(pkg, g, ops, xs, ids_per_batch)
+    layer.close()
+    del layer, xs
+    torch.cuda.empty_cache()
+    return record
+
+
+def main():
+    ap = argparse.ArgumentParser()
+    ap.add_argument("--gpus", type=int, default=1)
+    ap.add_argument("--steps", type=int, default=2000)
+    ap.add_argument("--warmup", type=int, default=200)
+    ap.add_argument("--config", default=None, choices=sorted(CONFIGS),
+                    help="measure only this configuration; default: c2 as the headline and c3, c4, c5 under `configs`")
+    ap.add_argument("--numerics", default=None, choices=["benchmark", "reference"],
+                    help="benchmark: sigmoid scores, renormalised, 128-wide activation blocks, 128 x 128 shared weight blocks (the headline); "
+                         "reference: the reference's own numerics (sqrt-softplus x 1.5, 32-wide blocks, 32 x 32, image-token bias)")
+    ap.add_argument("--no-cpu-baseline", action="store_true")
+    ap.add_argument("--overlap", type=int, default=None, choices=[0, 1],
+                    help="many rows: the shared expert on a second stream beside the routed experts (the reference's dual-stream schedule, "
+                         "src/ffn.rs:1000-1040) or after them on the same stream; default: the layer's own choice")
+    ap.add_argument("--copy-probe", action="store_true", help="append four 256 MiB device copies (counter calibration)")
+    ap.add_argument("--profile-steps", type=int, default=64, help="eager passes with per-kernel HIP events for the roofline")
+    args = ap.parse_args()
+    if args.gpus != 1:
+        print("bench.py measures one GPU: the layer runs on a single MI355X (no sharding, no collectives); --gpus %d is not supported" % args.gpus,
+              file=sys.stderr)
+        sys.exit(2)
+    import torch
+    pkg = importlib.import_module("titanic-flash-41_amd")
+    pkg.counters = importlib.import_module("titanic-flash-41_amd.counters")
+    torch.cuda.set_device(0)
+    counter_file = pkg.counters.load()
+    headline = args.config or HEADLINE
+    numerics = args.numerics or ("reference" if headline.startswith("r") else "benchmark")
+    operands = {}
+    record = measure(pkg, headline, numerics, args.steps, args.warmup, args.profile_steps, args.overlap, operands, counter_file,
+                     not args.no_cpu_baseline)
+    line = {"metric": "MoE-layer tokens/s", "value": record.pop("value"), "unit": record.pop("unit"), "n_gpus": 1,
+            "steps": record.pop("steps"), "warmup": record.pop("warmup"), "ms_per_step": record.pop("ms_per_step"),
+            "higher_is_better": True, "scaling": "weak", "vs_baseline": None,
+            "dtype": "fp4 (e2m1 weights, ue8m0 scales) x fp8 (e4m3 activations), f32 accumulate", "data": "synthetic"}
+    line.update(record)
+    if args.config is None:
+        # the other benchmark configurations, each with its own step counts (the headline's are the ones asked for)
+        line["configs"] = {}
+        for name in OTHERS:
+            line["configs"][name] = measure(pkg, name, "benchmark", 2000, 200, args.profile_steps, args.overlap, operands, counter_file, False)
     if args.copy_probe:
         src = torch.empty(256 << 20, dtype=torch.uint8, device="cuda").random_(0, 255)
         dst = torch.empty_like(src)
         for _ in range(4):
             dst.copy_(src)
         torch.cuda.synchronize()
-    layer.close()
     print(json.dumps(line))
 
 

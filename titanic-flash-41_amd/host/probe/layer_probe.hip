@@ -92,22 +92,34 @@ int main(int argc, char** argv) {
         HIP_OK(hipMemcpy(d, x.data(), x.size() * 2, hipMemcpyHostToDevice));
         inputs.push_back((uint64_t)d);
     }
-    double tiles = 0;        // 16-row tiles (= expert weight sets streamed) a pass, averaged over the batches
-    std::vector<int32_t> tile_base(E + 1);
+    double tiles = 0, active = 0, routes = 0;        // tiles, experts with rows and live routes a pass, averaged over the batches
+    std::vector<int32_t> tile_base(E + 1), ids((size_t)rows * g.topk);
     for (int b = 0; b < batches; ++b) {
         if (tfh_layer_run(layer, inputs[b], error, sizeof error)) { std::fprintf(stderr, "run: %s\n", error); return 1; }
         if (tfh_layer_tap(layer, "tile_base", tile_base.data(), tile_base.size() * 4, error, sizeof error) < 0) { std::fprintf(stderr, "tap: %s\n", error); return 1; }
+        if (tfh_layer_tap(layer, "ids", ids.data(), ids.size() * 4, error, sizeof error) < 0) { std::fprintf(stderr, "tap: %s\n", error); return 1; }
         tiles += tile_base[E];
+        std::vector<char> seen(E, 0);
+        for (int32_t e : ids) if (e >= 0 && e < (int32_t)E) { routes += 1; if (!seen[e]) { seen[e] = 1; active += 1; } }
     }
-    tiles /= batches;
-    // algorithmic bytes of the two streaming launches: every tile's expert weights and scales once, the shared expert's once,
-    // the rows' codes, intermediates and outputs
+    tiles /= batches; active /= batches; routes /= batches;
+    // algorithmic bytes of the two launches of the routed experts.  Few rows (streaming launches; the shared expert streams in
+    // them): every 16-row tile's expert weights and scales once, the shared expert's once, the rows' codes, intermediates and
+    // outputs.  Many rows (grouped GEMM; the shared expert runs in kernels of its own): every expert with rows streams its
+    // weights and scales once, the token codes are read once a route, the intermediate is FP8 codes and block scales.
     const double K = g.topk;
     // owners of at most eight rows: the shared expert's up / gate weights stream in the front-end launch, not in the FC1 launch
     const bool early_shared = rows <= 64 && H <= 5120;
-    const double fc1_bytes = tiles * (2.0 * I * H / 2 + 2.0 * I * H / 32) + (early_shared ? 0.0 : 2.0 * S * H) + rows * (2.0 * H + K * I * 2 + 2.0 * S);
-    const double fc2_bytes = tiles * (1.0 * H * I / 2 + 1.0 * H * I / 32) + 1.0 * H * S + rows * (K * I * 2 + K * H * 2 + 2.0 * S + 2.0 * H);
-    std::printf("{\"tiles\": %.3f, \"fc1_algorithmic_bytes\": %.0f, \"fc2_algorithmic_bytes\": %.0f}\n", tiles, fc1_bytes, fc2_bytes);
+    double fc1_bytes, fc2_bytes;
+    if (rows <= 64) {
+        fc1_bytes = tiles * (2.0 * I * H / 2 + 2.0 * I * H / 32) + (early_shared ? 0.0 : 2.0 * S * H) + rows * (2.0 * H + K * I * 2 + 2.0 * S);
+        fc2_bytes = tiles * (1.0 * H * I / 2 + 1.0 * H * I / 32) + 1.0 * H * S + rows * (K * I * 2 + K * H * 2 + 2.0 * S + 2.0 * H);
+    } else {
+        fc1_bytes = active * (2.0 * I * H / 2 + 2.0 * I * H / 32) + routes * (H + H / 128.0) + routes * (I + I / 128.0);
+        fc2_bytes = active * (1.0 * H * I / 2 + 1.0 * H * I / 32) + routes * (I + I / 128.0) + routes * H * 2.0;
+    }
+    std::printf("{\"tiles\": %.3f, \"active_experts\": %.3f, \"routes\": %.1f, \"fc1_algorithmic_bytes\": %.0f, \"fc2_algorithmic_bytes\": %.0f}\n",
+                tiles, active, routes, fc1_bytes, fc2_bytes);
     float ms[6] = {0, 0, 0, 0, 0, 0};
     if (rows <= 64) {
         if (tfh_layer_profile_marks(layer, inputs.data(), batches, passes, 0, ms, error, sizeof error)) { std::fprintf(stderr, "profile: %s\n", error); return 1; }

@@ -27,6 +27,13 @@ class Geometry(ctypes.Structure):
 _lib = None
 
 
+def library_sha256():
+    """SHA-256 of the kernel library file as it lies beside this module (what a counter file is stamped with)."""
+    import hashlib
+    with open(KERNEL_LIB, "rb") as f:
+        return hashlib.sha256(f.read()).hexdigest()
+
+
 def load():
     global _lib
     if _lib is not None:
