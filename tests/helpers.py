@@ -250,6 +250,35 @@ def bf(a):
     return oracle.bf16_to_f32(a).astype(np.float64)
 
 
+def error_report(got_u16, want_u16, floor=1e-3, bound=1e-2):
+    """The layer-output tolerance in both readings.  `max_rel`: max |got - want| over max |want| (relative to the tensor's
+    largest magnitude).  `max_elem_rel`: max over elements of |got - want| / max(|want|, floor * max |want|), the per-element
+    relative error with an absolute floor below which an element's own magnitude no longer shrinks its allowance;
+    `frac_above`: the fraction of elements whose per-element figure exceeds `bound`; `mean_abs`: mean |got - want|."""
+    g, w = bf(got_u16), bf(want_u16)
+    if w.size == 0:
+        return {"max_rel": 0.0, "mean_abs": 0.0, "max_elem_rel": 0.0, "frac_above": 0.0, "elements": 0}
+    scale = np.abs(w).max() + 1e-30
+    diff = np.abs(g - w)
+    elem = diff / np.maximum(np.abs(w), floor * scale)
+    return {"max_rel": float(diff.max() / scale), "mean_abs": float(diff.mean()), "max_elem_rel": float(elem.max()),
+            "frac_above": float((elem > bound).mean()), "elements": int(w.size)}
+
+
+def assert_output_tolerance(name, got_u16, want_u16, max_rel=1e-2, mean_abs=1e-3, frac_above=None, max_elem_rel=None):
+    """Prints both readings of the tolerance and asserts the stated bounds: max relative error (of the tensor's largest
+    magnitude) and mean absolute error always; the per-element figures where the caller states a bound for them."""
+    r = error_report(got_u16, want_u16)
+    print("  %s: max rel %.3e (bound %.0e), mean abs %.3e (bound %.0e); per element with floor 1e-3 max|want|: max %.3e, above 1e-2: %.3e of %d"
+          % (name, r["max_rel"], max_rel, r["mean_abs"], mean_abs, r["max_elem_rel"], r["frac_above"], r["elements"]))
+    assert r["max_rel"] <= max_rel and r["mean_abs"] <= mean_abs, (name, r)
+    if frac_above is not None:
+        assert r["frac_above"] <= frac_above, (name, r)
+    if max_elem_rel is not None:
+        assert r["max_elem_rel"] <= max_elem_rel, (name, r)
+    return r
+
+
 def error_stats(got_u16, want_u16):
     """(max relative error against the reference's largest magnitude per row, mean absolute error)."""
     g, w = bf(got_u16), bf(want_u16)

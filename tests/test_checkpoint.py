@@ -31,6 +31,75 @@ def test_operands_come_back_in_atlas_order(written):
         assert np.array_equal(arrays[name], getattr(ops, name).numpy()), name      # up before gate (routed), gate before up (shared)
 
 
+GOLDEN = os.path.join(os.path.dirname(os.path.abspath(__file__)), "golden", "layout_names.json")
+
+
+def table_from_fixture(prefix, hidden, experts, width):
+    """The reference's name table (tests/golden/layout_names.json, read out of src/layout.rs:247-275) for a layer of these
+    dimensions: {(name, dtype, shape)}."""
+    f = json.load(open(GOLDEN))
+    dims = {"H": hidden, "E": experts, "I": width}
+
+    def shape(entry):
+        out = []
+        for d in entry["dims"]:
+            head, _, div = d.partition("/")
+            out.append((dims[head] if head in dims else int(head)) // (int(div) if div else 1))
+        return tuple(out)
+    rows = set()
+    for entry in f["per_expert"]:
+        for e in range(experts):
+            rows.add((entry["name"].replace("{p}", prefix).replace("{e}", str(e)), entry["dtype"], shape(entry)))
+    for entry in f["per_layer"]:
+        rows.add((entry["name"].replace("{p}", prefix), entry["dtype"], shape(entry)))
+    return f, rows
+
+
+def test_the_loader_requires_exactly_the_references_name_table():
+    # the reference's own model: hidden 5120, 384 experts, the unpadded expert width 2304, 32 x 32 shared weight blocks
+    f, want = table_from_fixture("layers.17", 5120, 384, 2304)
+    assert (f["hidden"], f["experts"], f["expert_width"]) == (5120, 384, 2304)
+    for entry in f["per_expert"] + f["per_layer"]:        # the symbolic shapes reproduce the numbers read from the reference
+        assert tuple(entry["shape"]) == next(s for n, d, s in want if n == entry["name"].replace("{p}", "layers.17").replace("{e}", "0")), entry
+    g = geometry(5120, 384, 6, 2304, 2304, "reference")
+    got = host.checkpoint_contract(g, "layers.17")
+    assert len(got) == len(set(got)) == 6 * 384 + 9
+    assert set(got) == want
+    # and a small layer's table, the one the tests below write and load
+    g = geometry(512, 4, 2, 512, 512, "reference")
+    assert set(host.checkpoint_contract(g, "layers.3")) == table_from_fixture("layers.3", 512, 4, 512)[1]
+
+
+def test_every_tensor_of_the_table_is_required_and_no_other_is_read(written, tmp_path):
+    g, ops, root = written
+    _, table = table_from_fixture("layers.3", 512, 4, 512)
+    index = json.load(open(os.path.join(root, "model.safetensors.index.json")))
+    assert set(index["weight_map"]) == {name for name, _, _ in table}       # the writer follows the same table
+    # dropping any one kind of tensor from the index and its shard header is noticed by name
+    for victim in ["layers.3.ffn.experts.2.w3.scale", "layers.3.ffn.shared_experts.w2.scale", "layers.3.ffn.gate.bias_vl"]:
+        bad = copy_of(root, tmp_path / victim.replace(".", "_"))
+        path = os.path.join(bad, "model.safetensors.index.json")
+        idx = json.load(open(path))
+        shard = idx["weight_map"].pop(victim)
+        json.dump(idx, open(path, "w"))
+        def drop(header, body, victim=victim):
+            header.pop(victim)
+            return header, body
+        rewrite(bad, shard, drop)
+        with pytest.raises(host.HostError, match="missing tensor " + victim.replace(".", r"\.") + "|unindexed|hole|gap|disagree"):
+            host.checkpoint_layer(g, bad, "layers.3")
+    # a wrong dtype for a tensor of the right byte size
+    bad = copy_of(root, tmp_path / "dtype")
+    victim = "layers.3.ffn.experts.1.w2.weight"
+    shard = index["weight_map"][victim]
+    def retype(header, body):
+        header[victim]["dtype"] = "F8_E4M3"
+        return header, body
+    rewrite(bad, shard, retype)
+    with pytest.raises(host.HostError, match="tensor contract mismatch: " + victim):
+        host.checkpoint_layer(g, bad, "layers.3")
+
+
 def rewrite(root, shard, edit):
     path = os.path.join(root, shard)
     data = open(path, "rb").read()
@@ -125,4 +194,7 @@ def test_layer_from_a_checkpoint_equals_the_layer_from_the_operands(tmp_path):
     loaded.set_tokens()
     loaded.run(x)
     assert np.array_equal(loaded.tap("out"), want)
+    # and the loaded layer against the oracle, tap by tap, like a layer built from the operands
+    from test_gpu_layer import check_layer
+    check_layer(g, ops, x.cpu(), loaded.taps())
     loaded.close()

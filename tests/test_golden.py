@@ -10,7 +10,7 @@ import pytest
 import torch
 
 import oracle
-from helpers import CONFIGS, GpuLayer, bf16_ulp_distance, error_stats, geometry, oracle_layer, pkg, synth
+from helpers import CONFIGS, GpuLayer, assert_output_tolerance, bf16_ulp_distance, geometry, oracle_layer, pkg, synth
 
 GOLDEN = os.path.join(os.path.dirname(os.path.abspath(__file__)), "golden")
 NAMES = ["gate_w", "bias", "bias_alt", "w13", "s13", "w2", "s2", "sh_w13", "sh_s13", "sh_w2", "sh_s2"]
@@ -84,7 +84,6 @@ def test_gpu_layer_matches_the_c1_fixture(mode):
     phys = np.nonzero(occupied[:n])[0]
     K, I = g.topk, g.intermediate
     assert bf16_ulp_distance(taps["h"][phys], f["h"].reshape(-1, I)[f["token_map"][phys]]) <= 2.0
-    rel, mean = error_stats(taps["out"], f["out"])
-    assert rel <= 2e-2 and mean <= 1e-3, (rel, mean)
+    assert_output_tolerance("layer output against the fixture", taps["out"], f["out"], max_rel=2e-2, mean_abs=1e-3)
     assert not taps["out"][7].any() or np.array_equal(taps["out"][7], taps["shared_down"][7])   # row 7: no routed part
     layer.close()

@@ -101,10 +101,9 @@ def test_paired_owners_pool_into_one_launch():
     pool_a, pool_b = layer.pair_run(xa_d, tokens_a, live_a, xb_d, tokens_b, live_b, pool_shared=True)
     assert np.array_equal(pool_a[:live_a], alone[0][:live_a]) and np.array_equal(pool_b[:live_b], alone[1][:live_b]), "pooled shared expert"
     # and against the oracle, like any other schedule
-    from helpers import error_stats, oracle_layer
+    from helpers import assert_output_tolerance, oracle_layer
     want = oracle_layer(g, ops, xb, tokens_b, live_b)["out"]
-    rel, mean = error_stats(out_b[:live_b], want[:live_b])
-    assert rel <= 2e-2 and mean <= 1e-3, (rel, mean)
+    assert_output_tolerance("owner B's output", out_b[:live_b], want[:live_b], max_rel=2e-2, mean_abs=1e-3)
     with pytest.raises(host.HostError, match="paired FFN needs two live prefixes"):
         layer.pair_run(xa_d, tokens_a, 0, xb_d, tokens_b, live_b)
     layer.close()

@@ -11,7 +11,7 @@ import pytest
 import torch
 
 import oracle
-from helpers import (CONFIGS, GpuLayer, bf, bf16_ulp_distance, error_stats, geometry, native, np_of, oracle_fc2_from, oracle_layer,
+from helpers import (CONFIGS, GpuLayer, assert_output_tolerance, bf, bf16_ulp_distance, error_stats, geometry, native, np_of, oracle_fc2_from, oracle_layer,
                      synth, u16)
 
 pytestmark = pytest.mark.gpu
@@ -80,9 +80,8 @@ def check_layer(g, ops, x, taps, tokens=None, live=None, padding=None, exact_log
     n_live = rows if live is None else min(live, rows)
     routed, out = oracle.ffn_sum_shared(taps["route_out"], taps["shared_down"], n_live)
     assert np.array_equal(taps["routed"][:n_live], routed[:n_live]) and np.array_equal(taps["out"], out), "combine differs"
-    rel, mean = error_stats(taps["out"], again["out"])
-    assert rel <= max_rel and mean <= MEAN_ABS, ("layer output", rel, mean)
-    return rel, mean
+    r = assert_output_tolerance("layer output", taps["out"], again["out"], max_rel=max_rel, mean_abs=MEAN_ABS)
+    return r["max_rel"], r["mean_abs"]
 
 
 @pytest.mark.parametrize("mode", ["benchmark", "reference"])

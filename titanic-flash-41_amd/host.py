@@ -227,6 +227,21 @@ class Layer:
         return dict(zip(["tile_m", "max_tiles", "scratch_bytes", "atlas_bytes", "expert_bytes", "scale_code_bytes", "raw_rows", "coded_rows"], v))
 
 
+def checkpoint_contract(geometry, prefix):
+    """What the loader requires of a checkpoint for one layer: a list of (tensor name, dtype string, shape tuple)."""
+    lib = load()
+    lib.tfh_checkpoint_contract.restype = ctypes.c_longlong
+    lib.tfh_checkpoint_contract.argtypes = [ctypes.c_char_p, ctypes.c_void_p, ctypes.c_char_p, ctypes.c_size_t]
+    need = lib.tfh_checkpoint_contract(prefix.encode(), ctypes.byref(geometry), None, 0)
+    text = ctypes.create_string_buffer(need)
+    lib.tfh_checkpoint_contract(prefix.encode(), ctypes.byref(geometry), text, need)
+    rows = []
+    for line in text.value.decode().splitlines():
+        name, dtype, shape = line.split(" ")
+        rows.append((name, dtype, tuple(int(d) for d in shape.split(","))))
+    return rows
+
+
 def checkpoint_layer(geometry, root, prefix):
     """Scans a safetensors checkpoint directory and assembles one layer's operands on the host (no device involved).
     Returns (dict of numpy arrays in the canonical layout, tensors in the checkpoint, shards)."""

@@ -105,6 +105,18 @@ int tfh_checkpoint_layer(const char* root, const char* prefix, const ca_geometry
         counts[0] = checkpoint.tensors(); counts[1] = checkpoint.shards();
     });
 }
+// The loader's tensor contract for one layer as text, a tensor a line: "<name> <dtype> <d0>,<d1>".  Returns the length the
+// text needs (with its terminator); fills `out` when `out_len` holds it.
+long long tfh_checkpoint_contract(const char* prefix, const ca_geometry* geometry, char* out, size_t out_len) {
+    std::string text;
+    for (const tf::TensorContract& t : tf::ffn_layer_contract(prefix, *geometry)) {
+        text += t.name + " " + t.dtype + " ";
+        for (size_t i = 0; i < t.shape.size(); ++i) text += (i ? "," : "") + std::to_string(t.shape[i]);
+        text += "\n";
+    }
+    if (out && out_len > text.size()) std::memcpy(out, text.c_str(), text.size() + 1);
+    return (long long)text.size() + 1;
+}
 void tfh_layer_destroy(void* handle) { delete (Handle*)handle; }
 // The geometry the layer runs with (the caller's, with the expert widths padded to multiples of 512): the widths of the taps.
 void tfh_layer_geometry(void* handle, ca_geometry* out) { *out = ((Handle*)handle)->native->geometry(); }

@@ -245,28 +245,35 @@ std::vector<uint8_t> Checkpoint::read(const std::string& name) const {
     return out;
 }
 
-LayerOperandsHost load_ffn_layer(const Checkpoint& cp, const std::string& p, const ca_geometry& g) {
+std::vector<TensorContract> ffn_layer_contract(const std::string& p, const ca_geometry& g) {
     const uint64_t H = g.hidden, E = g.experts, I = g.intermediate, S = g.shared_intermediate, bn = g.shared_bn, bk = g.shared_bk;
-    LayerOperandsHost out;
-    // the contract first (src/layout.rs:247-275), then the bytes
+    std::vector<TensorContract> c;
     for (uint64_t e = 0; e < E; ++e) {
         const std::string x = p + ".ffn.experts." + std::to_string(e) + ".";
         for (const char* name : {"w1", "w3"}) {
-            cp.require(x + name + ".weight", "I8", {I, H / 2});
-            cp.require(x + name + ".scale", "F8_E8M0", {I, H / 32});
+            c.push_back({x + name + ".weight", "I8", {I, H / 2}});
+            c.push_back({x + name + ".scale", "F8_E8M0", {I, H / 32}});
         }
-        cp.require(x + "w2.weight", "I8", {H, I / 2});
-        cp.require(x + "w2.scale", "F8_E8M0", {H, I / 32});
+        c.push_back({x + "w2.weight", "I8", {H, I / 2}});
+        c.push_back({x + "w2.scale", "F8_E8M0", {H, I / 32}});
     }
     for (const char* name : {"w1", "w3"}) {
-        cp.require(p + ".ffn.shared_experts." + name + ".weight", "F8_E4M3", {S, H});
-        cp.require(p + ".ffn.shared_experts." + name + ".scale", "F8_E8M0", {S / bn, H / bk});
+        c.push_back({p + ".ffn.shared_experts." + name + ".weight", "F8_E4M3", {S, H}});
+        c.push_back({p + ".ffn.shared_experts." + name + ".scale", "F8_E8M0", {S / bn, H / bk}});
     }
-    cp.require(p + ".ffn.shared_experts.w2.weight", "F8_E4M3", {H, S});
-    cp.require(p + ".ffn.shared_experts.w2.scale", "F8_E8M0", {H / bn, S / bk});
-    cp.require(p + ".ffn.gate.weight", "BF16", {E, H});
-    cp.require(p + ".ffn.gate.bias", "F32", {E});
-    cp.require(p + ".ffn.gate.bias_vl", "F32", {E});
+    c.push_back({p + ".ffn.shared_experts.w2.weight", "F8_E4M3", {H, S}});
+    c.push_back({p + ".ffn.shared_experts.w2.scale", "F8_E8M0", {H / bn, S / bk}});
+    c.push_back({p + ".ffn.gate.weight", "BF16", {E, H}});
+    c.push_back({p + ".ffn.gate.bias", "F32", {E}});
+    c.push_back({p + ".ffn.gate.bias_vl", "F32", {E}});
+    return c;
+}
+
+LayerOperandsHost load_ffn_layer(const Checkpoint& cp, const std::string& p, const ca_geometry& g) {
+    const uint64_t H = g.hidden, E = g.experts, I = g.intermediate;
+    LayerOperandsHost out;
+    // the contract first (src/layout.rs:247-275), then the bytes
+    for (const TensorContract& t : ffn_layer_contract(p, g)) cp.require(t.name, t.dtype, t.shape);
 
     auto append = [&](std::vector<uint8_t>& to, const std::string& name, bool expert_scale) {
         const std::vector<uint8_t> bytes = cp.read(name);

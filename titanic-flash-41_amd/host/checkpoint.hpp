@@ -43,6 +43,10 @@ struct LayerOperandsHost {
     std::vector<float> bias, bias_alt;
     std::vector<uint8_t> w13, s13, w2, s2, sh_w13, sh_s13, sh_w2, sh_s2;
 };
+// What the loader requires of a checkpoint for one layer, in the order it checks it (src/layout.rs:247-275): every tensor's
+// name, dtype as the header spells it, and shape.  load_ffn_layer requires exactly these and reads nothing else.
+struct TensorContract { std::string name, dtype; std::vector<uint64_t> shape; };
+std::vector<TensorContract> ffn_layer_contract(const std::string& prefix, const ca_geometry& g);
 // prefix: the layer's name prefix in the checkpoint ("layers.7"): tensors "<prefix>.ffn.experts.<e>.w1.weight" ...
 LayerOperandsHost load_ffn_layer(const Checkpoint& checkpoint, const std::string& prefix, const ca_geometry& g);
 
