@@ -65,14 +65,14 @@ __device__ __forceinline__ void tf_mfma_settle(v4f (&acc)[8]) {
     asm volatile("s_nop 15\n\ts_nop 15"
                  : "+v"(acc[0]), "+v"(acc[1]), "+v"(acc[2]), "+v"(acc[3]), "+v"(acc[4]), "+v"(acc[5]), "+v"(acc[6]), "+v"(acc[7]));
 }
-// Requests that may still be in flight at the top of k-step `u` of an unrolled round of four: those issued in the LEAD - 1
-// k-steps before it.  Every k-step issues DATA requests, k-step 1 of a round two more (the next round's weight scales).
-// Requests the count does not know (the next tasks' permutation map, stores) only make the wait stricter: it lets the N
-// youngest stay in flight, and whatever is younger than the k-step's own requests may.
-template <int LEAD, int DATA>
+// Requests that may still be in flight at the barrier of k-step `u` of an unrolled round of four: those issued in the
+// LEAD - 1 k-steps before it.  Every k-step issues DATA requests, k-step EXTRA of a round two more (the next round's weight
+// scales).  Requests the count does not know (the next tasks' permutation map, stores) only make the wait stricter: it
+// lets the N youngest stay in flight, and whatever is younger than the k-step's own requests may.
+template <int LEAD, int DATA, int EXTRA>
 constexpr int tf_loads_behind(int u) {
     int n = 0;
-    for (int j = 1; j < LEAD; ++j) n += DATA + (((u - j) & 3) == 1 ? 2 : 0);
+    for (int j = 1; j < LEAD; ++j) n += DATA + (((u - j) & 3) == EXTRA ? 2 : 0);
     return n;
 }
 
@@ -210,7 +210,12 @@ __global__ void __launch_bounds__(512) tf_grouped_gemm(const GemmArgs p) {
     // weight tiles of the wave within a stage: FC1: four "up" tiles 4 wn + t, then the four "gate" tiles 8 + 4 wn + t of the same
     // columns; FC2: tiles 8 wn + t.  One base a wave plus a constant a tile.
     const int b_first = FC1 ? wn * 4 : wn * 8;
-    const int issue_slot = (wave + (wave >> 2) * 2) & 3;          // waves w and w + 4 share a SIMD: slots s and s + 2
+    // Waves w and w + 4 share a SIMD.  Waves 4 - 7 ("late") run half a k-step behind waves 0 - 3 ("early"): a wave passes one
+    // barrier a k-step, the early waves at its top, the late waves in its middle (and one more before their first k-step, as
+    // the early waves do after their last), so the early waves' barrier of k-step b is the late waves' of k-step b - 1.
+    // While one wave of a SIMD waits at its barrier and for its first operands from LDS, the other is in the middle of
+    // its products.
+    const bool late = wave >= 4;
     auto b_step = [](int t) constexpr { return FC1 ? (t < 4 ? t : 8 + t - 4) : t; };
 
     // ---- the first task's first k-steps, and the second task's slot ------------------------------------------------------------
@@ -225,9 +230,14 @@ __global__ void __launch_bounds__(512) tf_grouped_gemm(const GemmArgs p) {
     for (int d = 0; d < LEAD; ++d)
 #pragma unroll
         for (int op = 0; op < DATA; ++op) issue_op(now, op, d, d);
+    if (late) {                             // the late waves request one k-step further ahead throughout
+#pragma unroll
+        for (int op = 0; op < DATA; ++op) issue_op(now, op, LEAD, LEAD);
+    }
     TaskRef nxt = fetch(min(local + local_count, my_tasks - 1), 1);
     tf_wait_vm<0>();
     int cs = 0, ps = LEAD;                  // stage read in the current k-step; stage the k-step LEAD ahead is written to
+    if (late) __builtin_amdgcn_s_barrier();
     int slot = 0, slot_next = 1, slot_after = 2;
     for (int q = local; q < my_tasks; q += local_count) {
         const int rows = cur.rows, first_tile = cur.first_tile, ng = cur.ng;
@@ -253,23 +263,57 @@ __global__ void __launch_bounds__(512) tf_grouped_gemm(const GemmArgs p) {
             auto k_step = [&](auto u_constant, auto first_constant, auto last_constant, int ks) {
                 constexpr int u = decltype(u_constant)::value;
                 constexpr bool FIRST = decltype(first_constant)::value, LAST = decltype(last_constant)::value;
-                // the task's first LEAD k-steps landed before the previous task's stores went out (below)
-                if constexpr (!FIRST || u >= LEAD) tf_wait_vm<tf_loads_behind<LEAD, DATA>(u)>();
-                __builtin_amdgcn_s_barrier();
+                // The k-step's barrier: at the top for the early waves, in the middle for the late waves, whose barrier of k-step
+                // u is the early waves' of k-step u + 1.  Behind barrier b (the early waves' top of k-step b) the stage of k-step b
+                // is whole (every wave waited for its share before it) and no wave reads the stage of k-step b - 1 any more (the
+                // late waves have taken their last fragments of it into registers before their barrier), so every wave then
+                // requests its share of k-step b + LEAD into it: the early waves in k-step b, the late waves in the second half
+                // of their k-step b - 1.  A task's first k-steps landed before the previous task's stores went out (below).
+                if (!late) {
+                    if constexpr (!FIRST || u >= LEAD) tf_wait_vm<tf_loads_behind<LEAD, DATA, 1>(u)>();
+                    __builtin_amdgcn_s_barrier();
+                }
                 asm volatile("" ::: "memory");
                 if constexpr (FIRST && u == 0) install(then, nxt, slot_next);
-                constexpr bool OVER = LAST && u + LEAD >= 4;           // the requests belong to the next task
-                const int ks_ahead = OVER ? u + LEAD - 4 : ks + LEAD;
-                const Source& from = OVER ? then : now;
-                constexpr int OPS = DATA + (u == 1 ? 2 : 0);           // k-step 1 of a round: the next round's weight scales first
-                auto issue_range = [&](int lo, int hi) {
+                // requests of this k-step: `ahead` k-steps on (early waves LEAD, late waves LEAD + 1), the next task's in its last;
+                // one k-step of a round (`extra`: the early waves' 1, the late waves' 0) first requests the next round's weight
+                // scales: behind that k-step's barrier no wave reads this round's any more (they are in registers since the top
+                // of k-step 0), and the early waves' top of the next round's k-step 0 finds them landed by either count
+                auto issue_range = [&](auto ahead_constant, auto extra_constant) {
+                    constexpr int AHEAD = decltype(ahead_constant)::value;
+                    constexpr bool EXTRA = decltype(extra_constant)::value == u;
+                    constexpr bool OVER = LAST && u + AHEAD >= 4;
+                    const int ks_ahead = OVER ? u + AHEAD - 4 : ks + AHEAD;
+                    const Source& from = OVER ? then : now;
+                    const int stage = AHEAD == LEAD ? ps : (ps + 1 == NS ? 0 : ps + 1);
+                    if constexpr (EXTRA) {
 #pragma unroll
-                    for (int i = lo; i < hi; ++i) {
-                        if (u == 1 && i < 2) issue_op(LAST ? then : now, DATA + i, LAST ? 0 : ks + 3, 0);
-                        else issue_op(from, i - (u == 1 ? 2 : 0), ks_ahead, ps);
+                        for (int i = 0; i < 2; ++i) issue_op(LAST ? then : now, DATA + i, LAST ? 0 : ks + 4 - u, 0);
+                    }
+#pragma unroll
+                    for (int i = 0; i < DATA; ++i) issue_op(from, i, ks_ahead, stage);
+                };
+                const std::integral_constant<int, LEAD> early_ahead;
+                const std::integral_constant<int, LEAD + 1> late_ahead;
+                const std::integral_constant<int, 1> early_extra;
+                const std::integral_constant<int, 0> late_extra;
+                auto middle = [&]() {
+                    if (late) {
+                        // the late waves' share of the next k-step's stage (the next task's first, after a task's last k-step);
+                        // what they requested for the task's first LEAD + 1 k-steps landed before their last stores
+                        constexpr bool WAIT = u == 3 || !(FIRST && u + 1 <= LEAD);
+                        if constexpr (WAIT) tf_wait_vm<tf_loads_behind<LEAD, DATA, 0>(u)>();
+                        asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory");      // this k-step's last reads of its stage have returned
+                        __builtin_amdgcn_s_barrier();
+                        asm volatile("" ::: "memory");
+                        issue_range(late_ahead, late_extra);
                     }
                 };
-                if constexpr (FR == 0) issue_range(0, OPS);
+                constexpr int HALF = (FR + 1) / 2;                     // fragments before the late waves' barrier
+                if constexpr (FR == 0) {
+                    if (!late) issue_range(early_ahead, early_extra);
+                    middle();
+                }
                 if constexpr (FR > 0) {
                     const uint8_t* sa = s_a + cs * A_STAGE;
                     const uint8_t* sb = s_b + cs * B_STAGE + b_first * 1024 + lane16;
@@ -289,7 +333,8 @@ __global__ void __launch_bounds__(512) tf_grouped_gemm(const GemmArgs p) {
                     word[0] = sc[0];
 #pragma unroll
                     for (int f = 0; f < FR; ++f) {
-                        if (f + 1 < FR) {
+                        if (f == HALF) middle();
+                        if (f + 1 < FR && f + 1 <= HALF) {
                             lo[(f + 1) & 1] = *reinterpret_cast<const u4v*>(sa + a_lo + (f + 1) * 2048);
                             hi[(f + 1) & 1] = *reinterpret_cast<const u4v*>(sa + a_hi + (f + 1) * 2048);
                             word[(f + 1) & 1] = sc[(f + 1) * 16];
@@ -300,12 +345,21 @@ __global__ void __launch_bounds__(512) tf_grouped_gemm(const GemmArgs p) {
                         const v8i av = v8i{(int)l[0], (int)l[1], (int)l[2], (int)l[3], (int)h[0], (int)h[1], (int)h[2], (int)h[3]};
 #pragma unroll
                         for (int t = 0; t < 8; ++t) tf_mfma_weights_first<u, SEL>(acc[f][t], bf[t], av, bsc[t], sca);
-                        // this wave's requests of the k-step, all behind one fragment's products and a different fragment for the
-                        // two waves of a SIMD and for neighbouring SIMDs: a request holds its wave until the address unit takes it,
-                        // and eight waves requesting at once hold each other while no product is issued
-                        if (f == issue_slot % FR) issue_range(0, OPS);
+                        // the early waves' requests of the k-step behind their first fragment's products, so that their address
+                        // arithmetic runs under the matrix pipeline (the late waves': behind their barrier, above)
+                        if (f == 0) { if (!late) issue_range(early_ahead, early_extra); }
                         __builtin_amdgcn_sched_barrier(0);       // keeps fragment f + 2's reads behind these products: two register sets
+                        // the fragment behind the middle barrier's first leaves LDS before that barrier too, into the registers
+                        // these products have just read: behind the barrier no wave reads this stage
+                        if (f == HALF - 1 && HALF + 1 < FR) {
+                            static_assert(FR <= 4, "two register sets");
+                            lo[(HALF + 1) & 1] = *reinterpret_cast<const u4v*>(sa + a_lo + (HALF + 1) * 2048);
+                            hi[(HALF + 1) & 1] = *reinterpret_cast<const u4v*>(sa + a_hi + (HALF + 1) * 2048);
+                            word[(HALF + 1) & 1] = sc[(HALF + 1) * 16];
+                            __builtin_amdgcn_sched_barrier(0);
+                        }
                     }
+                    if constexpr (HALF == FR) middle();
                 }
                 cs = cs + 1 == NS ? 0 : cs + 1;
                 ps = ps + 1 == NS ? 0 : ps + 1;
@@ -435,6 +489,7 @@ __global__ void __launch_bounds__(512) tf_grouped_gemm(const GemmArgs p) {
         const int done = slot;
         slot = slot_next; slot_next = slot_after; slot_after = done;
     }
+    if (!late) __builtin_amdgcn_s_barrier();
 }
 
 // Shapes the streamed grouped GEMM takes: contraction lengths that are multiples of 512, at most 512 experts (one thread an
