@@ -15,6 +15,7 @@ CSRC = os.path.join(HERE, "csrc")
 HOST = os.path.join(HERE, "host")
 KERNEL_LIB = os.path.join(HERE, "libtitanic_moe_hip.so")
 CODE_OBJECT = os.path.join(HERE, "titanic_moe_gfx950.hsaco")
+REFERENCE_LAYER_OBJECT = os.path.join(HERE, "titanic_moe_gfx950_reference_layer.hsaco")
 HOST_LIB = os.path.join(HERE, "libtitanic_ffn_host.so")
 PROBE = os.path.join(HERE, "tf_layer_probe")
 MANIFEST = os.path.join(HERE, "manifest.json")
@@ -37,6 +38,8 @@ def build_kernels():
     src = os.path.join(CSRC, "abi.hip")
     _run(["hipcc", *DEVICE_FLAGS, "-fPIC", "-shared", src, "-o", KERNEL_LIB])
     _run(["hipcc", *DEVICE_FLAGS, "--genco", src, "-o", CODE_OBJECT])
+    # the kernels the reference launches by name with fixed argument lists, for its own layer's dimensions
+    _run(["hipcc", *DEVICE_FLAGS, "--genco", os.path.join(CSRC, "reference_layer.hip"), "-o", REFERENCE_LAYER_OBJECT])
     return KERNEL_LIB
 
 
@@ -65,6 +68,7 @@ def write_manifest():
         return hashlib.sha256(open(path, "rb").read()).hexdigest() if os.path.exists(path) else None
     manifest = {"schema": 1, "architecture": "gfx950", "abi": 1, "library": os.path.basename(KERNEL_LIB), "library_sha256": digest(KERNEL_LIB),
                 "code_object": os.path.basename(CODE_OBJECT), "code_object_sha256": digest(CODE_OBJECT),
+                "reference_layer_object": os.path.basename(REFERENCE_LAYER_OBJECT), "reference_layer_object_sha256": digest(REFERENCE_LAYER_OBJECT),
                 "host_library": os.path.basename(HOST_LIB), "host_library_sha256": digest(HOST_LIB)}
     with open(MANIFEST, "w") as f:
         json.dump(manifest, f, indent=1)

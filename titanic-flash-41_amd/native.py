@@ -8,6 +8,7 @@ import os
 HERE = os.path.dirname(os.path.abspath(__file__))
 KERNEL_LIB = os.path.join(HERE, "libtitanic_moe_hip.so")
 CODE_OBJECT = os.path.join(HERE, "titanic_moe_gfx950.hsaco")
+REFERENCE_LAYER_OBJECT = os.path.join(HERE, "titanic_moe_gfx950_reference_layer.hsaco")
 
 EXPORTS = ["ca_ffn_abi", "ca_ffn_configure", "ca_ffn_geometry", "ca_router_logits", "ca_shared_swiglu", "ca_ffn_add",
            "ca_router_logits_wide", "ca_kernel_launch", "ca_kernel_count", "ca_kernel_name", "ca_moe_nibble_permute",
