@@ -8,7 +8,7 @@ import pytest
 import torch
 
 import oracle
-from helpers import bf16_ulp_distance, configure, geometry, native, np_of, pkg, synth
+from helpers import GpuLayer, bf16_ulp_distance, configure, geometry, native, np_of, pkg, synth
 from test_gpu_layer import check_layer
 
 pytestmark = pytest.mark.gpu
@@ -87,3 +87,64 @@ def test_dense_product_of_few_rows():
         assert st == 0, st
         assert bf16_ulp_distance(np_of(out).view(np.uint16), want) <= 1.0, (m, n, k)
     native.load().ca_primitives_close(ctypes.c_void_p(ctx))
+
+
+def test_micro_sequence_keeps_fp32_projections_and_equals_entry_0():
+    # the reference's micro sequence (src/moe.rs:379-393, 625-629): gemm.mxfp8_quant_cute, moe.w4a8.compact_micro with an FP32
+    # projections buffer, moe.w4a16.topk_sum, through entries 12, 11, 2 with the operand lists of
+    # contracts/runtime-contract-micro-m4.json.  Route outputs and the sum: the bits of entry 0 (same arithmetic, a pair's
+    # result does not depend on how the routes are grouped); the FP32 projections: the oracle's within FP32 accumulation order.
+    import json
+    import os
+    from helpers import oracle_config
+    g = geometry(1024, 16, 2, 512, 512, "reference")
+    ops = synth.LayerOperands(g, "micro", device="cuda")
+    rows = 4
+    x = synth.activations("micro", rows, g.hidden).cuda().contiguous()
+    layer = GpuLayer(g, ops, rows)
+    taps = layer.run(x, fuse_route=False)
+    K, H, I, E, B = g.topk, g.hidden, g.intermediate, g.experts, g.act_block
+    pairs = rows * K
+    tiles = -(-pairs // 16) - 1 + min(E, pairs)
+    d = "cuda"
+    values = torch.zeros((rows, H), dtype=torch.uint8, device=d)
+    scale_rows = torch.zeros((rows, H // B), dtype=torch.uint8, device=d)
+    scale_mma = torch.zeros((rows, H // B), dtype=torch.uint8, device=d)
+    assert native.primitives_launch(layer.ctx, 12, [x, values, scale_rows, scale_mma], [rows, H, rows * 10]) == 0
+    torch.cuda.synchronize()
+    assert np.array_equal(np_of(values), taps["xq"]) and np.array_equal(np_of(scale_rows), taps["xs"]) and torch.equal(scale_rows, scale_mma)
+    floored = torch.zeros_like(values), torch.zeros_like(scale_rows)
+    assert native.primitives_launch(layer.ctx, 13, [x, floored[0], floored[1], None], [rows, H, 0]) == 0
+    torch.cuda.synchronize()
+    assert np.array_equal(np_of(floored[0]), taps["xq_min"]) and np.array_equal(np_of(floored[1]), taps["xs_min"])
+    inter = torch.zeros((tiles * 16, I), dtype=torch.int16, device=d)
+    proj = torch.full((pairs, 2 * I), float("nan"), dtype=torch.float32, device=d)
+    route_out = torch.zeros((rows, K, H), dtype=torch.int16, device=d)
+    ones = torch.ones(16, dtype=torch.float32, device=d)
+    tables = [torch.full((tiles,), -1, dtype=torch.int32, device=d), torch.full((tiles,), -1, dtype=torch.int32, device=d),
+              torch.full((E + 1,), -1, dtype=torch.int32, device=d), torch.full((tiles * 16,), -1, dtype=torch.int32, device=d),
+              torch.zeros((tiles * 16,), dtype=torch.float32, device=d)]
+    micro = [values, scale_rows, layer.w13, layer.s13, inter, proj, layer.weights, layer.ids, ones, ones, layer.w2, layer.s2, route_out, ones, ones] + tables
+    assert native.primitives_launch(layer.ctx, 11, micro, [pairs, 48]) == 0
+    out = torch.zeros((rows, H), dtype=torch.int16, device=d)
+    assert native.primitives_launch(layer.ctx, 2, [route_out, out, out], [rows, 0, 0]) == 0      # third pointer: reserved, never read
+    torch.cuda.synchronize()
+    assert np.array_equal(np_of(route_out).view(np.uint16), taps["route_out"])
+    assert np.array_equal(np_of(out).view(np.uint16), taps["routed"])
+    _, want_proj = oracle.expert_fc1(oracle_config(g), taps["xq"], taps["xs"], np_of(ops.w13), np_of(ops.s13), taps["ids"], want_proj=True)
+    got = np_of(proj).reshape(rows, K, 2 * I)
+    assert np.isfinite(got).all()
+    assert np.abs(got - want_proj).max() <= 2e-5 * np.abs(want_proj).max()
+    # argument checks: a pair count that is no multiple of top-k, too many rows
+    assert native.primitives_launch(layer.ctx, 11, micro, [pairs + 1, 48]) == -1
+    assert native.primitives_launch(layer.ctx, 11, micro, [65 * K, 48]) == -1
+    # the committed contract names these entries and operand lists
+    root = os.path.join(os.path.dirname(os.path.abspath(native.__file__)), "contracts")
+    contract = json.load(open(os.path.join(root, "runtime-contract-micro-m4.json")))
+    bindings = json.load(open(os.path.join(root, "bindings.json")))
+    assert [n["kernel_id"] for n in contract["nodes"]] == ["gemm.mxfp8_quant_cute", "moe.w4a8.compact_micro", "moe.w4a16.topk_sum"]
+    assert contract["projection_dtype"] == "float32"
+    for node in contract["nodes"]:
+        entry = bindings["entries"][node["entry"]]
+        assert entry["kernel_id"] == node["kernel_id"] and set(entry["pointers"]) == set(node["pointers"]) and set(entry["i32_scalars"]) == set(node["scalars"])
+    layer.close()

@@ -169,7 +169,7 @@ int codec_blocks(const Context& c, long long rows, int k) {
 }
 // `packed_input`: p[P_A] holds wire rows "dual_quant_rows_v1" (src/moe.rs:512-583) instead of BF16 rows.
 int launch_dynamic(const Context& c, bool route, const uint64_t* p, const int32_t* sc, hipStream_t s, int phases = 7, const uint64_t* sh = nullptr,
-                   const SumArgs* sum = nullptr, bool packed_input = false) {
+                   const SumArgs* sum = nullptr, bool packed_input = false, float* projections = nullptr) {
     const ca_geometry& g = c.g;
     const int rows = sc[S_TOKENS], tile_m = sc[S_TILE_M], groups = sc[S_GROUPS], max_tiles = sc[S_MAX_TILES];
     if (rows < 1 || rows > sc[S_MAX_ROWS] || groups < 1 || max_tiles < 1 || sc[S_ROWS_PADDED] != max_tiles * tile_m) return -1;
@@ -278,6 +278,7 @@ int launch_dynamic(const Context& c, bool route, const uint64_t* p, const int32_
         a.out = (uint16_t*)p[P_INTER];
         a.table_tiles = max_tiles;
         StreamArgs b = a;
+        a.proj = projections;
         b.a_codes = nullptr; b.a_scales = nullptr; b.a_bf16 = (const uint16_t*)p[P_INTER];
         b.q_codes = (uint8_t*)p[P_INTER_CODES]; b.q_scales = (uint8_t*)p[P_INTER_SCALES]; b.min_amax = 0.f;
         b.w = (const uint8_t*)p[P_W2]; b.ws = (const uint8_t*)p[P_S2];
@@ -298,7 +299,7 @@ int launch_dynamic(const Context& c, bool route, const uint64_t* p, const int32_
         mark(c, 4, s);
         return launch_status();
     }
-    if (sh) return -4;   // many rows: the shared expert runs through its own entry
+    if (sh || projections) return -4;   // many rows: the shared expert runs through its own entry; no FP32 projection tap
     if (!p[P_INTER_CODES] || !p[P_INTER_SCALES]) return -1;
     GemmArgs a{};
     a.a_codes = (const uint8_t*)p[P_PACKED]; a.a_scales = (const uint8_t*)p[P_SCALES];
@@ -329,8 +330,9 @@ int launch_topk_sum(const Context& c, const uint64_t* p, const int32_t* sc, hipS
     if (!p[0] || !p[1] || sc[0] < 0 || sc[1] != 0 || sc[2] != 0) return -1;
     if (sc[0] == 0) return 0;
     const long long n8 = (long long)sc[0] * (c.g.hidden >> 3);
-    ca_moe_topk_sum<<<(int)((n8 + 255) / 256), 256, 0, s>>>((const uint16_t*)p[0], (uint16_t*)p[1], sc[0], c.g.topk, c.g.hidden,
-                                                           (const int32_t*)p[2], sc[0]);
+    // the live rows arrive as active_m (the reference's host patches that scalar, src/moe.rs:1229); the third pointer is reserved
+    // and never read: a contract may bind it to any operand
+    ca_moe_topk_sum<<<(int)((n8 + 255) / 256), 256, 0, s>>>((const uint16_t*)p[0], (uint16_t*)p[1], sc[0], c.g.topk, c.g.hidden, nullptr, sc[0]);
     return launch_status();
 }
 // ---- entry 3: gemm.mxfp8_quant_cute --------------------------------------------------------------------------------
@@ -345,6 +347,54 @@ int launch_quant(const Context& c, const uint64_t* p, const int32_t* sc, hipStre
     ca_quantize_rows<<<blocks, 256, 0, s>>>((const uint16_t*)p[0], (uint8_t*)p[1], (uint8_t*)p[2], (uint8_t*)p[3], (uint8_t*)p[4], m, k,
                                             c.g.act_block);
     return launch_status();
+}
+// ---- entries 12, 13: gemm.mxfp8_quant_cute with the reference's own operand list (src/moe.rs:557-561, 573-575): source,
+// values, row-major block scales, and a second scale buffer.  The reference's second buffer holds the scales in the order
+// its matrix instructions read them; this library's kernels read the row-major ones, and the second buffer (may be null)
+// receives the same bytes.  Entry 12: no amax floor (the routed experts' flavour); entry 13: amax floored at 1e-4 (the
+// shared expert's).  `grid_x` is the reference kernel's launch width and is not used here.
+int launch_quant_reference(const Context& c, const uint64_t* p, const int32_t* sc, hipStream_t s, bool floored) {
+    const int m = sc[0], k = sc[1];
+    if (!p[0] || !p[1] || !p[2] || m < 1 || k < c.g.act_block || k % c.g.act_block || sc[2] < 0) return -1;
+    const long long items = (long long)m * (k >> 3);
+    int blocks = (int)((items + 255) / 256);
+    if (blocks > c.cus * 16) blocks = c.cus * 16;
+    ca_quantize_rows<<<blocks, 256, 0, s>>>((const uint16_t*)p[0], floored ? nullptr : (uint8_t*)p[1], floored ? nullptr : (uint8_t*)p[2],
+                                            floored ? (uint8_t*)p[1] : nullptr, floored ? (uint8_t*)p[2] : nullptr, m, k, c.g.act_block);
+    int status = launch_status();
+    if (status || !p[3]) return status;
+    return (int)hipMemcpyAsync((void*)p[3], (const void*)p[2], (size_t)m * (k / c.g.act_block), hipMemcpyDeviceToDevice, s);
+}
+// ---- entry 11: moe.w4a8.compact_micro (src/moe.rs:379-393, 625-629; runtime/kernels/moe-runtime-m6-micro-fp32-v1) -----
+// Both projections of the routed experts for a few rows whose token codes are already quantized (entry 12 before it), with
+// the FP32 projections of FC1 kept: projections[pair][2 I] (up, then gate).  Pointers: the reference's fifteen (the four
+// `ones` scale pointers are not read: E8M0 block scales carry every scale here), then this library's plan tables.  The
+// routes are grouped by expert as in entry 0, so an expert chosen by several rows streams once; a pair's results do not
+// depend on the grouping.  num_pairs = live rows x top-k.
+enum MicroPtr { M_CODES, M_CODE_SCALES, M_W13, M_S13, M_INTER, M_PROJ, M_WEIGHTS, M_IDS, M_ALPHA1, M_INPUT_SCALE, M_W2, M_S2, M_OUT, M_ALPHA2,
+                M_DOWN_SCALE, M_TASK_EXPERT, M_TASK_VALID, M_TILE_BASE, M_TOKEN_MAP, M_TILE_WEIGHTS, M_COUNT };
+int launch_micro(const Context& c, const uint64_t* p, const int32_t* sc, hipStream_t s) {
+    const ca_geometry& g = c.g;
+    const int pairs = sc[0];
+    for (int i = 0; i < M_COUNT; ++i)
+        if (!p[i] && i != M_PROJ && i != M_ALPHA1 && i != M_INPUT_SCALE && i != M_ALPHA2 && i != M_DOWN_SCALE) return -1;
+    if (pairs < 1 || pairs % g.topk || pairs / g.topk > TF_STREAM_MAX_ROWS || sc[1] < 0) return -1;
+    const int rows = pairs / g.topk;
+    const int tiles = (pairs + 15) / 16 - 1 + (g.experts < pairs ? g.experts : pairs);
+    if (tiles > TF_LDS_TILES) return -1;
+    // the plan alone: the front-end kernel with no columns to quantize
+    ca_moe_frontend<<<1, 512, 0, s>>>(nullptr, (const int32_t*)p[M_IDS], (const float*)p[M_WEIGHTS], nullptr, nullptr, (int32_t*)p[M_TOKEN_MAP],
+                                      (float*)p[M_TILE_WEIGHTS], (int32_t*)p[M_TASK_EXPERT], (int32_t*)p[M_TASK_VALID], (int32_t*)p[M_TILE_BASE],
+                                      rows, g.topk, g.experts, 0, 1, 16, g.act_block, nullptr, nullptr);
+    const int status = launch_status();
+    if (status) return status;
+    uint64_t q[P_DYN_COUNT] = {};
+    q[P_A] = p[M_CODES]; q[P_IDS] = p[M_IDS]; q[P_WEIGHTS] = p[M_WEIGHTS]; q[P_PACKED] = p[M_CODES]; q[P_SCALES] = p[M_CODE_SCALES];
+    q[P_INTER] = p[M_INTER]; q[P_TASK_EXPERT] = p[M_TASK_EXPERT]; q[P_TASK_VALID] = p[M_TASK_VALID]; q[P_TILE_BASE] = p[M_TILE_BASE];
+    q[P_TOKEN_MAP] = p[M_TOKEN_MAP]; q[P_TOKEN_WEIGHTS] = p[M_TILE_WEIGHTS]; q[P_W13] = p[M_W13]; q[P_S13] = p[M_S13]; q[P_W2] = p[M_W2];
+    q[P_S2] = p[M_S2]; q[P_SCATTER] = p[M_OUT];
+    const int32_t scalars[S_DYN_COUNT] = {rows, rows, tiles * 16, tiles, 16, 1};
+    return launch_dynamic(c, false, q, scalars, s, 6, nullptr, nullptr, false, (float*)p[M_PROJ]);
 }
 // ---- entry 4: gemm.dense (FP8 x FP8 block-scaled -> BF16) -----------------------------------------------------------
 int launch_dense(const Context& c, const uint64_t* p, const int32_t* sc, hipStream_t s) {
@@ -410,6 +460,9 @@ const EntryShape kEntries[] = {
     {"moe.front_end", P_DYN_COUNT, S_DYN_COUNT},
     {"ffn.experts_with_shared", P_ROUTE_COUNT + H_COUNT - 2 + 2, S_ROUTE_COUNT + 1},
     {"integration.tp_moe.dynamic", P_DYN_COUNT, S_DYN_COUNT},      // input_format dual_quant_rows_v1
+    {"moe.w4a8.compact_micro", M_COUNT, 2},
+    {"gemm.mxfp8_quant_cute", 4, 3},
+    {"gemm.mxfp8_quant_cute", 4, 3},
 };
 constexpr int kEntryCount = sizeof(kEntries) / sizeof(kEntries[0]);
 
@@ -608,6 +661,9 @@ int32_t ca_primitives_launch(void* context, int32_t index, const uint64_t* point
             return launch_dynamic(c, pointers[P_LOGITS] != 0, pointers, scalars, s, 7, sh, output ? &sum : nullptr);
         }
         case 10: return launch_dynamic(c, false, pointers, scalars, s, 7, nullptr, nullptr, true);
+        case 11: return launch_micro(c, pointers, scalars, s);
+        case 12: return launch_quant_reference(c, pointers, scalars, s, false);
+        case 13: return launch_quant_reference(c, pointers, scalars, s, true);
         default: return -3;
     }
 }

@@ -164,6 +164,7 @@ struct StreamArgs {
     float limit;
     uint16_t* out;                   // FC1: BF16 intermediate [phys_row][inter]; FC2: BF16 [route or row][hidden]
     uint16_t* tap;                   // FC1 dense: BF16 projections [row][2 inter] before the activation, may be null
+    float* proj;                     // FC1 routed: FP32 projections [route][2 inter] (up, then gate) before the activation, may be null
     int table_tiles;                 // routed: capacity of the plan tables in tiles (phase kernels: at most TF_LDS_TILES)
 };
 // A workgroup walks the plan's tile table for every item; read in place that is three dependent round trips (tile count,
@@ -292,6 +293,11 @@ __device__ __forceinline__ void tf_fc1_items(const StreamArgs& p, int item_first
                         const float u = fminf(fmaxf(tf_bf16(ub), lo), hi);
                         value = __fmul_rn(g / __fadd_rn(1.0f, tf_exp(-g)), u);
                     } else {
+                        if (p.proj != nullptr) {
+                            float* at = p.proj + (size_t)p.token_map[row] * 2 * p.inter + 16 * r.j + (lane & 15);
+                            at[0] = first;
+                            at[p.inter] = second;
+                        }
                         const float g = fminf(second, p.limit);
                         const float u = fminf(p.limit, fmaxf(-p.limit, first));
                         value = __fmul_rn(__fmul_rn(g, tf_logistic(g)), u);
