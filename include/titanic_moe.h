@@ -56,6 +56,24 @@ int ca_router_logits_wide_in(void* context, int rows, const void* x, const void*
 int ca_shared_swiglu_in(void* context, int rows, const void* input, void* output, void* stream);
 int ca_ffn_add_in(void* context, int rows, const void* routed, const void* shared, void* out, void* stream);
 
+/* ---- the decoder's FFN boundary either side of the layer ------------------------------------------------------- */
+/* Upstream: the reference's boundary hands the layer its normalized BF16 input together with that input's MXFP8 codes, and
+ * the layer then skips its own quantizer (src/decoder.rs:1654-1656 -> Layer::run_quantized_input, src/ffn.rs:974-975,
+ * 1053-1065).  The reference's producer is an operator binary (src/mhc.rs:606-614); this one is an RMS norm with a BF16
+ * boundary: normed = bf16((x / sqrt(mean(x^2) + eps)) * weight), then both MXFP8 flavours of `normed` in the context's
+ * activation block width: codes / scales (zero block -> scale byte 0; the routed experts' input), codes_min / scales_min (amax
+ * floored at 1e-4; the shared expert's input); either pair may be null.  x, normed: [rows][hidden] BF16; weight: [hidden]
+ * BF16.  hidden <= 8,192. */
+int ca_ffn_norm_quant(void* context, int rows, const void* x, const void* weight, float eps, void* normed, void* codes, void* scales,
+                      void* codes_min, void* scales_min, void* stream);
+/* Downstream: the route sum and the shared addition (ca_ffn_sum_shared: src/ffn.rs:1041-1044) with the residual addition
+ * that follows the layer in the decoder (src/decoder.rs:1497-1543 `finish_ffn`) in the same pass: routed (rows < live) =
+ * ordered FP32 sum of the top-k route outputs rounded to BF16; ffn = bf16(routed + shared) (flush-to-zero add), written to
+ * ffn_out unless null; residual_out = bf16(f32(ffn) + f32(residual)) (may alias residual).  The reference's own boundary mixes
+ * several residual streams in an operator binary; this is the single-stream addition. */
+int ca_ffn_sum_residual(void* context, int rows, int live, const void* routes, const void* shared, const void* residual, void* routed,
+                        void* ffn_out, void* residual_out, void* stream);
+
 /* ---- kernels the reference resolves by name from a code module (src/cuda.rs:199-226 Module::function + launch) -- */
 /* Launches the `extern "C" __global__` kernel `name` with the reference's launch tuple ([grid;3], [block;3], dynamic
  * shared bytes, stream, argument pointers).  -3 for an unknown name.  The same kernels are in titanic_moe_gfx950.hsaco

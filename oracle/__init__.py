@@ -261,6 +261,20 @@ def ffn_sum_shared(routes, shared, live=None, previous=None):
     return routed, out
 
 
+def rmsnorm(x, weight, eps):
+    x, weight = _c(x, np.uint16), _c(weight, np.uint16)
+    out = np.empty_like(x)
+    lib().orc_rmsnorm(_p(x), _p(weight), _p(out), _i32(x.shape[0]), _i32(x.shape[1]), ctypes.c_float(eps))
+    return out
+
+
+def residual_add(a, b):
+    a, b = _c(a, np.uint16), _c(b, np.uint16)
+    out = np.empty_like(a)
+    lib().orc_residual_add(_p(a), _p(b), _p(out), _i64(a.size))
+    return out
+
+
 # ---- whole layer ------------------------------------------------------------------------------------------------------
 def layer(cfg, x, tokens, live, gate_w, bias, bias_alt, w13, s13, w2, s2, sh_w13, sh_s13, sh_w2, sh_s2, padding=None):
     """Runs the whole layer; returns a dict of every tap."""

@@ -98,6 +98,9 @@ void orc_topk_sum(const uint16_t* routes, uint16_t* routed, int32_t rows, int32_
 void orc_ffn_add(const uint16_t* a, const uint16_t* b, uint16_t* out, int64_t n);
 void orc_ffn_sum_shared(const uint16_t* routes, const uint16_t* shared, uint16_t* routed, uint16_t* out,
                         int32_t rows, int32_t topk, int32_t hidden, int32_t live);
+/* the decoder's FFN boundary either side of the layer: RMS norm with a BF16 boundary; BF16 residual addition */
+void orc_rmsnorm(const uint16_t* x, const uint16_t* weight, uint16_t* out, int32_t rows, int32_t cols, float eps);
+void orc_residual_add(const uint16_t* a, const uint16_t* b, uint16_t* out, int64_t n);
 
 /* ---- whole layer --------------------------------------------------------------------------- */
 typedef struct {

@@ -1,6 +1,7 @@
 // C ABI of libtitanic_moe_hip.so: the entry points the reference's Rust FFN operators bind (see include/titanic_moe.h).
 // Nothing here allocates, frees or synchronizes; every entry point only enqueues kernels on the caller's stream.
 #include "../../include/titanic_moe.h"
+#include "boundary.cuh"
 #include "codec.cuh"
 #include "combine.cuh"
 #include "experts_gemm.cuh"
@@ -478,6 +479,7 @@ const KernelName kKernels[] = {
     TF_KERNEL(ca_expert_scale_code1), TF_KERNEL(ca_expert_scale_code1_check), TF_KERNEL(ca_expert_scale_code1_census),
     TF_KERNEL(ca_expert_scale_codes4), TF_KERNEL(ca_router_logits_mfma), TF_KERNEL(ca_codec_encode), TF_KERNEL(ca_codec_decode),
     TF_KERNEL(ca_codec_pack_bf16), TF_KERNEL(ca_codec_unpack_routed), TF_KERNEL(ca_codec_local_live), TF_KERNEL(ca_convert_formats),
+    TF_KERNEL(ca_rmsnorm_quant), TF_KERNEL(ca_ffn_sum_shared_residual),
 };
 constexpr int kKernelCount = sizeof(kKernels) / sizeof(kKernels[0]);
 
@@ -544,6 +546,27 @@ int ca_shared_swiglu_in(void* context, int rows, const void* input, void* output
 }
 int ca_ffn_add_in(void* context, int rows, const void* routed, const void* shared, void* out, void* stream) {
     return context ? ffn_add_of(((const Context*)context)->g, rows, routed, shared, out, stream) : -1;
+}
+// ---- the decoder's FFN boundary either side of the layer (boundary.cuh) -------------------------------------------------
+int ca_ffn_norm_quant(void* context, int rows, const void* x, const void* weight, float eps, void* normed, void* codes, void* scales,
+                      void* codes_min, void* scales_min, void* stream) {
+    if (!context || !x || !weight || !normed || rows < 1 || (!codes != !scales) || (!codes_min != !scales_min) || !(eps >= 0.f)) return -1;
+    const ca_geometry& g = ((const Context*)context)->g;
+    if (g.hidden > 8192 || g.hidden % g.act_block) return -4;
+    ca_rmsnorm_quant<<<rows, 256, 0, (hipStream_t)stream>>>((const uint16_t*)x, (const uint16_t*)weight, (uint16_t*)normed, (uint8_t*)codes,
+                                                            (uint8_t*)scales, (uint8_t*)codes_min, (uint8_t*)scales_min, g.hidden, g.act_block, eps);
+    return launch_status();
+}
+int ca_ffn_sum_residual(void* context, int rows, int live, const void* routes, const void* shared, const void* residual, void* routed,
+                        void* ffn_out, void* residual_out, void* stream) {
+    if (!context || !routes || !shared || !residual || !routed || !residual_out || rows < 1 || live < 0) return -1;
+    const ca_geometry& g = ((const Context*)context)->g;
+    const long long n = (long long)rows * g.hidden;
+    if (n > 0x7fffffffll) return -1;
+    ca_ffn_sum_shared_residual<<<(int)((n / 8 + 255) / 256), 256, 0, (hipStream_t)stream>>>(
+        (const uint16_t*)routes, (const uint16_t*)shared, (const uint16_t*)residual, (uint16_t*)routed, (uint16_t*)ffn_out, (uint16_t*)residual_out,
+        (int)n, live < rows ? live : rows, g.topk, g.hidden);
+    return launch_status();
 }
 int ca_moe_nibble_permute(void* data, uint64_t bytes, int inverse, void* stream) {
     if (!data || bytes % 4 || (inverse != 0 && inverse != 1)) return -1;

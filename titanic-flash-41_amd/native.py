@@ -15,7 +15,8 @@ EXPORTS = ["ca_ffn_abi", "ca_ffn_configure", "ca_ffn_geometry", "ca_router_logit
            "ca_primitives_abi", "ca_primitives_open", "ca_primitives_close", "ca_primitives_launch", "ca_primitives_launch2",
            "ca_primitives_entries", "ca_primitives_scratch_bytes", "ca_primitives_marks", "ca_encode", "ca_decode", "ca_local_live",
            "ca_pack_bf16", "ca_primitives_spin_limit", "ca_primitives_open_geometry", "ca_primitives_geometry", "ca_router_logits_in",
-           "ca_router_logits_wide_in", "ca_shared_swiglu_in", "ca_ffn_add_in", "ca_moe_dynamic_static", "ca_moe_dynamic_static_capacity"]
+           "ca_router_logits_wide_in", "ca_shared_swiglu_in", "ca_ffn_add_in", "ca_moe_dynamic_static", "ca_moe_dynamic_static_capacity",
+           "ca_ffn_norm_quant", "ca_ffn_sum_residual"]
 
 
 class Geometry(ctypes.Structure):
@@ -87,6 +88,8 @@ def load():
     lib.ca_router_logits_wide_in.argtypes = [vp, ctypes.c_int, vp, vp, vp, vp]
     lib.ca_shared_swiglu_in.argtypes = [vp, ctypes.c_int, vp, vp, vp]
     lib.ca_ffn_add_in.argtypes = [vp, ctypes.c_int, vp, vp, vp, vp]
+    lib.ca_ffn_norm_quant.argtypes = [vp, ctypes.c_int, vp, vp, ctypes.c_float, vp, vp, vp, vp, vp, vp]
+    lib.ca_ffn_sum_residual.argtypes = [vp, ctypes.c_int, ctypes.c_int, vp, vp, vp, vp, vp, vp, vp]
     _lib = lib
     return lib
 
@@ -110,6 +113,16 @@ class _Arg:
             self.c = ctypes.c_void_p(0)
         else:  # torch tensor
             self.c = ctypes.c_void_p(value.data_ptr())
+
+
+def open_context(geometry):
+    """A context of the library with this geometry (ca_primitives_open_geometry); close it with ca_primitives_close."""
+    lib = load()
+    status = ctypes.c_int32(0)
+    ctx = lib.ca_primitives_open_geometry(ctypes.byref(geometry), ctypes.byref(status))
+    if not ctx or status.value != 0:
+        raise RuntimeError("ca_primitives_open_geometry failed: %d" % status.value)
+    return ctx
 
 
 def ptr(t):
