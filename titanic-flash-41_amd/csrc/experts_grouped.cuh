@@ -66,39 +66,43 @@ __device__ __forceinline__ void tf_mfma_settle(v4f (&acc)[8]) {
                  : "+v"(acc[0]), "+v"(acc[1]), "+v"(acc[2]), "+v"(acc[3]), "+v"(acc[4]), "+v"(acc[5]), "+v"(acc[6]), "+v"(acc[7]));
 }
 // Requests that may still be in flight at the barrier of k-step `u` of an unrolled round of four: those issued in the
-// LEAD - 1 k-steps before it.  Every k-step issues DATA requests, k-step EXTRA of a round two more (the next round's weight
+// LEAD - 1 k-steps before it.  Every k-step issues DATA requests, k-step EXTRA of a round MORE more (the next round's weight
 // scales).  Requests the count does not know (the next tasks' permutation map, stores) only make the wait stricter: it
 // lets the N youngest stay in flight, and whatever is younger than the k-step's own requests may.
-template <int LEAD, int DATA, int EXTRA>
+template <int LEAD, int DATA, int EXTRA, int MORE>
 constexpr int tf_loads_behind(int u) {
     int n = 0;
-    for (int j = 1; j < LEAD; ++j) n += DATA + (((u - j) & 3) == EXTRA ? 2 : 0);
+    for (int j = 1; j < LEAD; ++j) n += DATA + (((u - j) & 3) == EXTRA ? MORE : 0);
     return n;
 }
 
 template <int MODE, int BM, bool WORDS>
 __global__ void __launch_bounds__(512) tf_grouped_gemm(const GemmArgs p) {
     constexpr bool FC1 = MODE == TF_GEMM_FC1_ROUTED;
-    constexpr int NS = BM == 256 ? 3 : 4, LEAD = NS - 1;
+    constexpr int NG = BM == 256 ? 1 : 2;    // column groups a task: a 128-row unit takes two, so that a wave's products a k-step
+                                             // (and with them the k-step's fixed costs a product) are those of a 256-row unit
+    constexpr int NS = 3, LEAD = NS - 1;
     constexpr int NA = BM / 64;              // 16-byte pieces of the token tile a thread requests a k-step
     constexpr int NF = BM / 64;              // 16-row fragments of a wave (BM / 4 rows)
+    constexpr int NT = 8 * NG;               // weight tiles a wave multiplies its fragments with
+    constexpr int NB = 2 * NG;               // weight tiles a wave requests a k-step
     constexpr int WROWS = BM / 4;
-    constexpr int DATA = NA + 1 + 2;         // requests a wave issues a k-step: token pieces, token scales, two weight tiles
-    constexpr int A_STAGE = BM * 128, B_STAGE = 16 * 1024;
+    constexpr int DATA = NA + 1 + NB;        // requests a wave issues a k-step: token pieces, token scales, weight tiles
+    constexpr int A_STAGE = BM * 128, B_STAGE = 16 * 1024 * NG;
     constexpr int ROW_WAVES = BM / 64;       // waves whose 64 lanes cover the tile's rows once; the other waves repeat them
     __shared__ __attribute__((aligned(1024))) uint8_t s_a[NS * A_STAGE];
     __shared__ __attribute__((aligned(1024))) uint8_t s_b[NS * B_STAGE];
     __shared__ __attribute__((aligned(256))) uint32_t s_asc[NS][BM];
-    __shared__ __attribute__((aligned(256))) uint32_t s_bsc[16 * 64];
+    __shared__ __attribute__((aligned(256))) uint32_t s_bsc[16 * NG * 64];
     __shared__ __attribute__((aligned(256))) int32_t s_src[3][BM];   // the permutation map's entry (route index) of each tile row, for three tasks in turn
-    __shared__ __attribute__((aligned(256))) float s_wgt[3][BM];     // FC2: routing weight of each tile row; FC1: row maxima of the two column halves
+    __shared__ __attribute__((aligned(256))) float s_wgt[NG == 2 ? 4 : 3][BM];   // FC2: routing weight of each tile row (three tasks in turn); FC1: row maxima of the column halves
     __shared__ uint16_t s_ubase[BM == 256 ? 514 : 2], s_tbase[BM == 256 ? 514 : 2];
     __shared__ int32_t s_part[8];
 
     const int tid = threadIdx.x, lane = tid & 63, wave = __builtin_amdgcn_readfirstlane(tid >> 6);
     const int wm = wave >> 1, wn = wave & 1, g = lane >> 4, r16 = lane & 15;
     const int KS = p.k / 128, scales_row = p.k / p.act_block;
-    const int groups = FC1 ? p.inter / 128 : p.hidden / 256;
+    const int groups = (FC1 ? p.inter / 128 : p.hidden / 256) / NG;          // a task's column groups: ng NG .. ng NG + NG - 1
     const int total_tiles = p.expert_tile_base[p.experts];
     int units = total_tiles;
     if constexpr (BM == 256) {
@@ -166,8 +170,8 @@ __global__ void __launch_bounds__(512) tf_grouped_gemm(const GemmArgs p) {
     // 32-bit byte offset, which stays the same for a whole task.
     struct Source {
         uint32_t a_off[NA], asc_off;
-        const uint8_t* b_base[2];
-        const uint8_t* bsc_base[2];
+        const uint8_t* b_base[NB];
+        const uint8_t* bsc_base[NB];
     };
     const uint32_t lds_a = tf_lds_addr(s_a), lds_b = tf_lds_addr(s_b), lds_asc = tf_lds_addr(&s_asc[0][0]), lds_bsc = tf_lds_addr(s_bsc);
     // The task's slot has landed and is visible (a wait for the requests and a barrier lie between its request and this).
@@ -187,21 +191,21 @@ __global__ void __launch_bounds__(512) tf_grouped_gemm(const GemmArgs p) {
         const uint8_t* w = p.w + (size_t)expert * p.w_expert_stride;
         const uint8_t* ws = p.ws + (size_t)expert * p.ws_expert_stride;
 #pragma unroll
-        for (int c = 0; c < 2; ++c) {
-            const int T = wave * 2 + c;
-            const int ntile = FC1 ? (T < 8 ? ng * 8 + T : p.inter / 16 + ng * 8 + T - 8) : ng * 16 + T;
+        for (int c = 0; c < NB; ++c) {
+            const int T = (wave * NB + c) & 15, cg = ng * NG + (wave * NB + c) / 16;       // tile within its column group, the group
+            const int ntile = FC1 ? (T < 8 ? cg * 8 + T : p.inter / 16 + cg * 8 + T - 8) : cg * 16 + T;
             src.b_base[c] = w + (size_t)ntile * KS * 1024;
             src.bsc_base[c] = ws + (size_t)ntile * (p.k / 512) * 256;
         }
     };
     const uint32_t lane16 = lane * 16, lane4 = lane * 4;
-    // Request `op` of k-step `ks` of a task into ring stage `stage`: ops [0, NA): token pieces, NA: token scales, NA + 1, NA + 2:
-    // weight tiles; ops DATA, DATA + 1: the weight scales of round `ks / 4` (four k-steps a word).
+    // Request `op` of k-step `ks` of a task into ring stage `stage`: ops [0, NA): token pieces, NA: token scales, then NB weight
+    // tiles; ops DATA .. DATA + NB - 1: those tiles' scales of round `ks / 4` (four k-steps a word).
     auto issue_op = [&](const Source& src, int op, int ks, int stage) {
         if (op < NA) tf_dma16(p.a_codes + (size_t)ks * 128, src.a_off[op], lds_a + stage * A_STAGE + (wave * NA + op) * 1024);
         else if (op == NA) tf_dma4(p.a_scales + (WORDS ? (ks >> 2) * 4 : ks * 4), src.asc_off, lds_asc + stage * (BM * 4) + (wave & (ROW_WAVES - 1)) * 256);
-        else if (op < DATA) tf_dma16(src.b_base[op - NA - 1] + (size_t)ks * 1024, lane16, lds_b + stage * B_STAGE + (wave * 2 + op - NA - 1) * 1024);
-        else tf_dma4(src.bsc_base[op - DATA] + (size_t)(ks >> 2) * 256, lane4, lds_bsc + (wave * 2 + op - DATA) * 256);
+        else if (op < DATA) tf_dma16(src.b_base[op - NA - 1] + (size_t)ks * 1024, lane16, lds_b + stage * B_STAGE + (wave * NB + op - NA - 1) * 1024);
+        else tf_dma4(src.bsc_base[op - DATA] + (size_t)(ks >> 2) * 256, lane4, lds_bsc + (wave * NB + op - DATA) * 256);
     };
 
     // ---- this lane's fragment addresses ----------------------------------------------------------------------------------
@@ -225,7 +229,7 @@ __global__ void __launch_bounds__(512) tf_grouped_gemm(const GemmArgs p) {
     tf_lds_barrier();
     install(now, cur, 0);
 #pragma unroll
-    for (int c = 0; c < 2; ++c) issue_op(now, DATA + c, 0, 0);
+    for (int c = 0; c < NB; ++c) issue_op(now, DATA + c, 0, 0);
 #pragma unroll
     for (int d = 0; d < LEAD; ++d)
 #pragma unroll
@@ -249,14 +253,14 @@ __global__ void __launch_bounds__(512) tf_grouped_gemm(const GemmArgs p) {
         // whatever its count.
         auto run_task = [&](auto frags_constant) {
             constexpr int FR = decltype(frags_constant)::value, FRA = FR > 0 ? FR : 1;
-            v4f acc[FRA][8];
+            v4f acc[FRA][NT];
 #pragma unroll
             for (int f = 0; f < FRA; ++f)
 #pragma unroll
-                for (int t = 0; t < 8; ++t) acc[f][t] = v4f{0.f, 0.f, 0.f, 0.f};
-            uint32_t bsc[8];
+                for (int t = 0; t < NT; ++t) acc[f][t] = v4f{0.f, 0.f, 0.f, 0.f};
+            uint32_t bsc[NT];
 #pragma unroll
-            for (int t = 0; t < 8; ++t) bsc[t] = 0;
+            for (int t = 0; t < NT; ++t) bsc[t] = 0;
             // One k-step.  FIRST / LAST: in the task's first / last round of four.  The requests of k-step ks + LEAD (the next
             // task's first k-steps in the last round: the ring runs on across tasks) are issued between the fragments' products,
             // so that their address arithmetic runs under the matrix pipeline.
@@ -270,7 +274,7 @@ __global__ void __launch_bounds__(512) tf_grouped_gemm(const GemmArgs p) {
                 // requests its share of k-step b + LEAD into it: the early waves in k-step b, the late waves in the second half
                 // of their k-step b - 1.  A task's first k-steps landed before the previous task's stores went out (below).
                 if (!late) {
-                    if constexpr (!FIRST || u >= LEAD) tf_wait_vm<tf_loads_behind<LEAD, DATA, 1>(u)>();
+                    if constexpr (!FIRST || u >= LEAD) tf_wait_vm<tf_loads_behind<LEAD, DATA, 1, NB>(u)>();
                     __builtin_amdgcn_s_barrier();
                 }
                 asm volatile("" ::: "memory");
@@ -288,7 +292,7 @@ __global__ void __launch_bounds__(512) tf_grouped_gemm(const GemmArgs p) {
                     const int stage = AHEAD == LEAD ? ps : (ps + 1 == NS ? 0 : ps + 1);
                     if constexpr (EXTRA) {
 #pragma unroll
-                        for (int i = 0; i < 2; ++i) issue_op(LAST ? then : now, DATA + i, LAST ? 0 : ks + 4 - u, 0);
+                        for (int i = 0; i < NB; ++i) issue_op(LAST ? then : now, DATA + i, LAST ? 0 : ks + 4 - u, 0);
                     }
 #pragma unroll
                     for (int i = 0; i < DATA; ++i) issue_op(from, i, ks_ahead, stage);
@@ -302,7 +306,7 @@ __global__ void __launch_bounds__(512) tf_grouped_gemm(const GemmArgs p) {
                         // the late waves' share of the next k-step's stage (the next task's first, after a task's last k-step);
                         // what they requested for the task's first LEAD + 1 k-steps landed before their last stores
                         constexpr bool WAIT = u == 3 || !(FIRST && u + 1 <= LEAD);
-                        if constexpr (WAIT) tf_wait_vm<tf_loads_behind<LEAD, DATA, 0>(u)>();
+                        if constexpr (WAIT) tf_wait_vm<tf_loads_behind<LEAD, DATA, 0, NB>(u)>();
                         asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory");      // this k-step's last reads of its stage have returned
                         __builtin_amdgcn_s_barrier();
                         asm volatile("" ::: "memory");
@@ -314,7 +318,49 @@ __global__ void __launch_bounds__(512) tf_grouped_gemm(const GemmArgs p) {
                     if (!late) issue_range(early_ahead, early_extra);
                     middle();
                 }
-                if constexpr (FR > 0) {
+                if constexpr (FR > 0 && NG == 2) {
+                    // Two column groups: the wave's (at most two) token fragments stay in registers for the whole k-step and
+                    // the weights pass in four blocks of four tiles (group, then "up" / "gate" or lower / upper half), the next
+                    // block leaving LDS under the current block's products.  The late waves' barrier stands before the last
+                    // block's products: every read of the stage has been issued a block earlier.
+                    const uint8_t* sa = s_a + cs * A_STAGE;
+                    const uint8_t* sb = s_b + cs * B_STAGE + lane16;
+                    const uint32_t* sc = &s_asc[cs][wm * WROWS + r16];
+                    auto block_at = [&](int b) constexpr { return ((b >> 1) * 16 + (FC1 ? ((b & 1) ? 8 + 4 * wn : 4 * wn) : 8 * wn + 4 * (b & 1))) * 1024; };
+                    u4v bf[2][4];
+#pragma unroll
+                    for (int t = 0; t < 4; ++t) bf[0][t] = *reinterpret_cast<const u4v*>(sb + block_at(0) + t * 1024);
+                    if constexpr (u == 0) {
+#pragma unroll
+                        for (int b = 0; b < 4; ++b)
+#pragma unroll
+                            for (int t = 0; t < 4; ++t) bsc[b * 4 + t] = s_bsc[block_at(b) / 16 + t * 64 + lane];
+                    }
+                    v8i av[FR];
+                    uint32_t sca[FR];
+#pragma unroll
+                    for (int f = 0; f < FR; ++f) {
+                        const u4v l = *reinterpret_cast<const u4v*>(sa + a_lo + f * 2048), h = *reinterpret_cast<const u4v*>(sa + a_hi + f * 2048);
+                        av[f] = v8i{(int)l[0], (int)l[1], (int)l[2], (int)l[3], (int)h[0], (int)h[1], (int)h[2], (int)h[3]};
+                        sca[f] = WORDS ? sc[f * 16] : sc[f * 16] >> (8 * g);
+                    }
+                    constexpr int SEL = WORDS ? u : 0;
+#pragma unroll
+                    for (int b = 0; b < 4; ++b) {
+                        if (b == 3) middle();
+                        if (b + 1 < 4) {
+#pragma unroll
+                            for (int t = 0; t < 4; ++t) bf[(b + 1) & 1][t] = *reinterpret_cast<const u4v*>(sb + block_at(b + 1) + t * 1024);
+                        }
+#pragma unroll
+                        for (int f = 0; f < FR; ++f)
+#pragma unroll
+                            for (int t = 0; t < 4; ++t) tf_mfma_weights_first<u, SEL>(acc[f][b * 4 + t], bf[b & 1][t], av[f], bsc[b * 4 + t], sca[f]);
+                        if (b == 0) { if (!late) issue_range(early_ahead, early_extra); }
+                        __builtin_amdgcn_sched_barrier(0);
+                    }
+                }
+                if constexpr (FR > 0 && NG == 1) {
                     const uint8_t* sa = s_a + cs * A_STAGE;
                     const uint8_t* sb = s_b + cs * B_STAGE + b_first * 1024 + lane16;
                     const uint32_t* sc = &s_asc[cs][wm * WROWS + r16];
@@ -382,101 +428,107 @@ __global__ void __launch_bounds__(512) tf_grouped_gemm(const GemmArgs p) {
                 round(std::false_type{}, std::true_type{}, KS - 4);
             }
 #pragma unroll
-            for (int f = 0; f < FR; ++f) tf_mfma_settle(acc[f]);
+            for (int f = 0; f < FR; ++f)
+#pragma unroll
+                for (int gi = 0; gi < NG; ++gi) tf_mfma_settle(*reinterpret_cast<v4f (*)[8]>(&acc[f][gi * 8]));
 
             // ---- epilogue: values first, then a wait for every request in flight (the next task's first k-steps, long landed
             // by now: its first LEAD k-steps then wait for nothing, in particular not for the stores below), then the stores ---
             // Lane (g, r16) of product (f, t) holds tile row wm WROWS + 16 f + r16 and the four consecutive columns 4 g + i of
-            // weight tile t.
-            if constexpr (FC1) {
-                // t < 4: "up" tiles, t >= 4: the "gate" tiles of the same columns 64 wn + 16 (t % 4) + 4 g + i of the group
-                float hv[FRA][4][4];
-                float amax[FRA][2];
-                uint32_t codes[FRA][4], exponent[FRA][2];
-                float (*s_max)[BM] = s_wgt;          // [wn][row]: FC1 keeps no routing weights here
+            // weight tile t of column group `cg`; the task's column groups one after the other.
 #pragma unroll
-                for (int f = 0; f < FR; ++f) {
+            for (int gi = 0; gi < NG; ++gi) {
+                const int cg = ng * NG + gi;
+                if constexpr (FC1) {
+                    // t < 4: "up" tiles, t >= 4: the "gate" tiles of the same columns 64 wn + 16 (t % 4) + 4 g + i of the group
+                    float hv[FRA][4][4];
+                    float amax[FRA][2];
+                    uint32_t codes[FRA][4], exponent[FRA][2];
+                    float (*s_max)[BM] = s_wgt + 2 * gi;          // [wn][row]: FC1 keeps no routing weights here
 #pragma unroll
-                    for (int j = 0; j < 4; ++j)
+                    for (int f = 0; f < FR; ++f) {
 #pragma unroll
-                        for (int i = 0; i < 4; ++i) {
-                            const float gv = fminf(acc[f][4 + j][i], p.limit), uv = fminf(p.limit, fmaxf(-p.limit, acc[f][j][i]));
-                            hv[f][j][i] = tf_bf16(tf_to_bf16(__fmul_rn(__fmul_rn(gv, tf_logistic_fast(gv)), uv)));
+                        for (int j = 0; j < 4; ++j)
+#pragma unroll
+                            for (int i = 0; i < 4; ++i) {
+                                const float gv = fminf(acc[f][gi * 8 + 4 + j][i], p.limit), uv = fminf(p.limit, fmaxf(-p.limit, acc[f][gi * 8 + j][i]));
+                                hv[f][j][i] = tf_bf16(tf_to_bf16(__fmul_rn(__fmul_rn(gv, tf_logistic_fast(gv)), uv)));
+                            }
+#pragma unroll
+                        for (int b = 0; b < 2; ++b) {
+                            float m = 0.f;
+#pragma unroll
+                            for (int j = 2 * b; j < 2 * b + 2; ++j)
+#pragma unroll
+                                for (int i = 0; i < 4; ++i) m = fmaxf(m, fabsf(hv[f][j][i]));
+                            m = fmaxf(m, __shfl_xor(m, 16));
+                            amax[f][b] = fmaxf(m, __shfl_xor(m, 32));       // over the 32 columns of weight tiles 2 b, 2 b + 1
                         }
-#pragma unroll
-                    for (int b = 0; b < 2; ++b) {
-                        float m = 0.f;
-#pragma unroll
-                        for (int j = 2 * b; j < 2 * b + 2; ++j)
-#pragma unroll
-                            for (int i = 0; i < 4; ++i) m = fmaxf(m, fabsf(hv[f][j][i]));
-                        m = fmaxf(m, __shfl_xor(m, 16));
-                        amax[f][b] = fmaxf(m, __shfl_xor(m, 32));       // over the 32 columns of weight tiles 2 b, 2 b + 1
                     }
-                }
-                if constexpr (WORDS) {               // one scale a row and 128 columns: both column halves (waves wn = 0, 1)
+                    if constexpr (WORDS) {               // one scale a row and 128 columns: both column halves (waves wn = 0, 1)
 #pragma unroll
-                    for (int f = 0; f < FR; ++f) if (g == 0) s_max[wn][wm * WROWS + 16 * f + r16] = fmaxf(amax[f][0], amax[f][1]);
-                    tf_lds_barrier();
+                        for (int f = 0; f < FR; ++f) if (g == 0) s_max[wn][wm * WROWS + 16 * f + r16] = fmaxf(amax[f][0], amax[f][1]);
+                        tf_lds_barrier();
+#pragma unroll
+                        for (int f = 0; f < FR; ++f) {
+                            const int row = wm * WROWS + 16 * f + r16;
+                            amax[f][0] = amax[f][1] = fmaxf(s_max[0][row], s_max[1][row]);
+                        }
+                    }
+#pragma unroll
+                    for (int f = 0; f < FR; ++f)
+#pragma unroll
+                        for (int b = 0; b < 2; ++b) {
+                            exponent[f][b] = tf_block_exponent(amax[f][b]);
+                            const float inv = tf_block_inverse(exponent[f][b]);
+#pragma unroll
+                            for (int j = 2 * b; j < 2 * b + 2; ++j)
+                                codes[f][j] = tf_pack_e4m3(__fmul_rn(hv[f][j][0], inv), __fmul_rn(hv[f][j][1], inv), __fmul_rn(hv[f][j][2], inv), __fmul_rn(hv[f][j][3], inv));
+                        }
+                    if (gi == 0) tf_wait_vm<0>();
 #pragma unroll
                     for (int f = 0; f < FR; ++f) {
                         const int row = wm * WROWS + 16 * f + r16;
-                        amax[f][0] = amax[f][1] = fmaxf(s_max[0][row], s_max[1][row]);
-                    }
-                }
+                        if (row < rows) {
+                            const size_t phys = (size_t)first_tile * 128 + row;
 #pragma unroll
-                for (int f = 0; f < FR; ++f)
-#pragma unroll
-                    for (int b = 0; b < 2; ++b) {
-                        exponent[f][b] = tf_block_exponent(amax[f][b]);
-                        const float inv = tf_block_inverse(exponent[f][b]);
-#pragma unroll
-                        for (int j = 2 * b; j < 2 * b + 2; ++j)
-                            codes[f][j] = tf_pack_e4m3(__fmul_rn(hv[f][j][0], inv), __fmul_rn(hv[f][j][1], inv), __fmul_rn(hv[f][j][2], inv), __fmul_rn(hv[f][j][3], inv));
-                    }
-                tf_wait_vm<0>();
-#pragma unroll
-                for (int f = 0; f < FR; ++f) {
-                    const int row = wm * WROWS + 16 * f + r16;
-                    if (row < rows) {
-                        const size_t phys = (size_t)first_tile * 128 + row;
-#pragma unroll
-                        for (int j = 0; j < 4; ++j) {
-                            const int col = ng * 128 + wn * 64 + j * 16 + 4 * g;
-                            *reinterpret_cast<uint32_t*>(p.h_codes + phys * p.inter + col) = codes[f][j];
-                            if (p.h_bf16 != nullptr)
-                                *reinterpret_cast<u2v*>(p.h_bf16 + phys * p.inter + col) = u2v{tf_pack_bf16(hv[f][j][0], hv[f][j][1]), tf_pack_bf16(hv[f][j][2], hv[f][j][3])};
-                        }
-                        if (g == 0) {
-                            if constexpr (WORDS) { if (wn == 0) p.h_scales[phys * (p.inter / 128) + ng] = (uint8_t)exponent[f][0]; }
-                            else {
-                                p.h_scales[phys * (p.inter / 32) + ng * 4 + wn * 2] = (uint8_t)exponent[f][0];
-                                p.h_scales[phys * (p.inter / 32) + ng * 4 + wn * 2 + 1] = (uint8_t)exponent[f][1];
+                            for (int j = 0; j < 4; ++j) {
+                                const int col = cg * 128 + wn * 64 + j * 16 + 4 * g;
+                                *reinterpret_cast<uint32_t*>(p.h_codes + phys * p.inter + col) = codes[f][j];
+                                if (p.h_bf16 != nullptr)
+                                    *reinterpret_cast<u2v*>(p.h_bf16 + phys * p.inter + col) = u2v{tf_pack_bf16(hv[f][j][0], hv[f][j][1]), tf_pack_bf16(hv[f][j][2], hv[f][j][3])};
+                            }
+                            if (g == 0) {
+                                if constexpr (WORDS) { if (wn == 0) p.h_scales[phys * (p.inter / 128) + cg] = (uint8_t)exponent[f][0]; }
+                                else {
+                                    p.h_scales[phys * (p.inter / 32) + cg * 4 + wn * 2] = (uint8_t)exponent[f][0];
+                                    p.h_scales[phys * (p.inter / 32) + cg * 4 + wn * 2 + 1] = (uint8_t)exponent[f][1];
+                                }
                             }
                         }
                     }
-                }
-            } else {
-                // output columns 256 ng + 128 wn + 16 t + 4 g + i of the row's route, scaled by its routing weight
-                u2v packed[FRA][8];
-                size_t out_at[FRA];
+                } else {
+                    // output columns 256 cg + 128 wn + 16 t + 4 g + i of the row's route, scaled by its routing weight
+                    u2v packed[FRA][8];
+                    size_t out_at[FRA];
 #pragma unroll
-                for (int f = 0; f < FR; ++f) {
-                    const int row = min(wm * WROWS + 16 * f + r16, BM - 1);
-                    const float share = s_wgt[slot][row];
-                    out_at[f] = (size_t)s_src[slot][row] * p.hidden + ng * 256 + wn * 128 + 4 * g;
+                    for (int f = 0; f < FR; ++f) {
+                        const int row = min(wm * WROWS + 16 * f + r16, BM - 1);
+                        const float share = s_wgt[slot][row];
+                        out_at[f] = (size_t)s_src[slot][row] * p.hidden + cg * 256 + wn * 128 + 4 * g;
 #pragma unroll
-                    for (int t = 0; t < 8; ++t)
-                        packed[f][t] = u2v{tf_pack_bf16(__fmul_rn(acc[f][t][0], share), __fmul_rn(acc[f][t][1], share)),
-                                           tf_pack_bf16(__fmul_rn(acc[f][t][2], share), __fmul_rn(acc[f][t][3], share))};
-                }
-                tf_wait_vm<0>();
-#pragma unroll
-                for (int f = 0; f < FR; ++f)
-                    if (wm * WROWS + 16 * f + r16 < rows) {
-#pragma unroll
-                        for (int t = 0; t < 8; ++t) *reinterpret_cast<u2v*>(p.out + out_at[f] + 16 * t) = packed[f][t];
+                        for (int t = 0; t < 8; ++t)
+                            packed[f][t] = u2v{tf_pack_bf16(__fmul_rn(acc[f][gi * 8 + t][0], share), __fmul_rn(acc[f][gi * 8 + t][1], share)),
+                                               tf_pack_bf16(__fmul_rn(acc[f][gi * 8 + t][2], share), __fmul_rn(acc[f][gi * 8 + t][3], share))};
                     }
+                    if (gi == 0) tf_wait_vm<0>();
+#pragma unroll
+                    for (int f = 0; f < FR; ++f)
+                        if (wm * WROWS + 16 * f + r16 < rows) {
+#pragma unroll
+                            for (int t = 0; t < 8; ++t) *reinterpret_cast<u2v*>(p.out + out_at[f] + 16 * t) = packed[f][t];
+                        }
+                }
             }
             if constexpr (FR == 0) tf_wait_vm<0>();
         };
@@ -496,7 +548,7 @@ __global__ void __launch_bounds__(512) tf_grouped_gemm(const GemmArgs p) {
 // expert in the unit prefix), whole column groups.
 inline bool tf_grouped_shape_ok(const GemmArgs& a, bool fc1) {
     return a.k >= 512 && a.k % 512 == 0 && (a.act_block == 32 || a.act_block == 128) && a.experts <= 512 &&
-           (fc1 ? (a.inter >= 128 && a.inter % 128 == 0) : (a.hidden >= 256 && a.hidden % 256 == 0));
+           (fc1 ? (a.inter >= 256 && a.inter % 256 == 0) : (a.hidden >= 512 && a.hidden % 512 == 0));
 }
 // `routes`: rows x top-k of the launch; experts with about two plan tiles or more on average run 256-row units.
 template <int MODE>
