@@ -1,6 +1,6 @@
 """Profiler runs of the layer, and the counter file the benchmark reads its measured HBM traffic from.
 
-    python -m titanic-flash-41_amd.counters run   [--out DIR] [--workloads c2,c3,c4,c5] [--shader]
+    python -m titanic-flash-41_amd.counters run   --out DIR [--workloads c2,c3,c4,c5] [--shader]
     python -m titanic-flash-41_amd.counters stamp DIR [--to profiles/counters.json]
 
 `run` needs a GPU.  For every workload it starts rocprofv3 on the stand-alone layer driver (tf_layer_probe: the benchmark
@@ -186,7 +186,7 @@ def main():
     ap = argparse.ArgumentParser()
     sub = ap.add_subparsers(dest="what", required=True)
     r = sub.add_parser("run")
-    r.add_argument("--out", default=os.path.join(ROOT, "gpurun_out", "counters"))
+    r.add_argument("--out", required=True, help="directory for the raw profiler output")
     r.add_argument("--workloads", default="c2,c3,c4,c5")
     r.add_argument("--shader", action="store_true")
     s = sub.add_parser("stamp")
