@@ -97,7 +97,8 @@ __global__ void __launch_bounds__(512) tf_grouped_gemm(const GemmArgs p) {
     __shared__ __attribute__((aligned(256))) int32_t s_src[3][BM];   // the permutation map's entry (route index) of each tile row, for three tasks in turn
     __shared__ __attribute__((aligned(256))) float s_wgt[NG == 2 ? 4 : 3][BM];   // FC2: routing weight of each tile row (three tasks in turn); FC1: row maxima of the column halves
     __shared__ uint16_t s_ubase[BM == 256 ? 514 : 2], s_tbase[BM == 256 ? 514 : 2];
-    __shared__ int32_t s_part[8];
+    __shared__ int32_t s_part[8], s_cpart[8], s_bound[9];
+    uint16_t* s_cbase = reinterpret_cast<uint16_t*>(s_a);      // prefix of the units' costs: needed before the ring starts only
 
     const int tid = threadIdx.x, lane = tid & 63, wave = __builtin_amdgcn_readfirstlane(tid >> 6);
     const int wm = wave >> 1, wn = wave & 1, g = lane >> 4, r16 = lane & 15;
@@ -105,29 +106,55 @@ __global__ void __launch_bounds__(512) tf_grouped_gemm(const GemmArgs p) {
     const int groups = (FC1 ? p.inter / 128 : p.hidden / 256) / NG;          // a task's column groups: ng NG .. ng NG + NG - 1
     const int total_tiles = p.expert_tile_base[p.experts];
     int units = total_tiles;
+    const int xcd = blockIdx.x & 7, local = blockIdx.x >> 3, local_count = gridDim.x >> 3;
+    int u_lo, u_hi;
     if constexpr (BM == 256) {
-        // units of two plan tiles: per expert ceil(tiles / 2); exclusive prefix over the experts (one thread an expert)
+        // units of two plan tiles: per expert ceil(tiles / 2); exclusive prefix over the experts (one thread an expert).  Beside
+        // it a prefix of what the units cost: a unit with more than 128 rows keeps both waves of every SIMD multiplying (5), one
+        // with fewer rows one wave a SIMD (3; up to 32 rows: half of that wave's fragments, 2).  The experts come in no
+        // particular order of size, and where they come sorted (popular experts first) equal counts of units an XCD would leave
+        // the XCDs with the small experts idle for a third of the launch: the XCDs take equal shares of the cost.
         const int e = tid;
         int tb = 0, tn = 0;
         if (e < p.experts) { tb = p.expert_tile_base[e]; tn = p.expert_tile_base[e + 1]; }
         const int mine = (tn - tb + 1) >> 1;
-        int prefix = mine;
+        int cost = 0;
+        if (mine > 0) {
+            const int last_rows = (tn - tb - 1) * 128 + p.task_valid_rows[(size_t)(tn - 1) * p.groups] - 256 * (mine - 1);
+            cost = 5 * (mine - 1) + (last_rows > 128 ? 5 : last_rows > 32 ? 3 : 2);
+        }
+        int prefix = mine, cprefix = cost;
 #pragma unroll
         for (int o = 1; o < 64; o <<= 1) {
-            const int below = __shfl_up(prefix, o);
-            if (lane >= o) prefix += below;
+            const int below = __shfl_up(prefix, o), cbelow = __shfl_up(cprefix, o);
+            if (lane >= o) { prefix += below; cprefix += cbelow; }
         }
-        if (lane == 63) s_part[wave] = prefix;
+        if (lane == 63) { s_part[wave] = prefix; s_cpart[wave] = cprefix; }
         __syncthreads();
-        for (int w = 0; w < wave; ++w) prefix += s_part[w];
-        if (e < p.experts) { s_ubase[e + 1] = (uint16_t)prefix; s_tbase[e] = (uint16_t)tb; }
+        for (int w = 0; w < wave; ++w) { prefix += s_part[w]; cprefix += s_cpart[w]; }
+        if (e < p.experts) { s_ubase[e + 1] = (uint16_t)prefix; s_tbase[e] = (uint16_t)tb; s_cbase[e + 1] = (uint16_t)cprefix; }
         if (e == p.experts - 1) s_tbase[e + 1] = (uint16_t)tn;
-        if (e == 0) s_ubase[0] = 0;
+        if (e == 0) { s_ubase[0] = 0; s_cbase[0] = 0; }
         __syncthreads();
         units = s_ubase[p.experts];
+        if (tid <= 8) {             // boundary tid of the XCDs' shares: the first unit at or behind tid eighths of the cost
+            const int total_cost = s_cbase[p.experts], target = (int)((long long)total_cost * tid / 8);
+            int lo = 0, hi = p.experts;                     // the expert with s_cbase[lo] <= target < s_cbase[lo + 1]
+            while (hi - lo > 1) {
+                const int mid = (lo + hi) >> 1;
+                if ((int)s_cbase[mid] <= target) lo = mid; else hi = mid;
+            }
+            const int in_expert = (int)s_ubase[lo + 1] - (int)s_ubase[lo];
+            const int bound = tid == 8 ? units : min((int)s_ubase[lo] + min((target - (int)s_cbase[lo]) / 5, in_expert), units);
+            s_bound[tid] = tid == 0 ? 0 : bound;
+        }
+        __syncthreads();
+        u_lo = s_bound[xcd];
+        u_hi = s_bound[xcd + 1];
+    } else {
+        u_lo = (int)((long long)units * xcd / 8);
+        u_hi = (int)((long long)units * (xcd + 1) / 8);
     }
-    const int xcd = blockIdx.x & 7, local = blockIdx.x >> 3, local_count = gridDim.x >> 3;
-    const int u_lo = (int)((long long)units * xcd / 8), u_hi = (int)((long long)units * (xcd + 1) / 8);
     const int my_tasks = (u_hi - u_lo) * groups;
     if (local >= my_tasks) return;
 
