@@ -1,29 +1,34 @@
 // Many-row (prefill) routed-expert projections: grouped GEMM with both operands streamed into LDS by the memory system.
 //
-// One task = one unit of an expert's physical rows (BM = 128: one plan tile; BM = 256: two consecutive plan tiles of the
-// same expert) x one column group (FC1: 128 intermediate columns = 128 "up" + 128 "gate" weight rows; FC2: 256 output
-// columns).  A workgroup of eight waves (two a SIMD) keeps a BM x 256 accumulator: wave (wm, wn) holds token rows
-// [wm BM/4, +BM/4) against weight rows [128 wn, +128) of the group, i.e. BM/64 x 8 products of
+// One task = one unit of an expert's physical rows x its column groups.  BM = 256: a unit is two consecutive plan tiles of
+// the same expert and a task takes one column group (FC1: 128 intermediate columns = 128 "up" + 128 "gate" weight rows;
+// FC2: 256 output columns).  BM = 128: a unit is one plan tile and a task takes two column groups, so that a wave's
+// products a k-step are the same in both.  A workgroup of eight waves (two a SIMD): wave (wm, wn) holds token rows
+// [wm BM/4, +BM/4) against weight rows [128 wn, +128) of each of the task's groups, i.e. 32 products of
 // v_mfma_scale_f32_16x16x128_f8f6f4 a k-step of 128.
 //
 // No operand of the main loop passes through vector registers on its way in: token codes (E4M3, gathered through the
 // permutation map), their UE8M0 scales, the prepared FP4 weights and their scales are written into LDS by
-// global_load_lds (16 or 4 bytes a lane, a wave's 64 lanes land at consecutive LDS addresses), LEAD k-steps ahead of
-// their use, in a ring of LEAD + 1 stages.  The loads are issued from inline assembly, so the compiler's own wait
+// global_load_lds (16 or 4 bytes a lane, a wave's 64 lanes land at consecutive LDS addresses), two k-steps ahead of
+// their use, in a ring of three stages.  The loads are issued from inline assembly, so the compiler's own wait
 // insertion does not know them (it would wait for every load in flight before each LDS read); the kernel counts them
-// itself: loads complete in issue order, every wave issues the same number of them in every k-step, and the wait at the
-// top of a k-step allows exactly the loads issued after that k-step's own to stay in flight.  One barrier a k-step
-// then makes every wave's share of the stage visible to all and frees the stage that was read a k-step ago.
+// itself: loads complete in issue order, every wave issues the same number of them in every k-step, and a wait allows
+// exactly the loads issued after the needed ones to stay in flight.
+//
+// The two waves of a SIMD run half a k-step apart (waves 0 - 3 "early", 4 - 7 "late"): a wave passes one barrier a k-step,
+// the early waves at its top, the late waves in its middle.  Behind a barrier the next stage is whole and the previous
+// one is free; while one wave of a SIMD waits at its barrier and for its first operands from LDS, the other multiplies.
 //
 // Token tile in LDS: row-major, 128 bytes a row and k-step, the 16-byte pieces of a row permuted by a function of the
 // row so that the eight lanes that copy one row read one whole 128-byte line of global memory while the sixteen rows a
 // matrix-instruction fragment reads at once fall into different banks.  Weights in LDS: as prepared (1 KiB a 16-row
 // weight tile and k-step in fragment order).
 //
-// Workgroups are persistent; workgroup b runs on XCD b % 8 and takes a contiguous eighth of the units, all column
-// groups of a unit at about the same time on neighbouring CUs of that XCD: a unit's token rows and an expert's weights
-// reach an XCD's L2 once while its workgroups pass.  The next task's first operands are requested before the current
-// task's epilogue (SwiGLU + FP8 requantization, or routing weight + scatter), which needs no registers for them.
+// Workgroups are persistent; workgroup b runs on XCD b % 8.  The XCDs take contiguous runs of the units of equal cost
+// (BM = 256; of equal count at BM = 128), all column groups of a unit at about the same time on neighbouring CUs of an
+// XCD: a unit's token rows reach the XCD's L2 once while its workgroups pass.  The next task's first operands are
+// requested before the current task's epilogue (SwiGLU + FP8 requantization, or routing weight + scatter), which needs no
+// registers for them.
 //
 // Reference semantics (contract level): the two phase kernels of the reference's dynamic MoE node
 // (src/moe.rs:1098-1289; runtime/kernels/moe-runtime-*/manifest.json precision string).
