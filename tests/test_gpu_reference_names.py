@@ -59,7 +59,7 @@ def module():
 
 def test_every_name_resolves(module):
     for name in ["ca_ffn_sum_shared", "ca_shared_swiglu_quant128", "ca_shared_swiglu_quant64", "ca_shared_swiglu_quant16_64", "ca_moe_frontend",
-                 "ca_moe_route_frontend", "ca_route_topk", "ca_tail_gate", "ca_block_scales_mma", "ca_pad_fp8_columns"]:
+                 "ca_moe_route_frontend", "ca_route_topk", "ca_tail_gate", "ca_block_scales_mma", "ca_pad_fp8_columns", "_router_triton_kernel"]:
         module.function(name)
 
 
@@ -119,6 +119,21 @@ def test_route_topk_nine_arguments(module):
     module.launch("ca_route_topk", 1, 512, [logits.cuda(), bias.cuda(), bias_alt.cuda(), tokens.cuda(), torch.tensor([live], dtype=torch.int32).cuda(),
                                            padding.cuda(), ids, weights, rows])
     want_ids, want_w = oracle.route_topk(oracle_config(g), logits.numpy(), bias.numpy(), bias_alt.numpy(), tokens.numpy(), live, padding.numpy())
+    assert np.array_equal(np_of(ids), want_ids) and np.array_equal(np_of(weights).view(np.uint32), want_w.view(np.uint32))
+
+
+def test_router_operator_symbol_with_the_operator_launchers_argument_list(module):
+    # src/triton_ops.rs:129-166: one block a row, the manifest's eight arguments as 64-bit words plus two zero words
+    rows, live = 6, 5
+    g, logits, bias, bias_alt, tokens = reference_inputs(rows)
+    ids = torch.zeros((rows, K), dtype=torch.int32, device="cuda")
+    weights = torch.zeros((rows, K), dtype=torch.float32, device="cuda")
+    tensors = [logits.cuda(), bias.cuda(), bias_alt.cuda(), tokens.cuda(), torch.tensor([live], dtype=torch.int32).cuda(), weights, ids]
+    words = [ctypes.c_uint64(t.data_ptr()) for t in tensors] + [ctypes.c_uint64(rows), ctypes.c_uint64(0), ctypes.c_uint64(0)]
+    argv = (ctypes.c_void_p * len(words))(*[ctypes.cast(ctypes.pointer(w), ctypes.c_void_p) for w in words])
+    assert module.hip.hipModuleLaunchKernel(module.function("_router_triton_kernel"), rows, 1, 1, 128, 1, 1, 0, None, argv, None) == 0
+    assert module.hip.hipDeviceSynchronize() == 0
+    want_ids, want_w = oracle.route_topk(oracle_config(g), logits.numpy(), bias.numpy(), bias_alt.numpy(), tokens.numpy(), live)
     assert np.array_equal(np_of(ids), want_ids) and np.array_equal(np_of(weights).view(np.uint32), want_w.view(np.uint32))
 
 

@@ -112,6 +112,17 @@ extern "C" __global__ void __launch_bounds__(1024) ca_route_topk(const float* lo
     tf_route_block<false>(logits, bias, bias_alt, tokens, live, padding, ids, weights, rows, p, blockIdx.x * waves, gridDim.x * waves,
                           gridDim.x == 1);
 }
+// The router operator `routing_vl` (src/ffn.rs:237, 380-395; runtime/kernels/routing-v1/manifest.json: symbol
+// _router_triton_kernel, one block a row, arguments scores, bias, bias_alt, input ids, live count, out weights, out indices, M,
+// then the two scratch words the reference's operator launcher appends, src/triton_ops.rs:141-142): the same top six of 384
+// with the weights before the indices.  Any block of whole waves; the block's first wave routes its row.
+extern "C" __global__ void __launch_bounds__(256) _router_triton_kernel(const float* scores, const float* bias, const float* bias_alt,
+                                                                         const long long* input_ids, const int32_t* live, float* out_weights,
+                                                                         int32_t* out_indices, int32_t M, const void*, const void*) {
+    if (threadIdx.x >= 64) return;
+    const RouteParams p{RL_EXPERTS, RL_TOPK, RL_SCORING, RL_ROUTE_SCALE, RL_ALT_TOKEN};
+    tf_route_block<false>(scores, bias, bias_alt, input_ids, live, nullptr, out_indices, out_weights, M, p, blockIdx.x, gridDim.x, false);
+}
 // kernels/moe_frontend.cuh:243-252: block 0 plans, every block quantizes the rows (32 columns a block, no floor).
 extern "C" __global__ void __launch_bounds__(512) ca_moe_frontend(const uint16_t* input, const int32_t* ids, const float* weights, uint8_t* packed,
                                                                   uint8_t* scales, int32_t* token_map, float* token_weights, int32_t* task_expert,
