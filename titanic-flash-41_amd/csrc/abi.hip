@@ -314,7 +314,7 @@ int launch_dynamic(const Context& c, bool route, const uint64_t* p, const int32_
     a.h_bf16 = (uint16_t*)p[P_INTER]; a.h_codes = (uint8_t*)p[P_INTER_CODES]; a.h_scales = (uint8_t*)p[P_INTER_SCALES];
     a.out = (uint16_t*)p[P_SCATTER];
     if (phases & 2) {
-        status = tf_grouped_shape_ok(a, true) ? tf_launch_grouped<TF_GEMM_FC1_ROUTED>(a, pairs, c.cus, s) : tf_launch_fc1_gemm(a, c.cus, s);
+        status = tf_launch_grouped<TF_GEMM_FC1_ROUTED>(a, pairs, c.cus, s);
         if (status) return status;
     }
     if (!(phases & 4)) return 0;
@@ -323,7 +323,7 @@ int launch_dynamic(const Context& c, bool route, const uint64_t* p, const int32_
     b.w = (const uint8_t*)p[P_W2]; b.ws = (const uint8_t*)p[P_S2];
     b.w_expert_stride = w2_stride; b.ws_expert_stride = s2_stride;
     b.k = g.intermediate;
-    return tf_grouped_shape_ok(b, false) ? tf_launch_grouped<TF_GEMM_FC2_ROUTED>(b, pairs, c.cus, s) : tf_launch_fc2_gemm(b, c.cus, s);
+    return tf_launch_grouped<TF_GEMM_FC2_ROUTED>(b, pairs, c.cus, s);
 }
 
 // ---- entry 2: moe.w4a16.topk_sum -----------------------------------------------------------------------------------

@@ -1,4 +1,5 @@
-// Many-row (prefill) expert projections: grouped GEMM on v_mfma_scale_f32_16x16x128_f8f6f4.
+// Many-row (prefill) projections of the FP8 shared expert and the dense product: GEMM on v_mfma_scale_f32_16x16x128_f8f6f4
+// (the kernel is written for routed FP4 experts as well; those run in experts_grouped.cuh and are not instantiated from here).
 //
 // One task = one M tile of 128 physical rows (one expert's rows, gathered through the permutation map) x one column
 // group.  A workgroup of eight waves (512 threads, two waves a SIMD) keeps a 128 x 256 accumulator: wave nq holds all
@@ -412,16 +413,8 @@ inline bool tf_gemm_shape_ok(const GemmArgs& a, bool fc1) {
     return a.k >= 512 && a.k % 512 == 0 && (a.act_block == 32 || a.act_block == 128) && a.k / a.act_block <= TF_GEMM_MAX_SCALES_ROW &&
            (fc1 ? (a.inter >= 128 && a.inter % 128 == 0) : (a.hidden >= 256 && a.hidden % 256 == 0));
 }
-inline int tf_launch_fc1_gemm(const GemmArgs& a, int cus, hipStream_t s) {
-    if (!tf_gemm_shape_ok(a, true)) return -4;
-    tf_gemm<false, TF_GEMM_FC1_ROUTED><<<tf_gemm_grid(cus), 512, 0, s>>>(a);
-    return (int)hipGetLastError();
-}
-inline int tf_launch_fc2_gemm(const GemmArgs& a, int cus, hipStream_t s) {
-    if (!tf_gemm_shape_ok(a, false)) return -4;
-    tf_gemm<false, TF_GEMM_FC2_ROUTED><<<tf_gemm_grid(cus), 512, 0, s>>>(a);
-    return (int)hipGetLastError();
-}
+// The routed experts' projections run in experts_grouped.cuh (tf_grouped_gemm); this kernel serves the FP8 shared expert and
+// the dense product.
 inline int tf_launch_dense_gemm(const GemmArgs& a, int cus, hipStream_t s) {
     if (!tf_gemm_shape_ok(a, false)) return -4;
     tf_gemm<true, TF_GEMM_DENSE><<<tf_gemm_grid(cus), 512, 0, s>>>(a);
