@@ -9,9 +9,9 @@ a run (FETCH_SIZE, WRITE_SIZE; with --shader also the L2 hit counters and the sh
 run ends with plain copies of 256 MiB, a kernel whose traffic is known, which the counters are scaled by.  The raw CSV files
 stay under DIR.
 
-`stamp` needs no GPU.  It reads DIR, scales the counters, and writes one JSON file: per workload and kernel the calls, the
-mean duration, the HBM bytes a launch (fetched + written), the algorithmic bytes the driver computed for the two streaming
-launches, and their ratio; stamped with the library's SHA-256 (the build manifest's) and, where a git work tree is
+`stamp` needs no GPU.  It reads DIR, scales the counters, and writes one JSON file: per workload, for the routed experts' two
+launches and the copy kernel, the calls, the mean duration, the HBM bytes a launch (fetched + written), the algorithmic bytes
+the driver computed, and their ratio (every other kernel: its mean duration); stamped with the library's SHA-256 (the build manifest's) and, where a git work tree is
 present, its commit.  bench.py multiplies that ratio with the algorithmic bytes of its own launches.
 """
 import argparse
@@ -151,6 +151,9 @@ def stamp(src, to):
             for k, v in counter_means(os.path.join(base, extra)).items():
                 if k in entry["kernels"]:
                     entry["kernels"][k].setdefault("counters", {}).update({c: m for c, (m, _) in v.items()})
+        # the summary keeps the routed projections and the copy kernel in full, every other kernel as its mean duration
+        entry["other_kernels_avg_us"] = {k: round(r["avg_us"], 1) for k, r in entry["kernels"].items() if r.get("role") is None}
+        entry["kernels"] = {k: r for k, r in entry["kernels"].items() if r.get("role") is not None}
         out["workloads"][w] = entry
     os.makedirs(os.path.dirname(os.path.abspath(to)), exist_ok=True)
     with open(to, "w") as f:
