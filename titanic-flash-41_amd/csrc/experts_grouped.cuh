@@ -586,6 +586,8 @@ inline bool tf_grouped_shape_ok(const GemmArgs& a, bool fc1) {
 template <int MODE>
 inline int tf_launch_grouped(const GemmArgs& a, long long routes, int cus, hipStream_t s) {
     if (!tf_grouped_shape_ok(a, MODE == TF_GEMM_FC1_ROUTED)) return -4;
+    // a lane's byte offset into the token codes is 32 bits: physical rows x contraction length must stay below 2^32
+    if ((unsigned long long)a.max_tiles * TF_GEMM_TILE_M * (unsigned long long)a.k > 0xffffffffull) return -4;
     const int grid = tf_gemm_grid(cus);
     const bool big = routes >= 192ll * a.experts, words = a.act_block == 128;
     if (big) {
