@@ -15,8 +15,9 @@ whole-layer tokens/s, the roofline of the dominant kernel (FC1 + SwiGLU of the r
 average duration, measured with two HIP events that take the kernel's start and completion on its launch stream), and the
 CPU baseline (the C oracle, a port of the reference semantics: the reference has no CPU path) timed on a bounded sample of
 the same workload, with all threads and with one.  `configs` then holds the same measurement of the speculative-verify step
-(c3) and the two prefill chunks (c4, c5: bound by the matrix units, flops over the FC1 launch's duration between events
-recorded around it).  With --config only that configuration runs and is the top level.
+(c3) and the two prefill chunks (c4, c5: the routed FC1 launch between events recorded around it; its flops a byte say which
+roof it lies under: at 4,096 rows an expert's weights serve 96 rows, 339 flop/B against the machine's 625, so HBM; at 16,384
+rows the matrix units; the line carries the fractions of both peaks either way).  With --config only that configuration runs and is the top level.
 
 `roofline.traffic` is the measured HBM bytes a launch of the dominant kernel: the ratio of measured to algorithmic bytes
 that the committed counter file holds for the same workload (profiles/counters.json, written by
@@ -45,7 +46,7 @@ CONFIGS = {
     "c3": dict(rows=32, hidden=4096, experts=256, topk=6, inter=2048, shared=2048,
                workload="speculative verify, 4 requests x 8 draft tokens = 32 rows; H 4096, E 256, top-6, I 2048, 1 shared expert"),
     "c4": dict(rows=4096, hidden=4096, experts=256, topk=6, inter=2048, shared=2048,
-               workload="prefill chunk of 4096 tokens, uniform routing; H 4096, E 256, top-6, I 2048, 1 shared expert"),
+               workload="prefill chunk of 4096 tokens, uniform routing (iid N(0, 1) logits, no selection bias); H 4096, E 256, top-6, I 2048, 1 shared expert"),
     "c5": dict(rows=16384, hidden=4096, experts=256, topk=6, inter=2048, shared=2048,
                workload="long prefill of 16384 tokens, Zipf(1.1) expert popularity; H 4096, E 256, top-6, I 2048, 1 shared expert"),
     # not benchmark configurations: the reference's own layer (runtime/model/config.json; src/ffn.rs:65-66, 245-258), in its own numerics
@@ -170,6 +171,9 @@ def measure(pkg, name, numerics, steps, warmup, profile_steps, overlap, operands
     if key not in operands:     # the benchmark configurations share one geometry: one set of synthetic weights serves them all
         operands[key] = synth.LayerOperands(g, "bench/%d/%d" % (cfg["hidden"], cfg["experts"]), device="cuda")
     ops = operands[key]
+    if name == "c4":      # uniform routing: no selection bias (the layer's N(0, 0.1) bias alone gives the busiest expert ten times the mean load)
+        ops = copy.copy(ops)
+        ops.bias = torch.zeros_like(ops.bias)
     if name == "c5":      # expert popularity ~ rank^-1.1: the busiest experts take more than ten times the mean load
         ops = copy.copy(ops)
         ops.bias = synth.zipf_bias(g.experts, 1.1, 0.06, device="cuda")
@@ -259,13 +263,20 @@ def measure(pkg, name, numerics, steps, warmup, profile_steps, overlap, operands
                           "traffic_over_algorithmic": ratio}
     if wide:
         tflops = fc1_flops / (fc1_ms * 1e-3) / 1e12
-        roofline = {"bound": "mfma", "kernel": "tf_grouped_gemm<FC1> (routed FC1 + SwiGLU + FP8 requantization)",
-                    "achieved": tflops, "peak": MFMA_FP8_PEAK_TFLOPS, "unit": "TFLOP/s", "frac": tflops / MFMA_FP8_PEAK_TFLOPS,
-                    "frac_of_fp4_peak": tflops / MFMA_FP4_PEAK_TFLOPS,
+        # which roof the launch lies under: its flops a byte against the machine's (FP8 peak over HBM peak, 625 flop/B)
+        gbs = fc1_bytes / (fc1_ms * 1e-3) / 1e9
+        intensity, ridge = fc1_flops / fc1_bytes, MFMA_FP8_PEAK_TFLOPS * 1e12 / (HBM_PEAK_GBS * 1e9)
+        hbm_side = intensity < ridge
+        roofline = {"bound": "hbm" if hbm_side else "mfma", "kernel": "tf_grouped_gemm<FC1> (routed FC1 + SwiGLU + FP8 requantization)",
+                    "achieved": gbs if hbm_side else tflops, "peak": HBM_PEAK_GBS if hbm_side else MFMA_FP8_PEAK_TFLOPS,
+                    "unit": "GB/s" if hbm_side else "TFLOP/s", "frac": gbs / HBM_PEAK_GBS if hbm_side else tflops / MFMA_FP8_PEAK_TFLOPS,
+                    "flop_per_byte": intensity, "ridge_flop_per_byte": ridge,
+                    "tflops": tflops, "frac_of_fp8_peak": tflops / MFMA_FP8_PEAK_TFLOPS, "frac_of_fp4_peak": tflops / MFMA_FP4_PEAK_TFLOPS,
+                    "frac_of_hbm_peak": gbs / HBM_PEAK_GBS,
                     "operands": "A = FP8 E4M3 activations, B = FP4 E2M1 weights: issues at the FP8 rate (measured)",
                     "traffic": ratio * fc1_bytes if ratio is not None else None, "traffic_source": traffic_source,
                     "bytes_or_flops_per_launch": fc1_flops, "per_launch_unit": "flop", "algorithmic_bytes_per_launch": fc1_bytes,
-                    "avg_launch_ms": fc1_ms, "weight_gbs": fc1_bytes / (fc1_ms * 1e-3) / 1e9,
+                    "avg_launch_ms": fc1_ms,
                     "timing": "HIP events recorded around the launch on its stream, eager passes of the layer's schedule"}
     else:
         roofline = {"bound": "hbm", "kernel": ("tf_phase1_stream (FC1 + SwiGLU of the routed experts; the shared expert's first projection streams in the front-end launch)"
