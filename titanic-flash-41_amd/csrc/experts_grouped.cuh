@@ -25,10 +25,13 @@
 // weight tile and k-step in fragment order).
 //
 // Workgroups are persistent; workgroup b runs on XCD b % 8.  The XCDs take contiguous runs of the units of equal cost
-// (BM = 256; of equal count at BM = 128), all column groups of a unit at about the same time on neighbouring CUs of an
-// XCD: a unit's token rows reach the XCD's L2 once while its workgroups pass.  The next task's first operands are
-// requested before the current task's epilogue (SwiGLU + FP8 requantization, or routing weight + scatter), which needs no
-// registers for them.
+// (BM = 256; of equal count at BM = 128).  BM = 128: all column groups of a unit at about the same time on neighbouring
+// CUs of an XCD, so a unit's token rows reach the XCD's L2 once while its workgroups pass.  BM = 256, where an expert has
+// several units and its weights do not stay in the L2 from one to the next: four units of an expert side by side, column
+// group by column group, so that neighbouring workgroups want the same weight columns at the same time; units of more
+// than 128 rows first (one duration: the neighbours stay in step), the experts' short last units after them.  The next
+// task's first operands are requested before the current task's epilogue (SwiGLU + FP8 requantization, or routing weight
+// + scatter), which needs no registers for them.
 //
 // Reference semantics (contract level): the two phase kernels of the reference's dynamic MoE node
 // (src/moe.rs:1098-1289; runtime/kernels/moe-runtime-*/manifest.json precision string).
@@ -101,8 +104,9 @@ __global__ void __launch_bounds__(512) tf_grouped_gemm(const GemmArgs p) {
     __shared__ __attribute__((aligned(256))) uint32_t s_bsc[16 * NG * 64];
     __shared__ __attribute__((aligned(256))) int32_t s_src[3][BM];   // the permutation map's entry (route index) of each tile row, for three tasks in turn
     __shared__ __attribute__((aligned(256))) float s_wgt[NG == 2 ? 4 : 3][BM];   // FC2: routing weight of each tile row (three tasks in turn); FC1: row maxima of the column halves
-    __shared__ uint16_t s_ubase[BM == 256 ? 514 : 2], s_tbase[BM == 256 ? 514 : 2];
-    __shared__ int32_t s_part[8], s_cpart[8], s_bound[9];
+    __shared__ uint16_t s_ubase[BM == 256 ? 514 : 2], s_nbase[BM == 256 ? 514 : 2];      // units / short last units before expert e
+    __shared__ int32_t s_part[8], s_cpart[8], s_npart[8], s_bound[9], s_nbound[9];
+    constexpr int SHARE = 4;                 // BM == 256: units of an expert whose tasks of one column group run next to each other
     uint16_t* s_cbase = reinterpret_cast<uint16_t*>(s_a);      // prefix of the units' costs: needed before the ring starts only
 
     const int tid = threadIdx.x, lane = tid & 63, wave = __builtin_amdgcn_readfirstlane(tid >> 6);
@@ -112,7 +116,7 @@ __global__ void __launch_bounds__(512) tf_grouped_gemm(const GemmArgs p) {
     const int total_tiles = p.expert_tile_base[p.experts];
     int units = total_tiles;
     const int xcd = blockIdx.x & 7, local = blockIdx.x >> 3, local_count = gridDim.x >> 3;
-    int u_lo, u_hi;
+    int u_lo, u_hi, n_lo = 0, n_hi = 0;      // the XCD's units; BM == 256: short last units before them
     if constexpr (BM == 256) {
         // units of two plan tiles: per expert ceil(tiles / 2); exclusive prefix over the experts (one thread an expert).  Beside
         // it a prefix of what the units cost: a unit with more than 128 rows keeps both waves of every SIMD multiplying (5), one
@@ -123,23 +127,23 @@ __global__ void __launch_bounds__(512) tf_grouped_gemm(const GemmArgs p) {
         int tb = 0, tn = 0;
         if (e < p.experts) { tb = p.expert_tile_base[e]; tn = p.expert_tile_base[e + 1]; }
         const int mine = (tn - tb + 1) >> 1;
-        int cost = 0;
+        int cost = 0, small_last = 0;        // small: the expert's last unit has at most 128 rows (one wave a SIMD multiplies: a shorter task)
         if (mine > 0) {
             const int last_rows = (tn - tb - 1) * 128 + p.task_valid_rows[(size_t)(tn - 1) * p.groups] - 256 * (mine - 1);
             cost = 5 * (mine - 1) + (last_rows > 128 ? 5 : last_rows > 32 ? 3 : 2);
+            small_last = last_rows <= 128;
         }
-        int prefix = mine, cprefix = cost;
+        int prefix = mine, cprefix = cost, nprefix = small_last;
 #pragma unroll
         for (int o = 1; o < 64; o <<= 1) {
-            const int below = __shfl_up(prefix, o), cbelow = __shfl_up(cprefix, o);
-            if (lane >= o) { prefix += below; cprefix += cbelow; }
+            const int below = __shfl_up(prefix, o), cbelow = __shfl_up(cprefix, o), nbelow = __shfl_up(nprefix, o);
+            if (lane >= o) { prefix += below; cprefix += cbelow; nprefix += nbelow; }
         }
-        if (lane == 63) { s_part[wave] = prefix; s_cpart[wave] = cprefix; }
+        if (lane == 63) { s_part[wave] = prefix; s_cpart[wave] = cprefix; s_npart[wave] = nprefix; }
         __syncthreads();
-        for (int w = 0; w < wave; ++w) { prefix += s_part[w]; cprefix += s_cpart[w]; }
-        if (e < p.experts) { s_ubase[e + 1] = (uint16_t)prefix; s_tbase[e] = (uint16_t)tb; s_cbase[e + 1] = (uint16_t)cprefix; }
-        if (e == p.experts - 1) s_tbase[e + 1] = (uint16_t)tn;
-        if (e == 0) { s_ubase[0] = 0; s_cbase[0] = 0; }
+        for (int w = 0; w < wave; ++w) { prefix += s_part[w]; cprefix += s_cpart[w]; nprefix += s_npart[w]; }
+        if (e < p.experts) { s_ubase[e + 1] = (uint16_t)prefix; s_nbase[e + 1] = (uint16_t)nprefix; s_cbase[e + 1] = (uint16_t)cprefix; }
+        if (e == 0) { s_ubase[0] = 0; s_nbase[0] = 0; s_cbase[0] = 0; }
         __syncthreads();
         units = s_ubase[p.experts];
         if (tid <= 8) {             // boundary tid of the XCDs' shares: the first unit at or behind tid eighths of the cost
@@ -152,10 +156,14 @@ __global__ void __launch_bounds__(512) tf_grouped_gemm(const GemmArgs p) {
             const int in_expert = (int)s_ubase[lo + 1] - (int)s_ubase[lo];
             const int bound = tid == 8 ? units : min((int)s_ubase[lo] + min((target - (int)s_cbase[lo]) / 5, in_expert), units);
             s_bound[tid] = tid == 0 ? 0 : bound;
+            // short last units before the boundary
+            s_nbound[tid] = tid == 0 ? 0 : tid == 8 ? (int)s_nbase[p.experts] : (int)s_nbase[bound >= (int)s_ubase[lo + 1] ? lo + 1 : lo];
         }
         __syncthreads();
         u_lo = s_bound[xcd];
         u_hi = s_bound[xcd + 1];
+        n_lo = s_nbound[xcd];
+        n_hi = s_nbound[xcd + 1];
     } else {
         u_lo = (int)((long long)units * xcd / 8);
         u_hi = (int)((long long)units * (xcd + 1) / 8);
@@ -174,19 +182,46 @@ __global__ void __launch_bounds__(512) tf_grouped_gemm(const GemmArgs p) {
         return v;
     };
     const uint32_t lds_src = tf_lds_addr(&s_src[0][0]), lds_wgt = tf_lds_addr(&s_wgt[0][0]);
-    int walk = 0;                            // BM == 256: the expert of the last unit looked up (units are asked for in ascending order)
+    // BM == 256: the XCD's tasks in two parts.  First the units of more than 128 rows (every unit but an expert's last, and
+    // the last one too if it is that long: both waves of every SIMD multiply, one duration): within an expert the units
+    // fastest, SHARE at a time, then the column groups, so that the workgroups next to each other in a round multiply SHARE
+    // row blocks by the same weight columns at about the same time and those weights cross the fabric once for all of them
+    // (an expert's weights do not stay in an XCD's L2 from one unit to the next; equal durations keep the neighbours in
+    // step, and a workgroup that falls behind finds its weights in the L2 and catches up).  Then the experts' short last
+    // units (s_nbase counts them), a unit's column groups next to each other.
+    const int first_part = (u_hi - n_hi) - (u_lo - n_lo);          // units of the first part
+    const int w_lo = u_lo - n_lo;                                   // units of the first part before this XCD's
+    int walk = 0, walk_last = 0;             // the expert of the last unit looked up in either part (each asked for in ascending order)
+    auto lds16 = [](const uint16_t* at) { return __builtin_amdgcn_readfirstlane((int)*at); };
     auto fetch = [&](int q, int slot) {
         TaskRef r;
-        const int un = q / groups, unit = u_lo + un;
-        r.ng = q - un * groups;
         if constexpr (BM == 256) {
-            while (__builtin_amdgcn_readfirstlane((int)s_ubase[walk + 1]) <= unit) ++walk;       // s_ubase[walk] <= unit < s_ubase[walk + 1]
-            const int k2 = unit - __builtin_amdgcn_readfirstlane((int)s_ubase[walk]);
-            const int tb = __builtin_amdgcn_readfirstlane((int)s_tbase[walk]), tn = __builtin_amdgcn_readfirstlane((int)s_tbase[walk + 1]);
-            r.expert = walk;
+            int unit;
+            if (q < first_part * groups) {
+                // position w among the units of the first part; expert e holds [s_ubase[e] - s_nbase[e], s_ubase[e + 1] - s_nbase[e + 1])
+                const int w = w_lo + q / groups;
+                while (lds16(&s_ubase[walk + 1]) - lds16(&s_nbase[walk + 1]) <= w) ++walk;
+                const int before = lds16(&s_nbase[walk]);
+                const int a = max(lds16(&s_ubase[walk]) - before, w_lo), b = min(lds16(&s_ubase[walk + 1]) - lds16(&s_nbase[walk + 1]), w_lo + first_part);
+                const int t = q - (a - w_lo) * groups, blk = t / (SHARE * groups);
+                const int mb = min(SHARE, b - a - SHARE * blk), rem = t - blk * SHARE * groups;
+                r.ng = rem / mb;
+                unit = a + SHARE * blk + (rem - r.ng * mb) + before;
+                r.expert = walk;
+            } else {
+                const int j = (q - first_part * groups) / groups;
+                r.ng = q - first_part * groups - j * groups;
+                while (lds16(&s_nbase[walk_last + 1]) <= n_lo + j) ++walk_last;      // the expert of the (n_lo + j)-th short last unit
+                unit = lds16(&s_ubase[walk_last + 1]) - 1;
+                r.expert = walk_last;
+            }
+            const int k2 = unit - lds16(&s_ubase[r.expert]);
+            const int tb = scalar_load(p.expert_tile_base + r.expert), tn = scalar_load(p.expert_tile_base + r.expert + 1);
             r.first_tile = tb + 2 * k2;
             r.rows = min(BM, (tn - tb - 1) * 128 + scalar_load(p.task_valid_rows + (size_t)(tn - 1) * p.groups) - 256 * k2);
         } else {
+            const int un = q / groups, unit = u_lo + un;
+            r.ng = q - un * groups;
             r.first_tile = unit;
             r.expert = scalar_load(p.task_expert + (size_t)unit * p.groups);
             r.rows = scalar_load(p.task_valid_rows + (size_t)unit * p.groups);
