@@ -277,7 +277,6 @@ __global__ void __launch_bounds__(512) tf_grouped_gemm(const GemmArgs p) {
 
     // ---- this lane's fragment addresses ----------------------------------------------------------------------------------
     const int swz = (r16 & 7) ^ (r16 >> 3);
-    const int a_lo = (wm * WROWS + r16) * 128 + ((g ^ swz) << 4), a_hi = a_lo ^ 64;     // + 2,048 a fragment
     // weight tiles of the wave within a stage: FC1: four "up" tiles 4 wn + t, then the four "gate" tiles 8 + 4 wn + t of the same
     // columns; FC2: tiles 8 wn + t.  One base a wave plus a constant a tile.
     const int b_first = FC1 ? wn * 4 : wn * 8;
@@ -312,7 +311,12 @@ __global__ void __launch_bounds__(512) tf_grouped_gemm(const GemmArgs p) {
     int slot = 0, slot_next = 1, slot_after = 2;
     for (int q = local; q < my_tasks; q += local_count) {
         const int rows = cur.rows, first_tile = cur.first_tile, ng = cur.ng;
-        const int nf = max(0, min(NF, (rows - wm * WROWS + 15) >> 4));     // fragments of this wave with valid rows
+        // A unit of at most BM / 2 rows spreads them over all eight waves (wave row groups of BM / 8 rows, half the fragments
+        // each) instead of leaving the upper row groups' waves without products: both waves of every SIMD then multiply, one
+        // under the other's barrier and LDS latency.
+        const int wbase = wm * (rows <= BM / 2 ? WROWS / 2 : WROWS);          // first tile row of this wave
+        const int nf = max(0, min(rows <= BM / 2 ? NF / 2 : NF, (rows - wbase + 15) >> 4));     // fragments of this wave with valid rows
+        const int a_lo = (wbase + r16) * 128 + ((g ^ swz) << 4), a_hi = a_lo ^ 64;     // + 2,048 a fragment
         TaskRef after = nxt;
 
         // One task, compiled for 0, NF / 2 or NF fragments of the wave so that no product sits under a branch and the
@@ -392,7 +396,7 @@ __global__ void __launch_bounds__(512) tf_grouped_gemm(const GemmArgs p) {
                     // block's products: every read of the stage has been issued a block earlier.
                     const uint8_t* sa = s_a + cs * A_STAGE;
                     const uint8_t* sb = s_b + cs * B_STAGE + lane16;
-                    const uint32_t* sc = &s_asc[cs][wm * WROWS + r16];
+                    const uint32_t* sc = &s_asc[cs][wbase + r16];
                     auto block_at = [&](int b) constexpr { return ((b >> 1) * 16 + (FC1 ? ((b & 1) ? 8 + 4 * wn : 4 * wn) : 8 * wn + 4 * (b & 1))) * 1024; };
                     u4v bf[2][4];
 #pragma unroll
@@ -430,7 +434,7 @@ __global__ void __launch_bounds__(512) tf_grouped_gemm(const GemmArgs p) {
                 if constexpr (FR > 0 && NG == 1) {
                     const uint8_t* sa = s_a + cs * A_STAGE;
                     const uint8_t* sb = s_b + cs * B_STAGE + b_first * 1024 + lane16;
-                    const uint32_t* sc = &s_asc[cs][wm * WROWS + r16];
+                    const uint32_t* sc = &s_asc[cs][wbase + r16];
                     u4v bf[8];
 #pragma unroll
                     for (int t = 0; t < 8; ++t) bf[t] = *reinterpret_cast<const u4v*>(sb + b_step(t) * 1024);
@@ -501,7 +505,7 @@ __global__ void __launch_bounds__(512) tf_grouped_gemm(const GemmArgs p) {
 
             // ---- epilogue: values first, then a wait for every request in flight (the next task's first k-steps, long landed
             // by now: its first LEAD k-steps then wait for nothing, in particular not for the stores below), then the stores ---
-            // Lane (g, r16) of product (f, t) holds tile row wm WROWS + 16 f + r16 and the four consecutive columns 4 g + i of
+            // Lane (g, r16) of product (f, t) holds tile row wbase + 16 f + r16 and the four consecutive columns 4 g + i of
             // weight tile t of column group `cg`; the task's column groups one after the other.
 #pragma unroll
             for (int gi = 0; gi < NG; ++gi) {
@@ -534,11 +538,11 @@ __global__ void __launch_bounds__(512) tf_grouped_gemm(const GemmArgs p) {
                     }
                     if constexpr (WORDS) {               // one scale a row and 128 columns: both column halves (waves wn = 0, 1)
 #pragma unroll
-                        for (int f = 0; f < FR; ++f) if (g == 0) s_max[wn][wm * WROWS + 16 * f + r16] = fmaxf(amax[f][0], amax[f][1]);
+                        for (int f = 0; f < FR; ++f) if (g == 0) s_max[wn][wbase + 16 * f + r16] = fmaxf(amax[f][0], amax[f][1]);
                         tf_lds_barrier();
 #pragma unroll
                         for (int f = 0; f < FR; ++f) {
-                            const int row = wm * WROWS + 16 * f + r16;
+                            const int row = wbase + 16 * f + r16;
                             amax[f][0] = amax[f][1] = fmaxf(s_max[0][row], s_max[1][row]);
                         }
                     }
@@ -555,7 +559,7 @@ __global__ void __launch_bounds__(512) tf_grouped_gemm(const GemmArgs p) {
                     if (gi == 0) tf_wait_vm<0>();
 #pragma unroll
                     for (int f = 0; f < FR; ++f) {
-                        const int row = wm * WROWS + 16 * f + r16;
+                        const int row = wbase + 16 * f + r16;
                         if (row < rows) {
                             const size_t phys = (size_t)first_tile * 128 + row;
 #pragma unroll
@@ -580,7 +584,7 @@ __global__ void __launch_bounds__(512) tf_grouped_gemm(const GemmArgs p) {
                     size_t out_at[FRA];
 #pragma unroll
                     for (int f = 0; f < FR; ++f) {
-                        const int row = min(wm * WROWS + 16 * f + r16, BM - 1);
+                        const int row = min(wbase + 16 * f + r16, BM - 1);
                         const float share = s_wgt[slot][row];
                         out_at[f] = (size_t)s_src[slot][row] * p.hidden + cg * 256 + wn * 128 + 4 * g;
 #pragma unroll
@@ -591,7 +595,7 @@ __global__ void __launch_bounds__(512) tf_grouped_gemm(const GemmArgs p) {
                     if (gi == 0) tf_wait_vm<0>();
 #pragma unroll
                     for (int f = 0; f < FR; ++f)
-                        if (wm * WROWS + 16 * f + r16 < rows) {
+                        if (wbase + 16 * f + r16 < rows) {
 #pragma unroll
                             for (int t = 0; t < 8; ++t) *reinterpret_cast<u2v*>(p.out + out_at[f] + 16 * t) = packed[f][t];
                         }
