@@ -84,6 +84,18 @@ constexpr int tf_loads_behind(int u) {
     return n;
 }
 
+// What a 256-row unit costs by its rows (more than 128 / more than 32 / fewer), for the XCDs' shares.
+#ifndef TF_UNIT_COST
+#define TF_UNIT_COST 5
+#define TF_UNIT_COST_SHORT 3
+#define TF_UNIT_COST_TINY 2
+#endif
+#ifndef TF_GROUPED_SHARE
+#define TF_GROUPED_SHARE 4
+#endif
+// 256-row units: the prefix of the units' costs is held in 16 bits
+#define TF_GROUPED_MAX_UNITS (65535 / TF_UNIT_COST)
+
 template <int MODE, int BM, bool WORDS>
 __global__ void __launch_bounds__(512) tf_grouped_gemm(const GemmArgs p) {
     constexpr bool FC1 = MODE == TF_GEMM_FC1_ROUTED;
@@ -106,7 +118,7 @@ __global__ void __launch_bounds__(512) tf_grouped_gemm(const GemmArgs p) {
     __shared__ __attribute__((aligned(256))) float s_wgt[NG == 2 ? 4 : 3][BM];   // FC2: routing weight of each tile row (three tasks in turn); FC1: row maxima of the column halves
     __shared__ uint16_t s_ubase[BM == 256 ? 514 : 2], s_nbase[BM == 256 ? 514 : 2];      // units / short last units before expert e
     __shared__ int32_t s_part[8], s_cpart[8], s_npart[8], s_bound[9], s_nbound[9];
-    constexpr int SHARE = 4;                 // BM == 256: units of an expert whose tasks of one column group run next to each other
+    constexpr int SHARE = TF_GROUPED_SHARE;  // BM == 256: units of an expert whose tasks of one column group run next to each other
     uint16_t* s_cbase = reinterpret_cast<uint16_t*>(s_a);      // prefix of the units' costs: needed before the ring starts only
 
     const int tid = threadIdx.x, lane = tid & 63, wave = __builtin_amdgcn_readfirstlane(tid >> 6);
@@ -130,7 +142,7 @@ __global__ void __launch_bounds__(512) tf_grouped_gemm(const GemmArgs p) {
         int cost = 0, small_last = 0;        // small: the expert's last unit has at most 128 rows (one wave a SIMD multiplies: a shorter task)
         if (mine > 0) {
             const int last_rows = (tn - tb - 1) * 128 + p.task_valid_rows[(size_t)(tn - 1) * p.groups] - 256 * (mine - 1);
-            cost = 5 * (mine - 1) + (last_rows > 128 ? 5 : last_rows > 32 ? 3 : 2);
+            cost = TF_UNIT_COST * (mine - 1) + (last_rows > 128 ? TF_UNIT_COST : last_rows > 32 ? TF_UNIT_COST_SHORT : TF_UNIT_COST_TINY);
             small_last = last_rows <= 128;
         }
         int prefix = mine, cprefix = cost, nprefix = small_last;
@@ -154,7 +166,7 @@ __global__ void __launch_bounds__(512) tf_grouped_gemm(const GemmArgs p) {
                 if ((int)s_cbase[mid] <= target) lo = mid; else hi = mid;
             }
             const int in_expert = (int)s_ubase[lo + 1] - (int)s_ubase[lo];
-            const int bound = tid == 8 ? units : min((int)s_ubase[lo] + min((target - (int)s_cbase[lo]) / 5, in_expert), units);
+            const int bound = tid == 8 ? units : min((int)s_ubase[lo] + min((target - (int)s_cbase[lo]) / TF_UNIT_COST, in_expert), units);
             s_bound[tid] = tid == 0 ? 0 : bound;
             // short last units before the boundary
             s_nbound[tid] = tid == 0 ? 0 : tid == 8 ? (int)s_nbase[p.experts] : (int)s_nbase[bound >= (int)s_ubase[lo + 1] ? lo + 1 : lo];
@@ -628,7 +640,7 @@ inline int tf_launch_grouped(const GemmArgs& a, long long routes, int cus, hipSt
     // a lane's byte offset into the token codes is 32 bits: physical rows x contraction length must stay below 2^32
     if ((unsigned long long)a.max_tiles * TF_GEMM_TILE_M * (unsigned long long)a.k > 0xffffffffull) return -4;
     const int grid = tf_gemm_grid(cus);
-    const bool big = routes >= 192ll * a.experts, words = a.act_block == 128;
+    const bool big = routes >= 192ll * a.experts && a.max_tiles / 2 + a.experts <= TF_GROUPED_MAX_UNITS, words = a.act_block == 128;
     if (big) {
         if (words) tf_grouped_gemm<MODE, 256, true><<<grid, 512, 0, s>>>(a);
         else tf_grouped_gemm<MODE, 256, false><<<grid, 512, 0, s>>>(a);
