@@ -11,7 +11,7 @@ stay under DIR.
 
 `stamp` needs no GPU.  It reads DIR, scales the counters, and writes one JSON file: per workload, for the routed experts' two
 launches and the copy kernel, the calls, the mean duration, the HBM bytes a launch (fetched + written), the algorithmic bytes
-the driver computed, and their ratio (every other kernel: its mean duration); stamped with the library's SHA-256 (the build manifest's) and, where a git work tree is
+the driver computed, and their ratio, per kernel and summed over a projection's kernels (every other kernel: its mean duration); stamped with the library's SHA-256 (the build manifest's) and, where a git work tree is
 present, its commit.  bench.py multiplies that ratio with the algorithmic bytes of its own launches.
 """
 import argparse
@@ -148,6 +148,19 @@ def stamp(src, to):
                 algorithmic = entry.get(rec["role"] + "_algorithmic_bytes") if rec["role"] in ("fc1", "fc2") else None
                 if algorithmic:
                     rec["algorithmic_bytes"], rec["traffic_over_algorithmic"] = algorithmic, rec["hbm_bytes"] / algorithmic
+        # a projection may run as more than one launch a pass (the many-row GEMM: the long units, then the experts' odd last
+        # tiles): its traffic and duration are the sums over its kernels, which run once a pass each
+        entry["roles"] = {}
+        for role in ("fc1", "fc2"):
+            recs = [r for r in entry["kernels"].values() if r["role"] == role and "hbm_bytes" in r]
+            algorithmic = entry.get(role + "_algorithmic_bytes")
+            if recs and algorithmic:
+                total = sum(r["hbm_bytes"] for r in recs)
+                entry["roles"][role] = {"kernels": len(recs), "avg_us": sum(r["avg_us"] for r in recs), "hbm_bytes": total,
+                                        "algorithmic_bytes": algorithmic, "traffic_over_algorithmic": total / algorithmic}
+                for r in recs:
+                    if len(recs) > 1:
+                        r.pop("traffic_over_algorithmic", None)
         for extra in ("l2", "shader"):
             for k, v in counter_means(os.path.join(base, extra)).items():
                 if k in entry["kernels"]:
@@ -163,8 +176,9 @@ def stamp(src, to):
     for w, entry in out["workloads"].items():
         for k, rec in entry["kernels"].items():
             if rec.get("role") in ("fc1", "fc2"):
-                print("%s %-4s %-50s %9.1f us  hbm %.4g B  x%.3f" % (w, rec["role"], k[:50], rec["avg_us"], rec.get("hbm_bytes", float("nan")),
-                                                                   rec.get("traffic_over_algorithmic", float("nan"))))
+                print("%s %-4s %-50s %9.1f us  hbm %.4g B" % (w, rec["role"], k[:50], rec["avg_us"], rec.get("hbm_bytes", float("nan"))))
+        for role, rec in entry["roles"].items():
+            print("%s %-4s %d kernel(s) %9.1f us  hbm %.4g B  x%.3f" % (w, role, rec["kernels"], rec["avg_us"], rec["hbm_bytes"], rec["traffic_over_algorithmic"]))
 
 
 def load(path=None):
@@ -180,7 +194,10 @@ def traffic_ratio(counters, workload, role="fc1"):
     """Measured HBM bytes over algorithmic bytes of the workload's kernel of that role, or None."""
     if not counters or workload not in counters.get("workloads", {}):
         return None
-    for rec in counters["workloads"][workload]["kernels"].values():
+    entry = counters["workloads"][workload]
+    if role in entry.get("roles", {}):
+        return entry["roles"][role]["traffic_over_algorithmic"]
+    for rec in entry["kernels"].values():
         if rec.get("role") == role and "traffic_over_algorithmic" in rec:
             return rec["traffic_over_algorithmic"]
     return None
