@@ -57,20 +57,34 @@ int ca_shared_swiglu_in(void* context, int rows, const void* input, void* output
 int ca_ffn_add_in(void* context, int rows, const void* routed, const void* shared, void* out, void* stream);
 
 /* ---- the decoder's FFN boundary either side of the layer ------------------------------------------------------- */
-/* Upstream: the reference's boundary hands the layer its normalized BF16 input together with that input's MXFP8 codes, and
- * the layer then skips its own quantizer (src/decoder.rs:1654-1656 -> Layer::run_quantized_input, src/ffn.rs:974-975,
- * 1053-1065).  The reference's producer is an operator binary (src/mhc.rs:606-614); this one is an RMS norm with a BF16
- * boundary: normed = bf16((x / sqrt(mean(x^2) + eps)) * weight), then both MXFP8 flavours of `normed` in the context's
- * activation block width: codes / scales (zero block -> scale byte 0; the routed experts' input), codes_min / scales_min (amax
- * floored at 1e-4; the shared expert's input); either pair may be null.  x, normed: [rows][hidden] BF16; weight: [hidden]
- * BF16.  hidden <= 8,192. */
+/* Upstream, the reference's producer `hc_combine_norm_quant` (runtime/kernels/mhc-norm-quant-v1/mhc-norm-quant.py:15-44 and its
+ * layout8 twin; loaded at src/mhc.rs:606-614, launched at :981-990): the row's `streams` residual streams x [rows][streams][H]
+ * (BF16) are collapsed with the predecessor's pre-coefficients pre [rows][streams] (FP32; null: all 1) by ordered FP32 fused
+ * multiply-adds and rounded to BF16; normed = bf16((value / sqrt(mean(value^2) + 1e-20)) * weight); then the shared-flavour
+ * MXFP8 quantizer in the context's activation block width (amax floored at 1e-4): codes_min [rows][H] (the reference's Q),
+ * scales_min [rows][H / block] (SR), and the same scale bytes at the reference's matrix-instruction offsets in mma_scales (SM:
+ * ceil(rows / 128) * ceil(H / 128) * 512 bytes; 32-wide blocks only; bytes of absent rows are not written).  normed and the
+ * (codes_min, scales_min) pair feed Layer::run_quantized_input (src/ffn.rs:974-975, 1053-1065; src/decoder.rs:1654-1656).
+ * Additive: codes / scales, the routed experts' flavour of the same row (zero block -> scale byte 0).  Each of the two pairs and
+ * mma_scales may be null.  The reference's approximate reciprocal root is replaced by a correctly rounded one.  H <= 8,192. */
+int ca_hc_combine_norm_quant(void* context, int rows, int streams, const void* x, const float* pre, const void* weight, void* normed,
+                             void* codes_min, void* scales_min, void* mma_scales, void* codes, void* scales, void* stream);
+/* The single-stream case of the producer with a caller's eps (a plain RMS norm with a BF16 boundary), both flavours. */
 int ca_ffn_norm_quant(void* context, int rows, const void* x, const void* weight, float eps, void* normed, void* codes, void* scales,
                       void* codes_min, void* scales_min, void* stream);
-/* Downstream: the route sum and the shared addition (ca_ffn_sum_shared: src/ffn.rs:1041-1044) with the residual addition
- * that follows the layer in the decoder (src/decoder.rs:1497-1543 `finish_ffn`) in the same pass: routed (rows < live) =
- * ordered FP32 sum of the top-k route outputs rounded to BF16; ffn = bf16(routed + shared) (flush-to-zero add), written to
- * ffn_out unless null; residual_out = bf16(f32(ffn) + f32(residual)) (may alias residual).  The reference's own boundary mixes
- * several residual streams in an operator binary; this is the single-stream addition. */
+/* Downstream, the reference's `hc_post_tiles` (runtime/kernels/mhc-post-tiles-v1/mhc-post-tiles.py:11-27; launched at
+ * src/mhc.rs:1223-1234 behind the layer, src/decoder.rs:1497-1543 `finish_ffn`): the layer's output mixed into the four
+ * residual streams, y[row][c][h] = bf16(fma(C[3][c], r3, fma(C[2][c], r2, fma(C[1][c], r1, fma(post[c], a, C[0][c] * r0))))) with
+ * a = sublayer [rows][H], r_s = residual [rows][4][H] (BF16), post [rows][4], C = comb [rows][4][4] (FP32).  y may alias
+ * residual (a thread reads its columns of all four streams before it writes them). */
+int ca_hc_post(void* context, int rows, const void* sublayer, const void* residual, const float* post, const float* comb, void* y, void* stream);
+/* Additive: ca_ffn_sum_shared (src/ffn.rs:1041-1044) with ca_hc_post behind it in one pass: routed (rows < live) = ordered
+ * FP32 sum of the top-k route outputs rounded to BF16; ffn = bf16(routed + shared) (flush-to-zero add), written to ffn_out
+ * unless null; y = the post step of ffn. */
+int ca_ffn_sum_hc_post(void* context, int rows, int live, const void* routes, const void* shared, const void* residual, const float* post,
+                       const float* comb, void* routed, void* ffn_out, void* y, void* stream);
+/* Additive: the single-stream form of the same pass (one residual stream, coefficients 1): routed and ffn as above,
+ * residual_out = bf16(f32(ffn) + f32(residual)) (may alias residual). */
 int ca_ffn_sum_residual(void* context, int rows, int live, const void* routes, const void* shared, const void* residual, void* routed,
                         void* ffn_out, void* residual_out, void* stream);
 

@@ -268,6 +268,36 @@ def rmsnorm(x, weight, eps):
     return out
 
 
+def hc_mma_scale_bytes(rows, groups):
+    """Size of the MMA-offset scale array for `rows` rows of `groups` 32-wide blocks: whole tiles of 128 rows."""
+    return ((rows + 127) // 128) * ((groups + 3) // 4) * 512
+
+
+def hc_combine_norm_quant(x, pre, weight, block=32, eps=1e-20, mma=True):
+    """x [rows][streams][cols] BF16 bits, pre [rows][streams] f32 or None -> (y, q, sr, sm or None)."""
+    x, weight = _c(x, np.uint16), _c(weight, np.uint16)
+    rows, streams, cols = x.shape
+    pre = None if pre is None else _c(pre, np.float32)
+    y = np.empty((rows, cols), np.uint16)
+    q = np.empty((rows, cols), np.uint8)
+    sr = np.empty((rows, cols // block), np.uint8)
+    sm = np.zeros(hc_mma_scale_bytes(rows, cols // block), np.uint8) if mma else None
+    lib().orc_hc_combine_norm_quant(_p(x), None if pre is None else _p(pre), _p(weight), _p(y), _p(q), _p(sr),
+                                    None if sm is None else _p(sm), _i32(rows), _i32(cols), _i32(streams), _i32(block),
+                                    ctypes.c_float(eps))
+    return y, q, sr, sm
+
+
+def hc_post(a, residual, post, comb):
+    """a [rows][cols], residual [rows][streams][cols] BF16 bits; post [rows][streams], comb [rows][streams][streams] f32."""
+    a, residual = _c(a, np.uint16), _c(residual, np.uint16)
+    post, comb = _c(post, np.float32), _c(comb, np.float32)
+    rows, streams, cols = residual.shape
+    y = np.empty_like(residual)
+    lib().orc_hc_post(_p(a), _p(residual), _p(post), _p(comb), _p(y), _i32(rows), _i32(cols), _i32(streams))
+    return y
+
+
 def residual_add(a, b):
     a, b = _c(a, np.uint16), _c(b, np.uint16)
     out = np.empty_like(a)

@@ -100,6 +100,12 @@ void orc_ffn_sum_shared(const uint16_t* routes, const uint16_t* shared, uint16_t
                         int32_t rows, int32_t topk, int32_t hidden, int32_t live);
 /* the decoder's FFN boundary either side of the layer: RMS norm with a BF16 boundary; BF16 residual addition */
 void orc_rmsnorm(const uint16_t* x, const uint16_t* weight, uint16_t* out, int32_t rows, int32_t cols, float eps);
+/* the reference's boundary operators: runtime/kernels/mhc-norm-quant-v1/mhc-norm-quant.py, mhc-post-tiles-v1/mhc-post-tiles.py */
+void orc_hc_combine_norm_quant(const uint16_t* x, const float* pre, const uint16_t* weight, uint16_t* y, uint8_t* q,
+                               uint8_t* sr, uint8_t* sm, int32_t rows, int32_t cols, int32_t streams, int32_t block,
+                               float eps);
+void orc_hc_post(const uint16_t* a, const uint16_t* residual, const float* post, const float* comb, uint16_t* y,
+                 int32_t rows, int32_t cols, int32_t streams);
 void orc_residual_add(const uint16_t* a, const uint16_t* b, uint16_t* out, int64_t n);
 
 /* ---- whole layer --------------------------------------------------------------------------- */

@@ -43,7 +43,8 @@ class Module:
             else:
                 held.append(ctypes.c_int32(a))
         argv = (ctypes.c_void_p * len(held))(*[ctypes.cast(ctypes.pointer(h), ctypes.c_void_p) for h in held])
-        assert self.hip.hipModuleLaunchKernel(self.function(name), grid, 1, 1, block, 1, 1, shared, None, argv, None) == 0, name
+        gx, gy = grid if isinstance(grid, tuple) else (grid, 1)
+        assert self.hip.hipModuleLaunchKernel(self.function(name), gx, gy, 1, block, 1, 1, shared, None, argv, None) == 0, name
         assert self.hip.hipDeviceSynchronize() == 0, name
 
     def close(self):
@@ -59,7 +60,8 @@ def module():
 
 def test_every_name_resolves(module):
     for name in ["ca_ffn_sum_shared", "ca_shared_swiglu_quant128", "ca_shared_swiglu_quant64", "ca_shared_swiglu_quant16_64", "ca_moe_frontend",
-                 "ca_moe_route_frontend", "ca_route_topk", "ca_tail_gate", "ca_block_scales_mma", "ca_pad_fp8_columns", "_router_triton_kernel"]:
+                 "ca_moe_route_frontend", "ca_route_topk", "ca_tail_gate", "ca_block_scales_mma", "ca_pad_fp8_columns", "_router_triton_kernel",
+                 "ca_moe_group_sum_rows", "hc_combine_norm_quant", "hc_post_tiles"]:
         module.function(name)
 
 
@@ -192,6 +194,55 @@ def test_moe_route_frontend_twenty_three_arguments(module):
     check_plan(b, tiles, want_ids[:rows], want_w[:rows], groups, tile_m)
     codes, sc = oracle.quantize_rows(u16(x)[:rows], 32, 0.0)
     assert np.array_equal(np_of(packed), codes) and np.array_equal(np_of(scales), sc)
+
+
+def test_group_sum_rows_six_arguments(module):
+    # kernels/ffn_sum_shared.cuh:35-58 as src/decoder.rs:1000-1008 launches it: one group of a sequence-parallel chunk's route sums,
+    # laid out [destination rank][row of the group][5120]
+    rows, groups = 32, 2
+    quarter, per = rows // 4, rows // 4 // groups
+    live = 27
+    routes = synth.activations("names/group-routes", rows * K, H).reshape(rows, K, H).cuda()
+    summed = oracle.topk_sum(u16(routes))
+    for group in range(groups):
+        out = torch.full((4, per, H), 0x3c00, dtype=torch.int16, device="cuda")
+        threads = 4 * per * (H // 8)
+        module.launch("ca_moe_group_sum_rows", (threads + 255) // 256, 256, [routes, out, quarter, per, group, live])
+        got = u16(out)
+        for c in range(4):
+            for j in range(per):
+                row = c * quarter + group * per + j
+                if row < live:
+                    assert np.array_equal(got[c, j], summed[row]), (group, c, j)
+                else:
+                    assert np.all(got[c, j] == 0x3c00)             # rows at or past the live count are not written
+
+
+@pytest.mark.parametrize("rows,parts", [(6, 4), (16, 2), (128, 4)])
+def test_boundary_producer_by_the_operator_launchers_list(module, rows, parts):
+    # `hc_norm_quant_p4` / `_p2` (src/mhc.rs:606-614, 981-990): grid (rows, PARTS), 256 threads, X P W Y Q SR SM + the launcher's two
+    # scratch words (src/triton_ops.rs:141-142)
+    from test_boundary_steps import dev, hc_inputs
+    x, pre, w = hc_inputs(rows, H, name="names/hc")
+    y = torch.zeros((rows, H), dtype=torch.int16, device="cuda")
+    q, sr = torch.zeros((rows, H), dtype=torch.uint8, device="cuda"), torch.zeros((rows, H // 32), dtype=torch.uint8, device="cuda")
+    sm = torch.zeros(20480, dtype=torch.uint8, device="cuda")
+    module.launch("hc_combine_norm_quant", (rows, parts), 256, [dev(x), dev(pre), dev(w), y, q, sr, sm, None, None])
+    want_y, want_q, want_sr, want_sm = oracle.hc_combine_norm_quant(x, pre, w)
+    assert np.array_equal(u16(y), want_y) and np.array_equal(np_of(q), want_q) and np.array_equal(np_of(sr), want_sr)
+    assert np.array_equal(np_of(sm), want_sm)
+
+
+def test_boundary_post_step_by_the_operator_launchers_list(module):
+    # `hc_post_b128_w1` (src/mhc.rs:1223-1234): grid (rows, 40), A R POST C Y + two scratch words; any block
+    from test_boundary_steps import dev, post_inputs
+    rows = 6
+    a, r, post, comb = post_inputs(rows, H, "names/post")
+    want = oracle.hc_post(a, r, post, comb)
+    for block in (32, 64, 256):
+        y = torch.zeros((rows, 4, H), dtype=torch.int16, device="cuda")
+        module.launch("hc_post_tiles", (rows, 40), block, [dev(a), dev(r), dev(post), dev(comb), y, None, None])
+        assert np.array_equal(u16(y), want), block
 
 
 def test_tail_gate_scale_spread_and_column_padding(module):

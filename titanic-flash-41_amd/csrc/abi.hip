@@ -479,7 +479,8 @@ const KernelName kKernels[] = {
     TF_KERNEL(ca_expert_scale_code1), TF_KERNEL(ca_expert_scale_code1_check), TF_KERNEL(ca_expert_scale_code1_census),
     TF_KERNEL(ca_expert_scale_codes4), TF_KERNEL(ca_router_logits_mfma), TF_KERNEL(ca_codec_encode), TF_KERNEL(ca_codec_decode),
     TF_KERNEL(ca_codec_pack_bf16), TF_KERNEL(ca_codec_unpack_routed), TF_KERNEL(ca_codec_local_live), TF_KERNEL(ca_convert_formats),
-    TF_KERNEL(ca_rmsnorm_quant), TF_KERNEL(ca_ffn_sum_shared_residual),
+    TF_KERNEL(ca_rmsnorm_quant), TF_KERNEL(ca_ffn_sum_shared_residual), TF_KERNEL(ca_hc_combine_norm_quant_rows), TF_KERNEL(ca_hc_post_rows),
+    TF_KERNEL(ca_ffn_sum_shared_hc_post),
 };
 constexpr int kKernelCount = sizeof(kKernels) / sizeof(kKernels[0]);
 
@@ -555,6 +556,39 @@ int ca_ffn_norm_quant(void* context, int rows, const void* x, const void* weight
     if (g.hidden > 8192 || g.hidden % g.act_block) return -4;
     ca_rmsnorm_quant<<<rows, 256, 0, (hipStream_t)stream>>>((const uint16_t*)x, (const uint16_t*)weight, (uint16_t*)normed, (uint8_t*)codes,
                                                             (uint8_t*)scales, (uint8_t*)codes_min, (uint8_t*)scales_min, g.hidden, g.act_block, eps);
+    return launch_status();
+}
+int ca_hc_combine_norm_quant(void* context, int rows, int streams, const void* x, const float* pre, const void* weight, void* normed,
+                             void* codes_min, void* scales_min, void* mma_scales, void* codes, void* scales, void* stream) {
+    if (!context || !x || !weight || !normed || rows < 1 || rows > 65536 || streams < 1 || streams > 8 || (!codes != !scales) ||
+        (!codes_min != !scales_min))
+        return -1;
+    const ca_geometry& g = ((const Context*)context)->g;
+    if (g.hidden > 8192 || g.hidden % g.act_block) return -4;
+    if (mma_scales && g.act_block != 32) return -1;          // the reference's offsets are those of 32-wide blocks
+    ca_hc_combine_norm_quant_rows<<<dim3(rows, 1, 1), 256, 0, (hipStream_t)stream>>>(
+        (const uint16_t*)x, pre, (const uint16_t*)weight, (uint16_t*)normed, (uint8_t*)codes_min, (uint8_t*)scales_min, (uint8_t*)mma_scales,
+        (uint8_t*)codes, (uint8_t*)scales, g.hidden, streams, g.act_block, 1.0e-20f);
+    return launch_status();
+}
+int ca_hc_post(void* context, int rows, const void* sublayer, const void* residual, const float* post, const float* comb, void* y, void* stream) {
+    if (!context || !sublayer || !residual || !post || !comb || !y || rows < 1) return -1;
+    const ca_geometry& g = ((const Context*)context)->g;
+    const long long n8 = (long long)rows * (g.hidden >> 3);
+    if (n8 > 0x7fffffffll) return -1;
+    ca_hc_post_rows<<<(int)((n8 + 255) / 256), 256, 0, (hipStream_t)stream>>>((const uint16_t*)sublayer, (const uint16_t*)residual, post, comb,
+                                                                          (uint16_t*)y, rows, g.hidden);
+    return launch_status();
+}
+int ca_ffn_sum_hc_post(void* context, int rows, int live, const void* routes, const void* shared, const void* residual, const float* post,
+                       const float* comb, void* routed, void* ffn_out, void* y, void* stream) {
+    if (!context || !routes || !shared || !residual || !post || !comb || !routed || !y || rows < 1 || live < 0) return -1;
+    const ca_geometry& g = ((const Context*)context)->g;
+    const long long n8 = (long long)rows * (g.hidden >> 3);
+    if (n8 > 0x7fffffffll) return -1;
+    ca_ffn_sum_shared_hc_post<<<(int)((n8 + 255) / 256), 256, 0, (hipStream_t)stream>>>(
+        (const uint16_t*)routes, (const uint16_t*)shared, (const uint16_t*)residual, post, comb, (uint16_t*)routed, (uint16_t*)ffn_out, (uint16_t*)y,
+        rows, live < rows ? live : rows, g.topk, g.hidden);
     return launch_status();
 }
 int ca_ffn_sum_residual(void* context, int rows, int live, const void* routes, const void* shared, const void* residual, void* routed,

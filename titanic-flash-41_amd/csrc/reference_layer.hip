@@ -11,13 +11,16 @@
 #define ca_moe_frontend tf_general_moe_frontend
 #define ca_moe_route_frontend tf_general_moe_route_frontend
 #define ca_route_topk tf_general_route_topk
+#define ca_moe_group_sum_rows tf_general_moe_group_sum_rows
 #include "combine.cuh"
 #include "frontend.cuh"
 #include "shared.cuh"
+#include "boundary.cuh"
 #undef ca_ffn_sum_shared
 #undef ca_moe_frontend
 #undef ca_moe_route_frontend
 #undef ca_route_topk
+#undef ca_moe_group_sum_rows
 
 namespace {
 constexpr int RL_HIDDEN = 5120, RL_EXPERTS = 384, RL_TOPK = 6, RL_SHARED = 576, RL_SHARED_PADDED = 640;
@@ -142,6 +145,48 @@ extern "C" __global__ void __launch_bounds__(512) ca_moe_route_frontend(
     tf_route_frontend(input, ids, weights, packed, scales, token_map, token_weights, task_expert, task_valid_rows, expert_tile_base,
                       const_cast<float*>(logits), bias, bias_alt, tokens, live, padding, rows, topk, experts, cols, groups, tile_m, owner_rows, 32,
                       nullptr, nullptr, RL_SCORING, RL_ROUTE_SCALE, RL_ALT_TOKEN, nullptr, nullptr, 0, (int)gridDim.x, s_pool, 0);
+}
+
+// kernels/ffn_sum_shared.cuh:35-58 (src/decoder.rs:717, 1000): the route sum of one row group of a sequence-parallel chunk, laid
+// out for that group's own reduce-scatter: out[c][j][:] = bf16(ordered FP32 sum of the six route outputs of row
+// c * quarter + group * per + j), c = 0..3, j < per; rows at or past `live` are not written.  Any grid that covers
+// 4 * per * 5,120 / 8 threads; 8 columns a thread.
+extern "C" __global__ void __launch_bounds__(256) ca_moe_group_sum_rows(const uint16_t* routes, uint16_t* out, int quarter, int per, int group,
+                                                                        int live) {
+    constexpr int PER_ROW = RL_HIDDEN / 8;
+    const long long n = 4ll * per * PER_ROW;
+    for (long long i = (long long)blockIdx.x * blockDim.x + threadIdx.x; i < n; i += (long long)gridDim.x * blockDim.x) {
+        const int c8 = (int)(i % PER_ROW);
+        const long long t = i / PER_ROW;
+        const int j = (int)(t % per), c = (int)(t / per);
+        const int row = c * quarter + group * per + j;
+        if (row >= live) continue;
+        float sum[8];
+        tf_sum_routes(routes, row, c8, RL_TOPK, RL_HIDDEN, sum);
+        u4v o;
+#pragma unroll
+        for (int k = 0; k < 4; ++k) o[k] = tf_pack_bf16(sum[2 * k], sum[2 * k + 1]);
+        reinterpret_cast<u4v*>(out + ((long long)c * per + j) * RL_HIDDEN)[c8] = o;
+    }
+}
+
+// The boundary operator `hc_norm_quant_p4` / `hc_norm_quant_p2` (symbol hc_combine_norm_quant;
+// runtime/kernels/mhc-norm-quant-v1/mhc-norm-quant.py:15-44, src/mhc.rs:606-614, 981-990): four residual streams of 5,120
+// columns, grid (rows, PARTS), 256 threads, arguments X, P, W, Y, Q, SR, SM and the two scratch words the operator launcher
+// appends (src/triton_ops.rs:141-142).  eps 1e-20, 32-wide blocks.
+extern "C" __global__ void __launch_bounds__(256) hc_combine_norm_quant(const uint16_t* X, const float* P, const uint16_t* W, uint16_t* Y, uint8_t* Q,
+                                                                        uint8_t* SR, uint8_t* SM, const void*, const void*) {
+    tf_hc_norm_quant_row(X, P, W, Y, nullptr, nullptr, Q, SR, SM, RL_HIDDEN, 4, 32, 1.0e-20f);
+}
+// The boundary operator `hc_post_b128_w1` (symbol hc_post_tiles; runtime/kernels/mhc-post-tiles-v1/mhc-post-tiles.py:11-27,
+// src/mhc.rs:1223-1234): grid (rows, tiles), any block; a block takes 5,120 / tiles columns of its row, 8 a thread.
+extern "C" __global__ void hc_post_tiles(const uint16_t* A, const uint16_t* R, const float* POST, const float* C, uint16_t* Y, const void*,
+                                         const void*) {
+    constexpr int PER_ROW = RL_HIDDEN / 8;
+    const int tile_pieces = (PER_ROW + (int)gridDim.y - 1) / (int)gridDim.y, first = (int)blockIdx.y * tile_pieces;
+    const size_t row = blockIdx.x;
+    for (int q = first + (int)threadIdx.x; q < min(first + tile_pieces, PER_ROW); q += (int)blockDim.x)
+        tf_hc_post_piece(reinterpret_cast<const u4v*>(A + row * RL_HIDDEN)[q], R, POST, C, Y, row, q, RL_HIDDEN);
 }
 
 // kernels/core.cu:25-28 (src/mhc.rs:79: one block of 32 threads with a stated amount of dynamic LDS): a launch that starts

@@ -16,7 +16,7 @@ EXPORTS = ["ca_ffn_abi", "ca_ffn_configure", "ca_ffn_geometry", "ca_router_logit
            "ca_primitives_entries", "ca_primitives_scratch_bytes", "ca_primitives_marks", "ca_encode", "ca_decode", "ca_local_live",
            "ca_pack_bf16", "ca_primitives_spin_limit", "ca_primitives_open_geometry", "ca_primitives_geometry", "ca_router_logits_in",
            "ca_router_logits_wide_in", "ca_shared_swiglu_in", "ca_ffn_add_in", "ca_moe_dynamic_static", "ca_moe_dynamic_static_capacity",
-           "ca_ffn_norm_quant", "ca_ffn_sum_residual"]
+           "ca_ffn_norm_quant", "ca_ffn_sum_residual", "ca_hc_combine_norm_quant", "ca_hc_post", "ca_ffn_sum_hc_post"]
 
 
 class Geometry(ctypes.Structure):
@@ -90,6 +90,9 @@ def load():
     lib.ca_ffn_add_in.argtypes = [vp, ctypes.c_int, vp, vp, vp, vp]
     lib.ca_ffn_norm_quant.argtypes = [vp, ctypes.c_int, vp, vp, ctypes.c_float, vp, vp, vp, vp, vp, vp]
     lib.ca_ffn_sum_residual.argtypes = [vp, ctypes.c_int, ctypes.c_int, vp, vp, vp, vp, vp, vp, vp]
+    lib.ca_hc_combine_norm_quant.argtypes = [vp, ctypes.c_int, ctypes.c_int, vp, vp, vp, vp, vp, vp, vp, vp, vp, vp]
+    lib.ca_hc_post.argtypes = [vp, ctypes.c_int, vp, vp, vp, vp, vp, vp]
+    lib.ca_ffn_sum_hc_post.argtypes = [vp, ctypes.c_int, ctypes.c_int, vp, vp, vp, vp, vp, vp, vp, vp, vp]
     _lib = lib
     return lib
 
