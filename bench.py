@@ -7,14 +7,14 @@ A step is one pass of the whole layer (gate product, top-k + plan + token quanti
 expert, ordered sum + shared addition) over one batch of synthetic token rows that is already resident in HBM, replayed
 as a captured HIP graph as the reference replays its layer (src/probe.rs:1527-1542).  Sixteen distinct input batches
 (two at many rows) are cycled so every step routes to other experts and streams their weights from HBM, not from the last
-step's cache.  A graph holds one pass over each batch, so --steps and --warmup are rounded up to whole replays; the line
-says so and carries the numbers that ran.
+step's cache.  A graph holds one pass over each batch; a step count that is no multiple of the batch count ends with a
+shorter graph over the first batches, so exactly --steps steps are timed after exactly --warmup warm-up steps.
 
 Prints ONE JSON line.  Without --config its top level is the decode step (c2, the configuration the metric is quoted on):
 whole-layer tokens/s, the roofline of the dominant kernel (FC1 + SwiGLU of the routed experts; algorithmic bytes over its
 average duration, measured with two HIP events that take the kernel's start and completion on its launch stream), and the
 CPU baseline (the C oracle, a port of the reference semantics: the reference has no CPU path) timed on a bounded sample of
-the same workload, with all threads and with one.  `configs` then holds the same measurement of the speculative-verify step
+the same workload: its vectorised build with all threads (the reported value), the scalar build with all threads and with one.  `configs` then holds the same measurement of the speculative-verify step
 (c3) and the two prefill chunks (c4, c5: the routed FC1 launch between events recorded around it; its flops a byte say which
 roof it lies under: at 4,096 rows an expert's weights serve 96 rows, 339 flop/B against the machine's 625, so HBM; at 16,384
 rows the matrix units; the line carries the fractions of both peaks either way).  With --config only that configuration runs and is the top level.
@@ -85,37 +85,46 @@ def cpu_model():
     return "unknown"
 
 
-def cpu_baseline(pkg, g, ops, xs, taps_ids, budget_s=15.0, single_budget_s=8.0):
-    """Times the C oracle (staged, active experts only) on host cores for a bounded number of steps: with every thread the
-    process may use (at most 16), then with one thread (the scalar figure)."""
+def cpu_baseline(pkg, g, ops, xs, taps_ids, budget_s=12.0, scalar_budget_s=8.0, single_budget_s=8.0):
+    """Times the C oracle (staged, active experts only) on host cores for a bounded number of steps: its vectorised build
+    (AVX2 + FMA projection loops, OpenMP over weight rows) with every thread the process may use (at most 16) -- the reported
+    value --, then the scalar oracle with the same threads and with one thread."""
     sys.path.insert(0, os.path.join(ROOT, "tests"))
     import oracle
     import helpers
     allowed = len(os.sched_getaffinity(0)) if hasattr(os, "sched_getaffinity") else (os.cpu_count() or 1)
     threads = max(1, min(allowed, 16))
     rows = xs[0].shape[0]
+    # gather the operands the steps touch outside the timed regions (the oracle reads host memory)
+    subsets = [_HostSubset(ops, ids, g) for ids in taps_ids]
+    host_xs = [x.cpu() for x in xs]
 
-    def timed(n_threads, budget):
+    def timed(n_threads, budget, simd):
         oracle.set_threads(n_threads)
         done, spent = 0, 0.0
         while done < 4 * len(xs) and (done == 0 or spent + spent / done < budget):
-            x = xs[done % len(xs)]
-            # gather the operands the step touches outside the timed region (the oracle reads host memory)
-            small_ops = _HostSubset(ops, taps_ids[done % len(xs)], g)
             t0 = time.perf_counter()
-            helpers.oracle_layer(g, small_ops, x.cpu())
+            helpers.oracle_layer(g, subsets[done % len(xs)], host_xs[done % len(xs)], simd=simd)
             spent += time.perf_counter() - t0
             done += 1
         return done, spent
 
-    done, spent = timed(threads, budget_s)
-    done1, spent1 = timed(1, single_budget_s)
+    simd = oracle.simd_available()
+    if simd:
+        timed(threads, 0.0, True)           # first touch of the operands
+    done, spent = timed(threads, budget_s, simd)
+    done_s, spent_s = timed(threads, scalar_budget_s, False)
+    done1, spent1 = timed(1, single_budget_s, False)
     oracle.set_threads(threads)
+    build = "vectorised C oracle (AVX2 + FMA projection loops)" if simd else "scalar C oracle (the host has no AVX2 + FMA)"
     return {"value": rows * done / spent, "unit": "tokens/s", "cores": threads, "threads": threads, "kind": "port",
             "nproc": os.cpu_count(), "cpus_allowed": allowed, "cpu_model": cpu_model(),
-            "sample": "%d steps of this workload (%d rows each), C oracle with %d OpenMP threads, %.1f s" % (done, rows, threads, spent),
+            "sample": "%d steps of this workload (%d rows each), %s with %d OpenMP threads, %.1f s" % (done, rows, build, threads, spent),
+            "scalar": {"value": rows * done_s / spent_s, "unit": "tokens/s", "cores": threads,
+                       "sample": "%d steps of this workload, the scalar C oracle (one look-up and one fused multiply-add a product) with %d OpenMP threads, %.1f s"
+                                 % (done_s, threads, spent_s)},
             "single_thread": {"value": rows * done1 / spent1, "unit": "tokens/s", "cores": 1,
-                              "sample": "%d steps of this workload, the same C oracle with one thread, %.1f s" % (done1, spent1)}}
+                              "sample": "%d steps of this workload, the same scalar C oracle with one thread, %.1f s" % (done1, spent1)}}
 
 
 class _HostSubset:
@@ -143,7 +152,10 @@ class _Sparse:
 
     def __getitem__(self, ids):
         import torch
-        return self.data[torch.as_tensor([self.index[int(e)] for e in ids], dtype=torch.long)]
+        at = [self.index[int(e)] for e in ids]
+        if at == list(range(self.data.shape[0])):      # the held experts in their own order: no copy
+            return self.data
+        return self.data[torch.as_tensor(at, dtype=torch.long)]
 
 
 def geometry_of(native, cfg, numerics):
@@ -244,13 +256,21 @@ def measure(pkg, name, numerics, steps, warmup, profile_steps, overlap, operands
     max_load = float(np.mean([np.bincount(ids[ids >= 0].ravel(), minlength=E).max() for ids in ids_per_batch]))
 
     # whole-layer throughput: one graph holds a pass over each of the input batches (as the reference's graph holds its forty
-    # layers' passes); a step is one pass, so steps and warmup are rounded up to whole replays
-    asked = (steps, warmup)
-    graph = layer.capture(xs)
+    # layers' passes); a step is one pass.  Step counts that are no multiple of the batch count end with a shorter graph over
+    # the first batches, so exactly the steps asked for run, in the warm-up and in the timed region
+    full = layer.capture(xs)
+    tails = {}
+
+    def launches(count):
+        order = [full] * (count // batches)
+        if count % batches:
+            if count % batches not in tails:
+                tails[count % batches] = layer.capture(xs[:count % batches])
+            order.append(tails[count % batches])
+        return order
+    warm_order, timed_order = launches(warmup), launches(steps)
     torch.cuda.synchronize()
-    replays, warm = -(-steps // batches), -(-warmup // batches)
-    steps, warmup = replays * batches, warm * batches
-    ms = layer.time([graph], warm, replays)
+    ms = layer.time(warm_order + timed_order, len(warm_order), len(timed_order))
     torch.cuda.synchronize()
     ms_per_step = ms / steps
     value = rows / (ms_per_step * 1e-3)
@@ -287,7 +307,7 @@ def measure(pkg, name, numerics, steps, warmup, profile_steps, overlap, operands
                     "timing": "HIP events bound to the kernel's start and completion (hipExtLaunchKernelGGL) on its launch stream, eager passes of the layer's schedule"}
     record = {
         "value": value, "unit": "tokens/s", "steps": steps, "warmup": warmup, "ms_per_step": ms_per_step,
-        "steps_note": "asked for %d steps after %d warm-up steps; rounded up to whole replays of the %d-pass graph" % (asked[0], asked[1], batches),
+        "steps_note": "%d steps after %d warm-up steps: replays of a %d-pass graph, a shorter graph for the remainder" % (steps, warmup, batches),
         "config": {"workload": name + ": " + cfg["workload"],
                    "numerics": ("sigmoid top-k renormalised, 128-wide activation blocks" if numerics == "benchmark" else
                                 "reference numerics: sqrt-softplus scores x 1.5, 32-wide activation blocks, 32 x 32 shared weight blocks"),

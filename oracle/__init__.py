@@ -53,6 +53,7 @@ def lib():
             getattr(_lib, name).argtypes = args
         _lib.orc_scale_code1_check.restype = ctypes.c_uint32
         _lib.orc_scale_codes4.restype = ctypes.c_uint32
+        _lib.orc_simd_available.restype = ctypes.c_int32
     return _lib
 
 
@@ -206,32 +207,43 @@ def shared_swiglu_quant(x, block, limit=10.0):
     return act, codes, scales
 
 
-def fp8_linear(aq, a_scales, act_block, wq, w_scales, bn, bk):
+def simd_available():
+    """Whether the host has AVX2 + FMA, i.e. whether `simd=True` may be passed to the three projection functions."""
+    return bool(lib().orc_simd_available())
+
+
+def _projection(name, simd):
+    if simd and not simd_available():
+        raise RuntimeError("the vectorised oracle loops need AVX2 + FMA")
+    return getattr(lib(), ("orc_simd_" if simd else "orc_") + name)
+
+
+def fp8_linear(aq, a_scales, act_block, wq, w_scales, bn, bk, simd=False):
     aq, a_scales, wq, w_scales = _c(aq, np.uint8), _c(a_scales, np.uint8), _c(wq, np.uint8), _c(w_scales, np.uint8)
     rows, k = aq.shape
     n = wq.shape[0]
     out = np.empty((rows, n), np.uint16)
-    lib().orc_fp8_linear(_p(aq), _p(a_scales), _i32(act_block), _p(wq), _p(w_scales), _i32(bn), _i32(bk), _i32(rows),
+    _projection("fp8_linear", simd)(_p(aq), _p(a_scales), _i32(act_block), _p(wq), _p(w_scales), _i32(bn), _i32(bk), _i32(rows),
                          _i32(n), _i32(k), _p(out))
     return out
 
 
 # ---- routed experts ---------------------------------------------------------------------------------------------------
-def expert_fc1(cfg, xq, xs, w13, s13, ids, want_proj=False):
+def expert_fc1(cfg, xq, xs, w13, s13, ids, want_proj=False, simd=False):
     xq, xs, w13, s13, ids = _c(xq, np.uint8), _c(xs, np.uint8), _c(w13, np.uint8), _c(s13, np.uint8), _c(ids, np.int32)
     rows = xq.shape[0]
     h = np.empty((rows, cfg.topk, cfg.inter), np.uint16)
     proj = np.empty((rows, cfg.topk, 2 * cfg.inter), np.float32) if want_proj else None
-    lib().orc_expert_fc1(ctypes.byref(cfg), _p(xq), _p(xs), _p(w13), _p(s13), _p(ids), _i32(rows), _p(h), _p(proj))
+    _projection("expert_fc1", simd)(ctypes.byref(cfg), _p(xq), _p(xs), _p(w13), _p(s13), _p(ids), _i32(rows), _p(h), _p(proj))
     return (h, proj) if want_proj else h
 
 
-def expert_fc2(cfg, hq, hs, w2, s2, ids, weights):
+def expert_fc2(cfg, hq, hs, w2, s2, ids, weights, simd=False):
     hq, hs, w2, s2 = _c(hq, np.uint8), _c(hs, np.uint8), _c(w2, np.uint8), _c(s2, np.uint8)
     ids, weights = _c(ids, np.int32), _c(weights, np.float32)
     rows = ids.shape[0]
     out = np.empty((rows, cfg.topk, cfg.hidden), np.uint16)
-    lib().orc_expert_fc2(ctypes.byref(cfg), _p(hq), _p(hs), _p(w2), _p(s2), _p(ids), _p(weights), _i32(rows), _p(out))
+    _projection("expert_fc2", simd)(ctypes.byref(cfg), _p(hq), _p(hs), _p(w2), _p(s2), _p(ids), _p(weights), _i32(rows), _p(out))
     return out
 
 

@@ -92,6 +92,16 @@ void orc_expert_fc1(const orc_config* c, const uint8_t* xq, const uint8_t* xs, c
 void orc_expert_fc2(const orc_config* c, const uint8_t* hq, const uint8_t* hs, const uint8_t* w2, const uint8_t* s2,
                     const int32_t* ids, const float* weights, int32_t rows, uint16_t* route_out);
 
+/* vectorised (AVX2 + FMA, OpenMP) forms of the three loops above for the CPU baseline: same outputs up to the summation order
+ * inside a 32-wide block (tf_oracle_simd.c).  Call only where orc_simd_available() returns non-zero. */
+int32_t orc_simd_available(void);
+void orc_simd_expert_fc1(const orc_config* c, const uint8_t* xq, const uint8_t* xs, const uint8_t* w13,
+                         const uint8_t* s13, const int32_t* ids, int32_t rows, uint16_t* h, float* proj);
+void orc_simd_expert_fc2(const orc_config* c, const uint8_t* hq, const uint8_t* hs, const uint8_t* w2, const uint8_t* s2,
+                         const int32_t* ids, const float* weights, int32_t rows, uint16_t* route_out);
+void orc_simd_fp8_linear(const uint8_t* aq, const uint8_t* as, int32_t act_block, const uint8_t* wq, const uint8_t* ws,
+                         int32_t bn, int32_t bk, int32_t rows, int32_t n, int32_t k, uint16_t* out);
+
 /* ---- combine -------------------------------------------------------------------------------- */
 void orc_topk_sum(const uint16_t* routes, uint16_t* routed, int32_t rows, int32_t topk, int32_t hidden,
                   int32_t live);

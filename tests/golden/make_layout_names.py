@@ -18,6 +18,17 @@ DTYPES = {"F32": "F32", "Bf16": "BF16", "Fp8": "F8_E4M3", "E8m0": "F8_E8M0", "Pa
 HIDDEN = 5120            # config.text_config.hidden_size of the reference's model (runtime/model/config.json)
 
 
+def number(expr, bindings):
+    """A shape entry `name` or `name / digits` (a loop variable or a literal, optionally divided) as an integer; anything else
+    in the reference's text is refused, nothing of it is evaluated."""
+    m = re.fullmatch(r"(\w+)(?:\s*/\s*(\d+))?", expr.strip())
+    if not m:
+        raise ValueError("unexpected shape expression in the reference's contract: %r" % expr)
+    head, div = m.group(1), m.group(2)
+    base = bindings[head] if head in bindings else int(head)
+    return base // int(div) if div else base
+
+
 def symbolic(expr, value, bindings):
     """A shape entry as an expression in H, E, I: loop variables by their value's meaning, literals by their value."""
     names = {HIDDEN: "H", 384: "E", 2304: "I"}
@@ -53,7 +64,7 @@ def main():
             if tname is not None:
                 bind["n"] = HIDDEN if n == "d" else int(n)
                 bind["k"] = HIDDEN if k == "d" else int(k)
-            numbers = [eval(d.replace("/", "//"), {}, dict(bind)) for d in dims]
+            numbers = [number(d, bind) for d in dims]
             entries.append({"name": name.replace("{name}", tname) if tname else name, "dtype": DTYPES[dtype], "shape": numbers,
                             "dims": [symbolic(d, None, bind) for d in dims]})
     experts = int(re.search(r"for e in 0\.\.(\d+)", text).group(1))

@@ -182,9 +182,10 @@ class GpuLayer:
         return out
 
 
-def oracle_layer(g, ops, x, tokens=None, live=None, padding=None, logits=None, ids_weights=None):
+def oracle_layer(g, ops, x, tokens=None, live=None, padding=None, logits=None, ids_weights=None, simd=False):
     """Stage-by-stage oracle evaluation; routed experts are evaluated on the active experts only (ids remapped), so
-    configs with hundreds of experts stay cheap.  `logits` / `ids_weights` substitute the GPU's own upstream results."""
+    configs with hundreds of experts stay cheap.  `logits` / `ids_weights` substitute the GPU's own upstream results.
+    `simd`: the three projection loops in their vectorised form (the CPU baseline; another summation order inside a block)."""
     cfg = oracle_config(g)
     rows = x.shape[0]
     K, I, H, B = g.topk, g.intermediate, g.hidden, g.act_block
@@ -207,13 +208,13 @@ def oracle_layer(g, ops, x, tokens=None, live=None, padding=None, logits=None, i
     pick = torch.as_tensor(active if active else [0], dtype=torch.long)
     w13, s13 = np_of(ops.w13[pick.to(ops.w13.device)]), np_of(ops.s13[pick.to(ops.s13.device)])
     w2, s2 = np_of(ops.w2[pick.to(ops.w2.device)]), np_of(ops.s2[pick.to(ops.s2.device)])
-    t["h"] = oracle.expert_fc1(small, t["xq"], t["xs"], w13, s13, ids_small)
+    t["h"] = oracle.expert_fc1(small, t["xq"], t["xs"], w13, s13, ids_small, simd=simd)
     hq, hs = oracle.quantize_rows(t["h"].reshape(rows * K, I), B, 0.0)
     t["hq"], t["hs"] = hq.reshape(rows, K, I), hs.reshape(rows, K, I // B)
-    t["route_out"] = oracle.expert_fc2(small, t["hq"], t["hs"], w2, s2, ids_small, t["weights"])
-    t["shared_up"] = oracle.fp8_linear(t["xq_min"], t["xs_min"], B, np_of(ops.sh_w13), np_of(ops.sh_s13), g.shared_bn, g.shared_bk)
+    t["route_out"] = oracle.expert_fc2(small, t["hq"], t["hs"], w2, s2, ids_small, t["weights"], simd=simd)
+    t["shared_up"] = oracle.fp8_linear(t["xq_min"], t["xs_min"], B, np_of(ops.sh_w13), np_of(ops.sh_s13), g.shared_bn, g.shared_bk, simd=simd)
     t["shared_act"], t["shared_aq"], t["shared_as"] = oracle.shared_swiglu_quant(t["shared_up"], B, g.swiglu_limit)
-    t["shared_down"] = oracle.fp8_linear(t["shared_aq"], t["shared_as"], B, np_of(ops.sh_w2), np_of(ops.sh_s2), g.shared_bn, g.shared_bk)
+    t["shared_down"] = oracle.fp8_linear(t["shared_aq"], t["shared_as"], B, np_of(ops.sh_w2), np_of(ops.sh_s2), g.shared_bn, g.shared_bk, simd=simd)
     n_live = rows if live is None else min(live, rows)
     t["routed"], t["out"] = oracle.ffn_sum_shared(t["route_out"], t["shared_down"], n_live)
     return t

@@ -150,6 +150,32 @@ def test_shared_swiglu_and_add_entry_points():
     assert np.array_equal(u16(out), oracle.ffn_add(u16(a), u16(b)))
 
 
+def test_topk_sum_entry_takes_its_live_rows_from_active_m_alone():
+    # entry 2 (moe.w4a16.topk_sum): rows below the scalar active_m are summed, the others keep the buffer's contents; the third
+    # pointer is bound to the output buffer by the contracts (as the reference binds its node's spare pointers) and is never read
+    # as a live count -- BF16 bits there must not change the result
+    import ctypes
+    from helpers import geometry
+    g = geometry(1024, 16, 6, 512, 512, "benchmark")
+    ctx = native.open_context(g)
+    lib = native.load()
+    rows, live = 8, 5
+    routes = synth.to_bf16_bits(synth.normal("entry2/routes", (rows, g.topk, g.hidden))).cuda()
+    out = torch.full((rows, g.hidden), 0x3c00, dtype=torch.int16, device="cuda")
+    pointers = (ctypes.c_uint64 * 3)(routes.data_ptr(), out.data_ptr(), out.data_ptr())
+    scalars = (ctypes.c_int32 * 3)(live, 0, 0)
+    assert lib.ca_primitives_launch(ctypes.c_void_p(ctx), 2, pointers, 3, scalars, 3, None) == 0
+    torch.cuda.synchronize()
+    want = oracle.topk_sum(u16(routes), live=live, previous=np.full((rows, g.hidden), 0x3c00, np.uint16))
+    assert np.array_equal(u16(out), want) and np.all(u16(out)[live:] == 0x3c00)
+    pointers = (ctypes.c_uint64 * 3)(routes.data_ptr(), out.data_ptr(), 0)          # a null third pointer is as good
+    scalars = (ctypes.c_int32 * 3)(rows, 0, 0)
+    assert lib.ca_primitives_launch(ctypes.c_void_p(ctx), 2, pointers, 3, scalars, 3, None) == 0
+    torch.cuda.synchronize()
+    assert np.array_equal(u16(out), oracle.topk_sum(u16(routes)))
+    lib.ca_primitives_close(ctypes.c_void_p(ctx))
+
+
 def test_group_sum_rows_layout():
     hidden, topk, quarter, per, group, live = 1024, 6, 8, 4, 1, 27
     routes = synth.to_bf16_bits(synth.normal("group/routes", (32, topk, hidden)))

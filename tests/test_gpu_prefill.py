@@ -45,13 +45,18 @@ def test_wide_live_rows_and_skewed_routing():
     layer.close()
 
 
-@pytest.mark.parametrize("config", ["c4", "c5"])
-def test_full_size_prefill(config):
+@pytest.mark.parametrize("case", ["c4", "c4-uniform", "c5"])
+def test_full_size_prefill_row_sample_and_plan_invariants(case):
+    # the oracle runs on a sample of rows (sixteen spread over the batch and eight of the busiest expert's ragged last tile);
+    # every row is covered by the plan invariants here and by the permutation property below
+    config = case.split("-")[0]
     c = CONFIGS[config]
     g = geometry(c["hidden"], c["experts"], c["topk"], c["inter"], c["shared"], "benchmark")
     ops = synth.LayerOperands(g, config, device="cuda")
     if config == "c5":       # expert popularity ~ rank^-1.1 through the selection bias, as the benchmark sets it
         ops.bias = synth.zipf_bias(g.experts, 1.1, 0.06, device="cuda")
+    if case == "c4-uniform":  # the benchmark's c4: uniform routing, no selection bias (every expert active, about 96 rows each)
+        ops.bias = torch.zeros_like(ops.bias)
     rows = c["rows"]
     x = synth.activations(config, rows, g.hidden, device="cuda")
     layer = GpuLayer(g, ops, rows)
@@ -60,6 +65,9 @@ def test_full_size_prefill(config):
     if config == "c5":
         counts = np.bincount(taps["ids"].ravel(), minlength=g.experts)
         assert counts.max() > 10 * counts.mean(), "the busiest expert must take more than ten times the mean load"
+    if case == "c4-uniform":
+        counts = np.bincount(taps["ids"].ravel(), minlength=g.experts)
+        assert counts.min() > 0 and counts.max() < 2 * counts.mean(), "uniform routing: every expert active, none far above the mean"
     sample = np.arange(0, rows, rows // 16)[:16]
     # and rows of the busiest expert's last tile, the ragged one (partly filled; at 16,384 rows also the last of a 256-row
     # unit of two tiles): their routes run through the GEMM's short-tile variants

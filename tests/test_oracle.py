@@ -452,3 +452,38 @@ def test_layer_c_function_agrees_with_staged_evaluation_and_float64():
     got = bf(staged["out"])
     assert np.abs(got - ref).max() <= 0.06 * np.abs(ref).max()
     assert np.corrcoef(got.ravel(), ref.ravel())[0, 1] > 0.995    # FP8 activation noise; a swapped gate / up order or operand gives < 0.9
+
+
+@pytest.mark.skipif(not oracle.simd_available(), reason="the vectorised oracle loops need AVX2 + FMA")
+@pytest.mark.parametrize("mode", ["benchmark", "reference"])
+def test_vectorised_projection_loops_against_the_scalar_oracle(mode):
+    # the CPU baseline's build of the three projection loops: the same operands and roundings, a block's 32 products summed in
+    # eight lanes instead of one chain.  Against the scalar oracle: every BF16 output within one BF16 step (almost all equal),
+    # and against float64 on the dequantized operands as close as the scalar oracle is
+    import helpers
+    g = helpers.geometry(1024, 16, 2, 512, 512, mode)
+    ops = helpers.synth.LayerOperands(g, "simd-" + mode, device="cpu")
+    x = helpers.synth.activations("simd-" + mode, 12, g.hidden)
+    scalar = helpers.oracle_layer(g, ops, x)
+    fast = helpers.oracle_layer(g, ops, x, ids_weights=(scalar["ids"], scalar["weights"]), simd=True)
+    for name in ["h", "shared_up", "shared_down"]:
+        assert helpers.bf16_ulp_distance(fast[name], scalar[name]) <= 1.0, name
+        assert np.mean(fast[name] != scalar[name]) < 0.01, name
+    # downstream of a BF16 value that moved one step the FP8 codes of its block may move too; given the same codes FC2 agrees
+    cfg = helpers.oracle_config(g)
+    again = oracle.expert_fc2(cfg, scalar["hq"], scalar["hs"], helpers.np_of(ops.w2), helpers.np_of(ops.s2), scalar["ids"], scalar["weights"], simd=True)
+    assert helpers.bf16_ulp_distance(again, scalar["route_out"]) <= 1.0 and np.mean(again != scalar["route_out"]) < 0.01
+    r = helpers.error_stats(fast["out"], scalar["out"])
+    assert r[0] <= 1e-2 and r[1] <= 1e-3
+    # special values of the bit-arithmetic E4M3 decode: every code against the table decode, through a one-hot product
+    codes = np.arange(256, dtype=np.uint8)
+    k = 512
+    wq = np.zeros((256, k), np.uint8)
+    wq[np.arange(256), 7] = codes                                  # weight row j holds code j at column 7
+    aq = np.zeros((1, k), np.uint8)
+    aq[0, 7] = 0x38                                                # 1.0
+    ones = np.full((1, k // 32), 127, np.uint8)
+    ws = np.full((256 // 32, k // 32), 127, np.uint8)
+    a = oracle.fp8_linear(aq, ones, 32, wq, ws, 32, 32)
+    b = oracle.fp8_linear(aq, ones, 32, wq, ws, 32, 32, simd=True)
+    assert np.array_equal(a, b)

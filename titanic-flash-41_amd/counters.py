@@ -25,11 +25,12 @@ import sys
 HERE = os.path.dirname(os.path.abspath(__file__))
 ROOT = os.path.dirname(HERE)
 COPY_BYTES = 256 << 20
-# rows, passes, batches, copies, skew: the probe's arguments.  16,384 rows: the skew that gives the probe's operands the
-# benchmark workload's shape (every expert active, about 911 tiles of 128 rows, the same algorithmic bytes).
+# rows, passes, batches, copies, skew, rows a request: the probe's arguments.  16,384 rows: the skew that gives the probe's
+# operands the benchmark workload's shape (every expert active, about 911 tiles of 128 rows, the same algorithmic bytes).
+# 32 rows: four requests of eight draft tokens whose routes overlap as the benchmark's correlated rows do (about 40 tiles).
 WORKLOADS = {
     "c2": ("4", "64", "16", "4", "0"),
-    "c3": ("32", "64", "16", "4", "0"),
+    "c3": ("32", "64", "16", "4", "0", "8"),
     "c4": ("4096", "6", "2", "4", "0"),
     "c5": ("16384", "4", "2", "4", "0.02"),
 }

@@ -41,10 +41,10 @@
 // Lane l of the wave copies 16 (4) bytes from global address base + offset (a scalar base, the lane's own 32-bit byte
 // offset) to LDS byte address lds_base + 16 l (4 l).
 __device__ __forceinline__ void tf_dma16(const uint8_t* base, uint32_t offset, uint32_t lds_base) {
-    asm volatile("s_mov_b32 m0, %2\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %0, %1" ::"v"(offset), "s"(base), "s"(lds_base) : "memory");
+    asm volatile("s_mov_b32 m0, %2\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %0, %1" ::"v"(offset), "s"(base), "s"(lds_base) : "memory", "m0");
 }
 __device__ __forceinline__ void tf_dma4(const uint8_t* base, uint32_t offset, uint32_t lds_base) {
-    asm volatile("s_mov_b32 m0, %2\n\ts_nop 0\n\tglobal_load_lds_dword %0, %1" ::"v"(offset), "s"(base), "s"(lds_base) : "memory");
+    asm volatile("s_mov_b32 m0, %2\n\ts_nop 0\n\tglobal_load_lds_dword %0, %1" ::"v"(offset), "s"(base), "s"(lds_base) : "memory", "m0");
 }
 template <int N>
 __device__ __forceinline__ void tf_wait_vm() { asm volatile("s_waitcnt vmcnt(%0)" ::"n"(N) : "memory"); }

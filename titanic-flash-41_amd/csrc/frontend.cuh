@@ -218,8 +218,10 @@ __device__ __forceinline__ void tf_route_frontend(
         }
         __syncthreads();
         if (!last) return;
-        tf_route_block(logits, bias, bias_alt, tokens, live, nullptr, ids, weights, min(owner_rows, first_row + 4), p, first_row, waves, false,
-                       nullptr, nullptr, true);
+        // rows with a padding source are block 0's to write (from their source's routes): a group router that is still running
+        // after block 0's wait has expired must not write over them
+        tf_route_block(logits, bias, bias_alt, tokens, live, padding, ids, weights, min(owner_rows, first_row + 4), p, first_row, waves, false,
+                       nullptr, nullptr, true, true);
         tf_stores_done();
         __syncthreads();
         if (threadIdx.x == 0) atomicAdd(routed_groups, 1u);

@@ -66,9 +66,9 @@ extern "C" __global__ void ca_moe_nibble_permute_words(uint32_t* words, unsigned
 // [width]).  Output per matrix: the base word b * 0x01010101 (b = the commonest byte, or the byte below it when that one is
 // more common than the byte above); per unit 16 code words (bit 4 (r % 8) + j of word r / 8: byte j of row r is b + 1) and
 // 4 flag words (bit r % 32 of word r / 32: row r holds a byte outside {b, b + 1} and stays raw).
-// One workgroup of four waves a matrix.  The byte counts are taken a wave of bytes at a time by matching: the lanes that
+// One workgroup of (up to) four waves a matrix.  The byte counts are taken a wave of bytes at a time by matching: the lanes that
 // hold the same byte as the first lane still open are counted with one ballot and closed together (scale bytes take a
-// handful of values, so a wave's 64 bytes close in two or three rounds); the 256 counts are then ranked by all 256 threads
+// handful of values, so a wave's 64 bytes close in two or three rounds); the 256 counts are then ranked by all threads
 // at once (largest count, lowest byte on a tie, as one packed key).  A wave then codes a unit at a time, 64 rows a pass: a
 // row's four bits meet the seven other rows of its code word through three lane exchanges, and a pass's raw rows are one
 // ballot, which is the flag word pair.
@@ -91,9 +91,10 @@ __device__ __forceinline__ uint32_t tf_row_bits(uint32_t word, int width, uint32
 extern "C" __global__ void __launch_bounds__(256) ca_expert_scale_code1(const uint8_t* scales, uint32_t* code, uint32_t* flags, uint32_t* bases,
                                                                         int n, int columns) {
     __shared__ uint32_t s_count[4][256];          // a table a wave
-    __shared__ uint32_t s_best[4];
+    __shared__ unsigned long long s_best[4];
     __shared__ uint32_t s_total[256];
-    const int t = threadIdx.x, lane = t & 63, wave = t >> 6, waves = blockDim.x >> 6;
+    // any block of one to four whole waves (the reference launches 256 threads)
+    const int t = threadIdx.x, lane = t & 63, wave = t >> 6, threads = (int)blockDim.x, waves = threads >> 6;
     const int matrix = blockIdx.x, tiles = (n + 127) / 128, slices = (columns + 3) / 4;
     const uint8_t* bytes = scales + (size_t)matrix * n * columns;
     const int total = n * columns;
@@ -112,18 +113,24 @@ extern "C" __global__ void __launch_bounds__(256) ca_expert_scale_code1(const ui
         }
     }
     __syncthreads();
-    // thread v ranks byte v: key = count << 8 | (255 - v), so the largest key is the largest count and, on a tie, the lowest byte
-    uint32_t mine = 0;
-    if (t < 256) {
-        for (int w = 0; w < waves; ++w) mine += s_count[w][t];
-        s_total[t] = mine;
+    // a thread ranks bytes t, t + threads, ..: key = count << 8 | (255 - byte) in 64 bits (a matrix may hold 2^24 scale bytes and
+    // more), so the largest key is the largest count and, on a tie, the lowest byte
+    unsigned long long key = 0;
+    for (int v = t; v < 256; v += threads) {
+        uint32_t mine = 0;
+        for (int w = 0; w < waves; ++w) mine += s_count[w][v];
+        s_total[v] = mine;
+        const unsigned long long candidate = ((unsigned long long)mine << 8) | (unsigned long long)(255 - v);
+        key = candidate > key ? candidate : key;
     }
-    uint32_t key = t < 256 ? (mine << 8) | (uint32_t)(255 - t) : 0u;
 #pragma unroll
-    for (int o = 32; o > 0; o >>= 1) key = max(key, (uint32_t)__shfl_xor((int)key, o));
+    for (int o = 32; o > 0; o >>= 1) {
+        const unsigned long long other = ((unsigned long long)(uint32_t)__shfl_xor((int)(key >> 32), o) << 32) | (uint32_t)__shfl_xor((int)(uint32_t)key, o);
+        key = other > key ? other : key;
+    }
     if (lane == 0) s_best[wave] = key;
     __syncthreads();
-    for (int w = 0; w < waves; ++w) key = max(key, s_best[w]);
+    for (int w = 0; w < waves; ++w) key = s_best[w] > key ? s_best[w] : key;
     const int commonest = 255 - (int)(key & 255u);
     const bool below = commonest > 0 && (commonest == 255 || s_total[commonest - 1] > s_total[commonest + 1]);
     const uint32_t b = (uint32_t)(below ? commonest - 1 : commonest);

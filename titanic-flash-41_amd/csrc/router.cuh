@@ -214,13 +214,14 @@ __device__ __forceinline__ void tf_apply_padding(const int32_t* padding, int32_t
 }
 
 // Routes rows [first_row, first_row + waves of this block) of `rows`; rows at or past min(rows, live[0]) get ids -1 and
-// weights 0.  `padding` (may be null) is applied only by a single-block launch, after a block barrier.
+// weights 0.  `padding` (may be null) is applied only by a single-block launch, after a block barrier.  `leave_padded`: rows
+// with a padding source are not written at all (another workgroup of the launch writes them, with their source's experts).
 template <bool COHERENT = true>
 __device__ __forceinline__ void tf_route_block(const float* logits, const float* bias, const float* bias_alt,
                                                const long long* tokens, const int32_t* live, const int32_t* padding,
                                                int32_t* ids, float* weights, int rows, const RouteParams& p,
                                                int first_row, int row_stride, bool apply_padding, int32_t* s_ids = nullptr,
-                                               float* s_weights = nullptr, bool publish = false) {
+                                               float* s_weights = nullptr, bool publish = false, bool leave_padded = false) {
     const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
     const int live_count = live[0];
     const bool has_alt = bias_alt != nullptr && tokens != nullptr && p.alt_token >= 0;
@@ -241,6 +242,7 @@ __device__ __forceinline__ void tf_route_block(const float* logits, const float*
         }
         const long long token = has_alt ? tokens[row] : -1;
         const bool is_live = row < min(rows, live_count);
+        if (leave_padded && padding != nullptr && padding[row] >= 0) continue;       // uniform over the wave: one row a wave
         int32_t chosen[8];
         float share[8];
         if (is_live) {

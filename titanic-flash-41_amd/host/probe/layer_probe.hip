@@ -1,10 +1,12 @@
 // Stand-alone driver of the layer for profilers: no Python, no PyTorch, only the host mirror's C API and the HIP runtime.
 //
-//   tf_layer_probe <libtitanic_moe_hip.so> [rows=4] [passes=64] [batches=16] [copies=4] [skew=0]
+//   tf_layer_probe <libtitanic_moe_hip.so> [rows=4] [passes=64] [batches=16] [copies=4] [skew=0] [request=1]
 //
 // Builds the benchmark geometry (H 4096, E 256, top-6, I 2048, one shared expert) with pseudo-random operands (valid FP4 /
 // FP8 / UE8M0 codes: the values do not matter to a profiler, the routing is as spread as with real weights; skew > 0 adds the
-// selection bias -skew * ln(1 + expert), which concentrates the routes on the first experts), runs `passes`
+// selection bias -skew * ln(1 + expert), which concentrates the routes on the first experts; request > 1: every `request`
+// consecutive rows are one request's draft tokens, a shared base row plus noise of 0.3 times its spread, so that their routes
+// overlap as the speculative-verify workload's do), runs `passes`
 // eager passes of the layer's own schedule cycling through `batches` input batches, prints the mean durations the library's
 // marks give, and finally launches `copies` plain copies of 256 MiB (tf_probe_copy) so that a hardware-counter run holds a
 // kernel whose traffic is known: 268,435,456 bytes fetched and as many written per launch.
@@ -57,11 +59,12 @@ std::vector<uint16_t> random_bf16(size_t n, Rng& r, float amplitude) {
 }  // namespace
 
 int main(int argc, char** argv) {
-    if (argc < 2) { std::fprintf(stderr, "usage: %s <libtitanic_moe_hip.so> [rows] [passes] [batches] [copies] [skew]\n", argv[0]); return 2; }
+    if (argc < 2) { std::fprintf(stderr, "usage: %s <libtitanic_moe_hip.so> [rows] [passes] [batches] [copies] [skew] [request]\n", argv[0]); return 2; }
     const int rows = argc > 2 ? std::atoi(argv[2]) : 4, passes = argc > 3 ? std::atoi(argv[3]) : 64;
     const int batches = argc > 4 ? std::atoi(argv[4]) : 16, copies = argc > 5 ? std::atoi(argv[5]) : 4;
     const float skew = argc > 6 ? (float)std::atof(argv[6]) : 0.f;
-    if (rows < 1 || rows > 16384 || passes < 1 || batches < 1 || batches > 64 || copies < 0) { std::fprintf(stderr, "arguments out of range\n"); return 2; }
+    const int request = argc > 7 ? std::atoi(argv[7]) : 1;
+    if (rows < 1 || rows > 16384 || passes < 1 || batches < 1 || batches > 64 || copies < 0 || request < 1 || rows % request) { std::fprintf(stderr, "arguments out of range\n"); return 2; }
     const ca_geometry g = {4096, 256, 6, 2048, 2048, 0, 1.0f, 128, 128, 128, -1, 10.f};
     const size_t H = g.hidden, E = g.experts, I = g.intermediate, S = g.shared_intermediate;
     Rng rng{0x7469746eull};
@@ -86,7 +89,15 @@ int main(int argc, char** argv) {
     if (tfh_layer_set_tokens(layer, tokens.data(), rows, nullptr, error, sizeof error)) { std::fprintf(stderr, "tokens: %s\n", error); return 1; }
     std::vector<uint64_t> inputs;
     for (int b = 0; b < batches; ++b) {
-        const std::vector<uint16_t> x = random_bf16((size_t)rows * H, rng, 2.f);
+        std::vector<uint16_t> x = random_bf16((size_t)rows * H, rng, 2.f);
+        if (request > 1) {
+            auto value = [](uint16_t v) { const uint32_t b = (uint32_t)v << 16; float f; std::memcpy(&f, &b, 4); return f; };
+            for (int r = 0; r < rows; ++r) {
+                if (r % request == 0) continue;                          // a request's first row is its base
+                const uint16_t* base = &x[(size_t)(r - r % request) * H];
+                for (size_t c = 0; c < H; ++c) x[(size_t)r * H + c] = to_bf16(value(base[c]) + 0.3f * value(x[(size_t)r * H + c]));
+            }
+        }
         void* d = nullptr;
         HIP_OK(hipMalloc(&d, x.size() * 2));
         HIP_OK(hipMemcpy(d, x.data(), x.size() * 2, hipMemcpyHostToDevice));
