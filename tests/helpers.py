@@ -287,3 +287,100 @@ def error_stats(got_u16, want_u16):
         return 0.0, 0.0
     scale = np.abs(w).max() + 1e-30
     return float(np.abs(g - w).max() / scale), float(np.abs(g - w).mean())
+
+
+# ---- float64 evaluation of the layer on the same quantized operands ------------------------------------------------------
+_E2M1 = [0.0, 0.5, 1.0, 1.5, 2.0, 3.0, 4.0, 6.0, -0.0, -0.5, -1.0, -1.5, -2.0, -3.0, -4.0, -6.0]
+
+
+def _lut_e4m3(device):
+    return torch.tensor([float(oracle.lib().orc_e4m3_to_f32(i)) for i in range(256)], dtype=torch.float64, device=device)
+
+
+def dequant_mxfp4(w, s):
+    """Packed E2M1 bytes [n][k/2] (low nibble = even column) with UE8M0 scales [n][k/32] -> float64 [n][k] (exact)."""
+    lut = torch.tensor(_E2M1, dtype=torch.float64, device=w.device)
+    nib = torch.stack([w & 15, w >> 4], dim=-1).reshape(w.shape[0], -1).long()
+    scale = torch.pow(torch.tensor(2.0, dtype=torch.float64, device=w.device), s.double() - 127.0)
+    return lut[nib] * scale.repeat_interleave(32, dim=1)
+
+
+def dequant_fp8_blocks(w, s, bn, bk):
+    """E4M3 codes [n][k] with UE8M0 block scales [n/bn][k/bk] -> float64 (exact)."""
+    scale = torch.pow(torch.tensor(2.0, dtype=torch.float64, device=w.device), s.double() - 127.0)
+    return _lut_e4m3(w.device)[w.long()] * scale.repeat_interleave(bn, dim=0).repeat_interleave(bk, dim=1)
+
+
+def dequant_rows(codes, scales, block, device, zero_marks_zero_block):
+    """Activation rows: E4M3 codes [rows][k], UE8M0 scales [rows][k/block] (numpy) -> float64 tensor (exact)."""
+    q = torch.from_numpy(np.ascontiguousarray(codes)).to(device).long()
+    s = torch.from_numpy(np.ascontiguousarray(scales)).to(device)
+    scale = torch.pow(torch.tensor(2.0, dtype=torch.float64, device=device), s.double() - 127.0)
+    if zero_marks_zero_block:
+        scale = torch.where(s == 0, torch.zeros_like(scale), scale)
+    return _lut_e4m3(device)[q] * scale.repeat_interleave(block, dim=1)
+
+
+def _to_bf16_bits(t64):
+    return t64.to(torch.float32).to(torch.bfloat16).view(torch.int16).cpu().numpy().view(np.uint16)
+
+
+def exact_layer(g, ops, x, ids, weights, live=None, h_given=None):
+    """The layer with every dot product in float64 on the same quantized operands (dequantized exactly) and every
+    requantization point of the layer kept (token codes, BF16 intermediate and its codes, BF16 route outputs, BF16 shared
+    projections, the shared activation and its codes, the ordered FP32 route sum, the BF16 addition).  What a GPU or oracle
+    result differs from it by is its own accumulation error, and what that error does to the FP8 codes downstream.  Runs on
+    the operands' device (float64 matrix products of torch, an implementation of its own).  `h_given`: BF16 bits
+    [rows][K][I] to continue from instead of the float64 FC1 + SwiGLU (what follows a given activation exactly)."""
+    rows = x.shape[0]
+    K, I, H, B = g.topk, g.intermediate, g.hidden, g.act_block
+    dev = ops.w13.device
+    xb = u16(x)
+    t = {}
+    xq, xs = oracle.quantize_rows(xb, B, 0.0)
+    xq_min, xs_min = oracle.quantize_rows(xb, B, 1e-4)
+    xr = dequant_rows(xq, xs, B, dev, True)
+    h = np.zeros((rows * K, I), np.uint16)
+    flat_ids = np.asarray(ids).reshape(-1)
+    active = sorted(set(int(e) for e in flat_ids if 0 <= e < g.experts))
+    limit = float(g.swiglu_limit)
+    for e in active if h_given is None else []:
+        routes = np.nonzero(flat_ids == e)[0]
+        w = dequant_mxfp4(ops.w13[e], ops.s13[e])
+        proj = xr[torch.as_tensor(routes // K, device=dev)] @ w.T
+        up, gate = proj[:, :I], proj[:, I:]
+        gv = torch.clamp(gate, max=limit)
+        uv = torch.clamp(up, min=-limit, max=limit)
+        h[routes] = _to_bf16_bits(gv * torch.sigmoid(gv) * uv)
+    if h_given is not None:
+        h = np.ascontiguousarray(h_given).reshape(rows * K, I).copy()
+        h[~((flat_ids >= 0) & (flat_ids < g.experts))] = 0
+    hq, hs = oracle.quantize_rows(h, B, 0.0)
+    hd = dequant_rows(hq, hs, B, dev, True)
+    route_out = np.zeros((rows * K, H), np.uint16)
+    wts = torch.from_numpy(np.ascontiguousarray(np.asarray(weights, np.float32).reshape(-1))).to(dev).double()
+    for e in active:
+        routes = np.nonzero(flat_ids == e)[0]
+        at = torch.as_tensor(routes, device=dev)
+        w = dequant_mxfp4(ops.w2[e], ops.s2[e])
+        route_out[routes] = _to_bf16_bits((hd[at] @ w.T) * wts[at][:, None])
+    t["h"], t["hq"], t["hs"] = h.reshape(rows, K, I), hq.reshape(rows, K, I), hs.reshape(rows, K, -1)
+    t["route_out"] = route_out.reshape(rows, K, H)
+    xm = dequant_rows(xq_min, xs_min, B, dev, False)
+    t["shared_up"] = _to_bf16_bits(xm @ dequant_fp8_blocks(ops.sh_w13, ops.sh_s13, g.shared_bn, g.shared_bk).T)
+    t["shared_act"], aq, asc = oracle.shared_swiglu_quant(t["shared_up"], B, g.swiglu_limit)
+    t["shared_down"] = _to_bf16_bits(dequant_rows(aq, asc, B, dev, False) @ dequant_fp8_blocks(ops.sh_w2, ops.sh_s2, g.shared_bn, g.shared_bk).T)
+    n_live = rows if live is None else min(live, rows)
+    t["routed"], t["out"] = oracle.ffn_sum_shared(t["route_out"], t["shared_down"], n_live)
+    return t
+
+
+def accuracy_table(name, gpu_out, oracle_out, exact_out, factor=1.5):
+    """Both readings of the output error of the GPU and of the oracle against the float64 evaluation; asserts that the GPU is
+    as close to exact arithmetic as the oracle is (within `factor`, and an allowance of one part in 10^4 of the largest
+    magnitude for outputs where both are that close)."""
+    a, b = error_report(gpu_out, exact_out), error_report(oracle_out, exact_out)
+    print("  %s vs float64: GPU max rel %.3e, mean abs %.3e, per element max %.3e, above 1e-2 %.3e | oracle max rel %.3e, mean abs %.3e, "
+          "per element max %.3e, above 1e-2 %.3e" % (name, a["max_rel"], a["mean_abs"], a["max_elem_rel"], a["frac_above"], b["max_rel"], b["mean_abs"],
+                                                   b["max_elem_rel"], b["frac_above"]))
+    return a, b

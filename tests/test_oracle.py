@@ -487,3 +487,29 @@ def test_vectorised_projection_loops_against_the_scalar_oracle(mode):
     a = oracle.fp8_linear(aq, ones, 32, wq, ws, 32, 32)
     b = oracle.fp8_linear(aq, ones, 32, wq, ws, 32, 32, simd=True)
     assert np.array_equal(a, b)
+
+
+@pytest.mark.parametrize("mode", ["benchmark", "reference"])
+def test_layer_against_float64_on_the_same_quantized_operands(mode):
+    # the whole layer with every dot product in float64 (torch's matrix products on exactly dequantized operands) and every
+    # requantization point kept: the oracle's FP32 chains agree with it to the BF16 boundaries
+    import helpers
+    g = helpers.geometry(1024, 16, 2, 512, 512, mode)
+    ops = helpers.synth.LayerOperands(g, "c1", device="cpu")
+    x = helpers.synth.activations("c1", 8, g.hidden)
+    want = helpers.oracle_layer(g, ops, x)
+    exact = helpers.exact_layer(g, ops, x, want["ids"], want["weights"])
+    for name in ["h", "route_out", "shared_up", "shared_down", "out"]:
+        assert helpers.bf16_ulp_distance(want[name], exact[name], accumulation=0.0) <= 1.0, name
+        assert np.mean(want[name] != exact[name]) <= 1e-3, name
+    assert np.array_equal(want["hq"], exact["hq"]) or np.mean(want["hq"] != exact["hq"]) <= 1e-4
+    # a transposed operand, a dropped scale or the wrong half of the up / gate rows would move every value: the float64
+    # evaluation with up and gate swapped is far from the oracle
+    swapped = type("Ops", (), {})()
+    for k, v in vars(ops).items():
+        setattr(swapped, k, v)
+    I = g.intermediate
+    swapped.w13 = torch.cat([ops.w13[:, I:], ops.w13[:, :I]], dim=1)
+    swapped.s13 = torch.cat([ops.s13[:, I:], ops.s13[:, :I]], dim=1)
+    other = helpers.exact_layer(g, swapped, x, want["ids"], want["weights"])
+    assert np.mean(other["h"] != want["h"]) > 0.9
