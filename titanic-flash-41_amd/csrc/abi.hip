@@ -418,6 +418,7 @@ int launch_dense(const Context& c, const uint64_t* p, const int32_t* sc, hipStre
     a.a_codes = (const uint8_t*)p[0]; a.a_scales = (const uint8_t*)p[1];
     a.w = (const uint8_t*)p[2]; a.ws = (const uint8_t*)p[3]; a.bn = c.g.shared_bn; a.bk = c.g.shared_bk;
     a.dense_rows = m; a.k = k; a.hidden = n; a.act_block = c.g.act_block; a.out = (uint16_t*)p[4];
+    if (tf_grouped_dense_shape_ok(a, false)) return tf_launch_grouped_dense<TF_GEMM_DENSE>(a, c.cus, s);
     return tf_launch_dense_gemm(a, c.cus, s);
 }
 // ---- entry 5: ffn.shared_expert (up + clipped SwiGLU + requant + down, from the quantized input) ---------------------
@@ -439,12 +440,13 @@ int launch_shared(const Context& c, const uint64_t* p, const int32_t* sc, hipStr
     a.dense_rows = m; a.k = g.hidden; a.inter = g.shared_intermediate; a.hidden = g.hidden; a.act_block = g.act_block;
     a.limit = g.swiglu_limit; a.h_bf16 = (uint16_t*)p[H_ACT]; a.h_codes = (uint8_t*)p[H_ACT_CODES]; a.h_scales = (uint8_t*)p[H_ACT_SCALES];
     a.tap = (uint16_t*)p[H_UP_TAP];
-    int status = tf_launch_shared_fc1_gemm(a, c.cus, s);
+    int status = tf_grouped_dense_shape_ok(a, true) ? tf_launch_grouped_dense<TF_GEMM_FC1_SHARED>(a, c.cus, s) : tf_launch_shared_fc1_gemm(a, c.cus, s);
     if (status) return status;
     GemmArgs b{};
     b.a_codes = (const uint8_t*)p[H_ACT_CODES]; b.a_scales = (const uint8_t*)p[H_ACT_SCALES];
     b.w = (const uint8_t*)p[H_W2]; b.ws = (const uint8_t*)p[H_S2]; b.bn = g.shared_bn; b.bk = g.shared_bk;
     b.dense_rows = m; b.k = g.shared_intermediate; b.hidden = g.hidden; b.act_block = g.act_block; b.out = (uint16_t*)p[H_OUT];
+    if (tf_grouped_dense_shape_ok(b, false)) return tf_launch_grouped_dense<TF_GEMM_DENSE>(b, c.cus, s);
     return tf_launch_dense_gemm(b, c.cus, s);
 }
 

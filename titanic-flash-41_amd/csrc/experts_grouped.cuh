@@ -67,6 +67,12 @@ __device__ __forceinline__ void tf_mfma_weights_first(v4f& acc, const u4v& weigh
     asm volatile("v_mfma_scale_f32_16x16x128_f8f6f4 %0, %1, %2, %0, %3, %4 op_sel:[%5,%6,0] op_sel_hi:[%7,%8,0] cbsz:4"
                  : "+v"(acc) : "v"(weights), "v"(tokens), "v"(scale_w), "v"(scale_t), "n"(SW & 1), "n"(ST & 1), "n"(SW >> 1), "n"(ST >> 1));
 }
+// The same product with FP8 (E4M3) weights: eight registers a lane for the first operand too, no format modifier.
+template <int SW, int ST>
+__device__ __forceinline__ void tf_mfma_fp8_weights_first(v4f& acc, const v8i& weights, const v8i& tokens, uint32_t scale_w, uint32_t scale_t) {
+    asm volatile("v_mfma_scale_f32_16x16x128_f8f6f4 %0, %1, %2, %0, %3, %4 op_sel:[%5,%6,0] op_sel_hi:[%7,%8,0]"
+                 : "+v"(acc) : "v"(weights), "v"(tokens), "v"(scale_w), "v"(scale_t), "n"(SW & 1), "n"(ST & 1), "n"(SW >> 1), "n"(ST >> 1));
+}
 // The matrix pipeline's last results have reached the registers (the longest product takes 8 passes of 4 cycles; 32 idle
 // cycles follow the last product before any of these eight accumulators is read).
 __device__ __forceinline__ void tf_mfma_settle(v4f (&acc)[8]) {
@@ -98,22 +104,30 @@ constexpr int tf_loads_behind(int u) {
 
 template <int MODE, int BM, bool WORDS>
 __global__ void __launch_bounds__(512) tf_grouped_gemm(const GemmArgs p) {
-    constexpr bool FC1 = MODE == TF_GEMM_FC1_ROUTED;
-    constexpr int NG = BM == 256 ? 1 : 2;    // column groups a task: a 128-row unit takes two, so that a wave's products a k-step
-                                             // (and with them the k-step's fixed costs a product) are those of a 256-row unit
+    constexpr bool FC1 = MODE == TF_GEMM_FC1_ROUTED || MODE == TF_GEMM_FC1_SHARED;
+    // The FP8 shared expert and the dense product: rows in place (no plan, no permutation map: tile t holds rows 128 t ..),
+    // one weight matrix, E4M3 weights (2 KiB a 16-row weight tile and k-step: two requests) with row-major block scales.
+    constexpr bool FP8B = MODE == TF_GEMM_FC1_SHARED || MODE == TF_GEMM_DENSE;
+    static_assert(!FP8B || BM == 128, "FP8 weights: a ring stage holds a 128-row unit and one column group");
+    constexpr int BREQ = FP8B ? 2 : 1;       // 1 KiB requests a weight tile and k-step
+    constexpr int NG = FP8B || BM == 256 ? 1 : 2;    // column groups a task: a 128-row unit of FP4 weights takes two, so that a wave's products a
+                                             // k-step (and with them the k-step's fixed costs a product) are those of a 256-row unit
     constexpr int NS = 3, LEAD = NS - 1;
     constexpr int NA = BM / 64;              // 16-byte pieces of the token tile a thread requests a k-step
     constexpr int NF = BM / 64;              // 16-row fragments of a wave (BM / 4 rows)
     constexpr int NT = 8 * NG;               // weight tiles a wave multiplies its fragments with
     constexpr int NB = 2 * NG;               // weight tiles a wave requests a k-step
     constexpr int WROWS = BM / 4;
-    constexpr int DATA = NA + 1 + NB;        // requests a wave issues a k-step: token pieces, token scales, weight tiles
-    constexpr int A_STAGE = BM * 128, B_STAGE = 16 * 1024 * NG;
+    constexpr int DATA = NA + 1 + NB * BREQ; // requests a wave issues a k-step: token pieces, token scales, weight tiles
+    constexpr int MORE = FP8B ? 0 : NB;      // and once a round of four k-steps: the next round's prepared weight scale words
+    constexpr int A_STAGE = BM * 128, B_STAGE = 16 * 1024 * NG * BREQ;
     constexpr int ROW_WAVES = BM / 64;       // waves whose 64 lanes cover the tile's rows once; the other waves repeat them
     __shared__ __attribute__((aligned(1024))) uint8_t s_a[NS * A_STAGE];
     __shared__ __attribute__((aligned(1024))) uint8_t s_b[NS * B_STAGE];
     __shared__ __attribute__((aligned(256))) uint32_t s_asc[NS][BM];
-    __shared__ __attribute__((aligned(256))) uint32_t s_bsc[16 * NG * 64];
+    __shared__ __attribute__((aligned(256))) uint32_t s_bsc[FP8B ? 64 : 16 * NG * 64];
+    // FP8 weights: the block scales of the task's 256 weight rows, as they lie in memory ([row block][k / bk] bytes), for three tasks in turn
+    __shared__ __attribute__((aligned(256))) uint32_t s_wsc[FP8B ? 3 : 1][FP8B ? 512 : 64];
     __shared__ __attribute__((aligned(256))) int32_t s_src[3][BM];   // the permutation map's entry (route index) of each tile row, for three tasks in turn
     __shared__ __attribute__((aligned(256))) float s_wgt[NG == 2 ? 4 : 3][BM];   // FC2: routing weight of each tile row (three tasks in turn); FC1: row maxima of the column halves
     __shared__ uint16_t s_ubase[BM == 256 ? 514 : 2], s_nbase[BM == 256 ? 514 : 2];      // units / short last units before expert e
@@ -125,7 +139,7 @@ __global__ void __launch_bounds__(512) tf_grouped_gemm(const GemmArgs p) {
     const int wm = wave >> 1, wn = wave & 1, g = lane >> 4, r16 = lane & 15;
     const int KS = p.k / 128, scales_row = p.k / p.act_block;
     const int groups = (FC1 ? p.inter / 128 : p.hidden / 256) / NG;          // a task's column groups: ng NG .. ng NG + NG - 1
-    const int total_tiles = p.expert_tile_base[p.experts];
+    const int total_tiles = FP8B ? (p.dense_rows + 127) / 128 : p.expert_tile_base[p.experts];
     int units = total_tiles;
     const int xcd = blockIdx.x & 7, local = blockIdx.x >> 3, local_count = gridDim.x >> 3;
     int u_lo, u_hi, n_lo = 0, n_hi = 0;      // the XCD's units; BM == 256: short last units before them
@@ -231,6 +245,20 @@ __global__ void __launch_bounds__(512) tf_grouped_gemm(const GemmArgs p) {
             const int tb = scalar_load(p.expert_tile_base + r.expert), tn = scalar_load(p.expert_tile_base + r.expert + 1);
             r.first_tile = tb + 2 * k2;
             r.rows = min(BM, (tn - tb - 1) * 128 + scalar_load(p.task_valid_rows + (size_t)(tn - 1) * p.groups) - 256 * k2);
+        } else if constexpr (FP8B) {
+            const int un = q / groups, unit = u_lo + un;
+            r.ng = q - un * groups;
+            r.first_tile = unit;
+            r.expert = 0;
+            r.rows = min(BM, p.dense_rows - unit * BM);
+            // the block scales of the task's weight rows: word i of the slot = word i % wpr of row block i / wpr of the task
+            // (FC1: the column group's 128 "gate" rows, then its 128 "up" rows; otherwise 256 consecutive rows)
+            const int per_block = p.k / p.bk, wpr = per_block >> 2, half_blocks = 128 / p.bn;
+            const int i = min(wave * 64 + lane, 2 * half_blocks * wpr - 1), rb = i / wpr, j = i - rb * wpr;
+            const int block = FC1 ? (rb < half_blocks ? (r.ng * 128) / p.bn + rb : (p.inter + r.ng * 128) / p.bn + rb - half_blocks)
+                                  : (r.ng * 256) / p.bn + rb;
+            tf_dma4(p.ws, (uint32_t)(block * per_block + j * 4), tf_lds_addr(&s_wsc[slot][0]) + wave * 256);
+            return r;
         } else {
             const int un = q / groups, unit = u_lo + un;
             r.ng = q - un * groups;
@@ -257,7 +285,7 @@ __global__ void __launch_bounds__(512) tf_grouped_gemm(const GemmArgs p) {
     auto install = [&](Source& src, const TaskRef& task, int slot) {
         const int ng = task.ng, first_tile = task.first_tile, expert = task.expert, rows = task.rows;
         auto source_row = [&](int row) -> uint32_t {         // rows past the valid ones request the first row's bytes again
-            if constexpr (FC1) return (uint32_t)(s_src[slot][row < rows ? row : 0] / p.topk);
+            if constexpr (FC1 && !FP8B) return (uint32_t)(s_src[slot][row < rows ? row : 0] / p.topk);
             else return (uint32_t)(first_tile * 128 + (row < rows ? row : 0));
         };
 #pragma unroll
@@ -273,8 +301,8 @@ __global__ void __launch_bounds__(512) tf_grouped_gemm(const GemmArgs p) {
         for (int c = 0; c < NB; ++c) {
             const int T = (wave * NB + c) & 15, cg = ng * NG + (wave * NB + c) / 16;       // tile within its column group, the group
             const int ntile = FC1 ? (T < 8 ? cg * 8 + T : p.inter / 16 + cg * 8 + T - 8) : cg * 16 + T;
-            src.b_base[c] = w + (size_t)ntile * KS * 1024;
-            src.bsc_base[c] = ws + (size_t)ntile * (p.k / 512) * 256;
+            src.b_base[c] = w + (size_t)ntile * KS * (1024 * BREQ);
+            src.bsc_base[c] = ws + (size_t)ntile * (p.k / 512) * 256;       // (FP4 weights: prepared scale words)
         }
     };
     const uint32_t lane16 = lane * 16, lane4 = lane * 4;
@@ -283,7 +311,11 @@ __global__ void __launch_bounds__(512) tf_grouped_gemm(const GemmArgs p) {
     auto issue_op = [&](const Source& src, int op, int ks, int stage) {
         if (op < NA) tf_dma16(p.a_codes + (size_t)ks * 128, src.a_off[op], lds_a + stage * A_STAGE + (wave * NA + op) * 1024);
         else if (op == NA) tf_dma4(p.a_scales + (WORDS ? (ks >> 2) * 4 : ks * 4), src.asc_off, lds_asc + stage * (BM * 4) + (wave & (ROW_WAVES - 1)) * 256);
-        else if (op < DATA) tf_dma16(src.b_base[op - NA - 1] + (size_t)ks * 1024, lane16, lds_b + stage * B_STAGE + (wave * NB + op - NA - 1) * 1024);
+        else if (op < DATA) {
+            // FP8 weights: request 2 c + half is the 1 KiB plane `half` of the wave's tile c (consecutive in memory and in the stage)
+            const int c = (op - NA - 1) / BREQ, piece = op - NA - 1;
+            tf_dma16(src.b_base[c] + (size_t)ks * (1024 * BREQ) + (piece - c * BREQ) * 1024, lane16, lds_b + stage * B_STAGE + (wave * NB * BREQ + piece) * 1024);
+        }
         else tf_dma4(src.bsc_base[op - DATA] + (size_t)(ks >> 2) * 256, lane4, lds_bsc + (wave * NB + op - DATA) * 256);
     };
 
@@ -306,8 +338,10 @@ __global__ void __launch_bounds__(512) tf_grouped_gemm(const GemmArgs p) {
     tf_wait_vm<0>();
     tf_lds_barrier();
     install(now, cur, 0);
+    if constexpr (!FP8B) {
 #pragma unroll
-    for (int c = 0; c < NB; ++c) issue_op(now, DATA + c, 0, 0);
+        for (int c = 0; c < NB; ++c) issue_op(now, DATA + c, 0, 0);
+    }
 #pragma unroll
     for (int d = 0; d < LEAD; ++d)
 #pragma unroll
@@ -330,6 +364,17 @@ __global__ void __launch_bounds__(512) tf_grouped_gemm(const GemmArgs p) {
         const int nf = max(0, min(rows <= BM / 2 ? NF / 2 : NF, (rows - wbase + 15) >> 4));     // fragments of this wave with valid rows
         const int a_lo = (wbase + r16) * 128 + ((g ^ swz) << 4), a_hi = a_lo ^ 64;     // + 2,048 a fragment
         TaskRef after = nxt;
+        // FP8 weights: where the block scales of the wave's weight tile t start in the task's table (tile T of the stage: rows
+        // 16 T .. of the task's first 128 weight rows, or 16 (T - 8) .. of its second)
+        int wsc_row[8];
+        const int bk_shift = p.bk == 32 ? 5 : p.bk == 64 ? 6 : 7;
+        if constexpr (FP8B) {
+#pragma unroll
+            for (int t = 0; t < 8; ++t) {
+                const int T = b_first + b_step(t);
+                wsc_row[t] = ((FC1 && T >= 8 ? 128 / p.bn + ((T - 8) * 16) / p.bn : (T * 16) / p.bn)) * (p.k / p.bk);
+            }
+        }
 
         // One task, compiled for 0, NF / 2 or NF fragments of the wave so that no product sits under a branch and the
         // accumulators are as many as the wave needs; every wave issues the same requests and passes the same barriers
@@ -357,7 +402,7 @@ __global__ void __launch_bounds__(512) tf_grouped_gemm(const GemmArgs p) {
                 // requests its share of k-step b + LEAD into it: the early waves in k-step b, the late waves in the second half
                 // of their k-step b - 1.  A task's first k-steps landed before the previous task's stores went out (below).
                 if (!late) {
-                    if constexpr (!FIRST || u >= LEAD) tf_wait_vm<tf_loads_behind<LEAD, DATA, 1, NB>(u)>();
+                    if constexpr (!FIRST || u >= LEAD) tf_wait_vm<tf_loads_behind<LEAD, DATA, 1, MORE>(u)>();
                     __builtin_amdgcn_s_barrier();
                 }
                 asm volatile("" ::: "memory");
@@ -373,7 +418,7 @@ __global__ void __launch_bounds__(512) tf_grouped_gemm(const GemmArgs p) {
                     const int ks_ahead = OVER ? u + AHEAD - 4 : ks + AHEAD;
                     const Source& from = OVER ? then : now;
                     const int stage = AHEAD == LEAD ? ps : (ps + 1 == NS ? 0 : ps + 1);
-                    if constexpr (EXTRA) {
+                    if constexpr (EXTRA && !FP8B) {
 #pragma unroll
                         for (int i = 0; i < NB; ++i) issue_op(LAST ? then : now, DATA + i, LAST ? 0 : ks + 4 - u, 0);
                     }
@@ -389,7 +434,7 @@ __global__ void __launch_bounds__(512) tf_grouped_gemm(const GemmArgs p) {
                         // the late waves' share of the next k-step's stage (the next task's first, after a task's last k-step);
                         // what they requested for the task's first LEAD + 1 k-steps landed before their last stores
                         constexpr bool WAIT = u == 3 || !(FIRST && u + 1 <= LEAD);
-                        if constexpr (WAIT) tf_wait_vm<tf_loads_behind<LEAD, DATA, 0, NB>(u)>();
+                        if constexpr (WAIT) tf_wait_vm<tf_loads_behind<LEAD, DATA, 0, MORE>(u)>();
                         asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory");      // this k-step's last reads of its stage have returned
                         __builtin_amdgcn_s_barrier();
                         asm volatile("" ::: "memory");
@@ -445,12 +490,20 @@ __global__ void __launch_bounds__(512) tf_grouped_gemm(const GemmArgs p) {
                 }
                 if constexpr (FR > 0 && NG == 1) {
                     const uint8_t* sa = s_a + cs * A_STAGE;
-                    const uint8_t* sb = s_b + cs * B_STAGE + b_first * 1024 + lane16;
+                    const uint8_t* sb = s_b + cs * B_STAGE + b_first * (1024 * BREQ) + lane16;
                     const uint32_t* sc = &s_asc[cs][wbase + r16];
-                    u4v bf[8];
+                    u4v bf[8], bf_hi[FP8B ? 8 : 1];
 #pragma unroll
-                    for (int t = 0; t < 8; ++t) bf[t] = *reinterpret_cast<const u4v*>(sb + b_step(t) * 1024);
-                    if constexpr (u == 0) {
+                    for (int t = 0; t < 8; ++t) {
+                        bf[t] = *reinterpret_cast<const u4v*>(sb + b_step(t) * (1024 * BREQ));
+                        if constexpr (FP8B) bf_hi[t] = *reinterpret_cast<const u4v*>(sb + b_step(t) * 2048 + 1024);
+                    }
+                    if constexpr (FP8B) {
+                        // the weights' block scale of this k-step and lane group: byte (128 ks + 32 g) / bk of the tile's row block
+                        const uint8_t* table = reinterpret_cast<const uint8_t*>(&s_wsc[slot][0]) + ((ks * 128 + 32 * g) >> bk_shift);
+#pragma unroll
+                        for (int t = 0; t < 8; ++t) bsc[t] = table[wsc_row[t]];
+                    } else if constexpr (u == 0) {
 #pragma unroll
                         for (int t = 0; t < 8; ++t) bsc[t] = s_bsc[b_first * 64 + lane + b_step(t) * 64];
                     }
@@ -472,8 +525,16 @@ __global__ void __launch_bounds__(512) tf_grouped_gemm(const GemmArgs p) {
                         const uint32_t sca = WORDS ? word[f & 1] : word[f & 1] >> (8 * g);
                         constexpr int SEL = WORDS ? u : 0;
                         const v8i av = v8i{(int)l[0], (int)l[1], (int)l[2], (int)l[3], (int)h[0], (int)h[1], (int)h[2], (int)h[3]};
+                        if constexpr (FP8B) {
 #pragma unroll
-                        for (int t = 0; t < 8; ++t) tf_mfma_weights_first<u, SEL>(acc[f][t], bf[t], av, bsc[t], sca);
+                            for (int t = 0; t < 8; ++t) {
+                                const v8i bv = v8i{(int)bf[t][0], (int)bf[t][1], (int)bf[t][2], (int)bf[t][3], (int)bf_hi[t][0], (int)bf_hi[t][1], (int)bf_hi[t][2], (int)bf_hi[t][3]};
+                                tf_mfma_fp8_weights_first<0, SEL>(acc[f][t], bv, av, bsc[t], sca);
+                            }
+                        } else {
+#pragma unroll
+                            for (int t = 0; t < 8; ++t) tf_mfma_weights_first<u, SEL>(acc[f][t], bf[t], av, bsc[t], sca);
+                        }
                         // the early waves' requests of the k-step behind their first fragment's products, so that their address
                         // arithmetic runs under the matrix pipeline (the late waves': behind their barrier, above)
                         if (f == 0) { if (!late) issue_range(early_ahead, early_extra); }
@@ -528,15 +589,33 @@ __global__ void __launch_bounds__(512) tf_grouped_gemm(const GemmArgs p) {
                     float amax[FRA][2];
                     uint32_t codes[FRA][4], exponent[FRA][2];
                     float (*s_max)[BM] = s_wgt + 2 * gi;          // [wn][row]: FC1 keeps no routing weights here
+                    // the shared expert: "gate" tiles first, then "up"; both projections are rounded to BF16 (and kept, where the caller
+                    // asks for them), clamped in BF16, and the activation is the exact-sequence one (its bits are the oracle's)
+                    u2v tap_gate[FP8B ? FRA : 1][4], tap_up[FP8B ? FRA : 1][4];
+                    const float hi_lim = tf_bf16(tf_to_bf16(p.limit)), lo_lim = tf_bf16(tf_to_bf16(-p.limit));
 #pragma unroll
                     for (int f = 0; f < FR; ++f) {
 #pragma unroll
-                        for (int j = 0; j < 4; ++j)
+                        for (int j = 0; j < 4; ++j) {
+                            if constexpr (FP8B) {
+                                const v4f gq = acc[f][j], uq = acc[f][4 + j];
+                                tap_gate[f][j] = u2v{tf_pack_bf16(gq[0], gq[1]), tf_pack_bf16(gq[2], gq[3])};
+                                tap_up[f][j] = u2v{tf_pack_bf16(uq[0], uq[1]), tf_pack_bf16(uq[2], uq[3])};
 #pragma unroll
-                            for (int i = 0; i < 4; ++i) {
-                                const float gv = fminf(acc[f][gi * 8 + 4 + j][i], p.limit), uv = fminf(p.limit, fmaxf(-p.limit, acc[f][gi * 8 + j][i]));
-                                hv[f][j][i] = tf_bf16(tf_to_bf16(__fmul_rn(__fmul_rn(gv, tf_logistic_fast(gv)), uv)));
+                                for (int i = 0; i < 4; ++i) {
+                                    const uint32_t gw = tap_gate[f][j][i >> 1], uw = tap_up[f][j][i >> 1];
+                                    const float gv = fminf((i & 1) ? tf_bf16_hi(gw) : tf_bf16_lo(gw), hi_lim);
+                                    const float uv = fminf(fmaxf((i & 1) ? tf_bf16_hi(uw) : tf_bf16_lo(uw), lo_lim), hi_lim);
+                                    hv[f][j][i] = tf_bf16(tf_to_bf16(__fmul_rn(gv / __fadd_rn(1.0f, tf_exp(-gv)), uv)));
+                                }
+                            } else {
+#pragma unroll
+                                for (int i = 0; i < 4; ++i) {
+                                    const float gv = fminf(acc[f][gi * 8 + 4 + j][i], p.limit), uv = fminf(p.limit, fmaxf(-p.limit, acc[f][gi * 8 + j][i]));
+                                    hv[f][j][i] = tf_bf16(tf_to_bf16(__fmul_rn(__fmul_rn(gv, tf_logistic_fast(gv)), uv)));
+                                }
                             }
+                        }
 #pragma unroll
                         for (int b = 0; b < 2; ++b) {
                             float m = 0.f;
@@ -562,7 +641,7 @@ __global__ void __launch_bounds__(512) tf_grouped_gemm(const GemmArgs p) {
                     for (int f = 0; f < FR; ++f)
 #pragma unroll
                         for (int b = 0; b < 2; ++b) {
-                            exponent[f][b] = tf_block_exponent(amax[f][b]);
+                            exponent[f][b] = tf_block_exponent(FP8B ? fmaxf(amax[f][b], 1e-4f) : amax[f][b]);     // the shared expert's quantizer floors amax
                             const float inv = tf_block_inverse(exponent[f][b]);
 #pragma unroll
                             for (int j = 2 * b; j < 2 * b + 2; ++j)
@@ -580,6 +659,12 @@ __global__ void __launch_bounds__(512) tf_grouped_gemm(const GemmArgs p) {
                                 *reinterpret_cast<uint32_t*>(p.h_codes + phys * p.inter + col) = codes[f][j];
                                 if (p.h_bf16 != nullptr)
                                     *reinterpret_cast<u2v*>(p.h_bf16 + phys * p.inter + col) = u2v{tf_pack_bf16(hv[f][j][0], hv[f][j][1]), tf_pack_bf16(hv[f][j][2], hv[f][j][3])};
+                                if constexpr (FP8B) {
+                                    if (p.tap != nullptr) {
+                                        *reinterpret_cast<u2v*>(p.tap + phys * 2 * p.inter + col) = tap_gate[f][j];
+                                        *reinterpret_cast<u2v*>(p.tap + phys * 2 * p.inter + p.inter + col) = tap_up[f][j];
+                                    }
+                                }
                             }
                             if (g == 0) {
                                 if constexpr (WORDS) { if (wn == 0) p.h_scales[phys * (p.inter / 128) + cg] = (uint8_t)exponent[f][0]; }
@@ -597,12 +682,19 @@ __global__ void __launch_bounds__(512) tf_grouped_gemm(const GemmArgs p) {
 #pragma unroll
                     for (int f = 0; f < FR; ++f) {
                         const int row = min(wbase + 16 * f + r16, BM - 1);
-                        const float share = s_wgt[slot][row];
-                        out_at[f] = (size_t)s_src[slot][row] * p.hidden + cg * 256 + wn * 128 + 4 * g;
+                        if constexpr (FP8B) {          // dense product: rows in place, no routing weight
+                            out_at[f] = ((size_t)first_tile * 128 + row) * p.hidden + cg * 256 + wn * 128 + 4 * g;
 #pragma unroll
-                        for (int t = 0; t < 8; ++t)
-                            packed[f][t] = u2v{tf_pack_bf16(__fmul_rn(acc[f][gi * 8 + t][0], share), __fmul_rn(acc[f][gi * 8 + t][1], share)),
-                                               tf_pack_bf16(__fmul_rn(acc[f][gi * 8 + t][2], share), __fmul_rn(acc[f][gi * 8 + t][3], share))};
+                            for (int t = 0; t < 8; ++t)
+                                packed[f][t] = u2v{tf_pack_bf16(acc[f][t][0], acc[f][t][1]), tf_pack_bf16(acc[f][t][2], acc[f][t][3])};
+                        } else {
+                            const float share = s_wgt[slot][row];
+                            out_at[f] = (size_t)s_src[slot][row] * p.hidden + cg * 256 + wn * 128 + 4 * g;
+#pragma unroll
+                            for (int t = 0; t < 8; ++t)
+                                packed[f][t] = u2v{tf_pack_bf16(__fmul_rn(acc[f][gi * 8 + t][0], share), __fmul_rn(acc[f][gi * 8 + t][1], share)),
+                                                   tf_pack_bf16(__fmul_rn(acc[f][gi * 8 + t][2], share), __fmul_rn(acc[f][gi * 8 + t][3], share))};
+                        }
                     }
                     if (gi == 0) tf_wait_vm<0>();
 #pragma unroll
@@ -632,6 +724,23 @@ __global__ void __launch_bounds__(512) tf_grouped_gemm(const GemmArgs p) {
 inline bool tf_grouped_shape_ok(const GemmArgs& a, bool fc1) {
     return a.k >= 512 && a.k % 512 == 0 && (a.act_block == 32 || a.act_block == 128) && a.experts <= 512 &&
            (fc1 ? (a.inter >= 256 && a.inter % 256 == 0) : (a.hidden >= 512 && a.hidden % 512 == 0));
+}
+// The FP8 shared expert's first projection (MODE TF_GEMM_FC1_SHARED) and the dense product (TF_GEMM_DENSE) on the same ring:
+// whole column groups, contraction lengths that are multiples of 512, weight scale blocks of 32, 64 or 128 rows and columns.
+inline bool tf_grouped_dense_shape_ok(const GemmArgs& a, bool fc1) {
+    return a.k >= 512 && a.k % 512 == 0 && (a.act_block == 32 || a.act_block == 128) && (a.bn == 32 || a.bn == 64 || a.bn == 128) &&
+           (a.bk == 32 || a.bk == 64 || a.bk == 128) && a.k <= 8192 && a.dense_rows >= 1 &&
+           (unsigned long long)((a.dense_rows + 127) / 128) * 128ull * (unsigned long long)a.k <= 0xffffffffull &&
+           (fc1 ? (a.inter >= 128 && a.inter % 128 == 0) : (a.hidden >= 256 && a.hidden % 256 == 0));
+}
+template <int MODE>
+inline int tf_launch_grouped_dense(const GemmArgs& a, int cus, hipStream_t s) {
+    static_assert(MODE == TF_GEMM_FC1_SHARED || MODE == TF_GEMM_DENSE, "dense rows");
+    if (!tf_grouped_dense_shape_ok(a, MODE == TF_GEMM_FC1_SHARED)) return -4;
+    const int grid = tf_gemm_grid(cus);
+    if (a.act_block == 128) tf_grouped_gemm<MODE, 128, true><<<grid, 512, 0, s>>>(a);
+    else tf_grouped_gemm<MODE, 128, false><<<grid, 512, 0, s>>>(a);
+    return (int)hipGetLastError();
 }
 // `routes`: rows x top-k of the launch; experts with about two plan tiles or more on average run 256-row units.
 template <int MODE>
