@@ -46,7 +46,7 @@ SHADER_PASSES = {
 }
 # which kernel is which part of the layer: few rows / many rows
 ROLES = [("fc1", "tf_phase1_stream"), ("fc2", "tf_phase2_stream"), ("fc1", "tf_grouped_gemm<0"), ("fc2", "tf_grouped_gemm<2"),
-         ("fc1", "tf_gemm<false, 0"), ("fc2", "tf_gemm<false, 2"), ("copy", "tf_probe_copy")]
+         ("shared_fc1", "tf_grouped_gemm<1"), ("shared_fc2", "tf_grouped_gemm<3"), ("copy", "tf_probe_copy")]
 
 
 def role_of(kernel):
