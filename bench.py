@@ -102,7 +102,7 @@ def cpu_baseline(pkg, g, ops, xs, taps_ids, budget_s=12.0, scalar_budget_s=8.0, 
     def timed(n_threads, budget, simd):
         oracle.set_threads(n_threads)
         done, spent = 0, 0.0
-        while done < 4 * len(xs) and (done == 0 or spent + spent / done < budget):
+        while done < 4096 and (done == 0 or spent + spent / done < budget):
             t0 = time.perf_counter()
             helpers.oracle_layer(g, subsets[done % len(xs)], host_xs[done % len(xs)], simd=simd)
             spent += time.perf_counter() - t0
