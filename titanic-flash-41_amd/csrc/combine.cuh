@@ -21,12 +21,21 @@ extern "C" __global__ void __launch_bounds__(256) ca_ffn_add_rows(const uint16_t
 __device__ __forceinline__ void tf_sum_routes(const uint16_t* routes, long long row, int c8, int topk, int hidden, float (&sum)[8]) {
 #pragma unroll
     for (int k = 0; k < 8; ++k) sum[k] = 0.f;
-    for (int slot = 0; slot < topk; ++slot) {
-        const u4v v = reinterpret_cast<const u4v*>(routes + (row * topk + slot) * hidden)[c8];
+    // eight slots' loads are requested together and added in slot order (a slot at a time, a thread of a few-row launch would
+    // wait for one round trip a slot)
+    for (int first = 0; first < topk; first += 8) {
+        u4v v[8];
 #pragma unroll
-        for (int j = 0; j < 4; ++j) {
-            sum[2 * j] = __fadd_rn(sum[2 * j], tf_bf16_lo(v[j]));
-            sum[2 * j + 1] = __fadd_rn(sum[2 * j + 1], tf_bf16_hi(v[j]));
+        for (int s = 0; s < 8; ++s)
+            if (first + s < topk) v[s] = reinterpret_cast<const u4v*>(routes + (row * topk + first + s) * hidden)[c8];
+#pragma unroll
+        for (int s = 0; s < 8; ++s) {
+            if (first + s >= topk) break;
+#pragma unroll
+            for (int j = 0; j < 4; ++j) {
+                sum[2 * j] = __fadd_rn(sum[2 * j], tf_bf16_lo(v[s][j]));
+                sum[2 * j + 1] = __fadd_rn(sum[2 * j + 1], tf_bf16_hi(v[s][j]));
+            }
         }
     }
 }
@@ -51,15 +60,17 @@ extern "C" __global__ void __launch_bounds__(256) ca_ffn_sum_shared(const uint16
     const long long i = (long long)blockIdx.x * blockDim.x + threadIdx.x, per_row = hidden >> 3;
     if (i * 8 >= n) return;
     const long long row = i / per_row;
-    u4v routed = reinterpret_cast<const u4v*>(routed_out)[i];
+    const u4v y = reinterpret_cast<const u4v*>(shared)[i];          // requested with the routes, not after their sum
+    u4v routed;
     if (row < live) {
         float sum[8];
         tf_sum_routes(routes, row, (int)(i - row * per_row), topk, hidden, sum);
 #pragma unroll
         for (int j = 0; j < 4; ++j) routed[j] = tf_pack_bf16(sum[2 * j], sum[2 * j + 1]);
         reinterpret_cast<u4v*>(routed_out)[i] = routed;
+    } else {
+        routed = reinterpret_cast<const u4v*>(routed_out)[i];
     }
-    const u4v y = reinterpret_cast<const u4v*>(shared)[i];
     u4v o;
 #pragma unroll
     for (int j = 0; j < 4; ++j)
