@@ -36,6 +36,30 @@ def test_router_logits_bit_exact(hidden, experts, rows):
     assert native.load().ca_router_logits(0, native.ptr(dx), native.ptr(dw), native.ptr(out), None) == -1
 
 
+def test_many_row_router_logits_both_tile_heights():
+    # the many-row gate product runs 64-row workgroup tiles below 256 workgroups and 128-row tiles from there on; every logit is
+    # the same sum in the same order either way: 32,805 rows (128-row tiles, ragged last tile) must hold, bit for bit, what its
+    # first 1,000 rows give on their own (64-row tiles), and a sample of rows is held to the oracle's fixed-order product
+    hidden, experts = 512, 320                     # two expert groups of 256: the second one ragged
+    g = geometry(hidden, experts, 2, 512, 512)
+    configure(g)
+    rows = 32805
+    x = synth.activations("logits-wide", rows, hidden).cuda()
+    w = synth.to_bf16_bits(synth.normal("logits-wide/w", (experts, hidden), std=hidden ** -0.5)).cuda()
+    lib = native.load()
+    big = torch.full((rows, experts), float("nan"), dtype=torch.float32, device="cuda")
+    small = torch.full((1000, experts), float("nan"), dtype=torch.float32, device="cuda")
+    assert lib.ca_router_logits_wide(rows, native.ptr(x), native.ptr(w), native.ptr(big), None) == 0
+    assert lib.ca_router_logits_wide(1000, native.ptr(x), native.ptr(w), native.ptr(small), None) == 0
+    torch.cuda.synchronize()
+    assert torch.equal(big[:1000].view(torch.int32), small.view(torch.int32))
+    assert not torch.isnan(big).any()
+    sample = np.unique(np.concatenate([np.arange(0, rows, 1999), [63, 64, 127, 128, 999, rows - 38, rows - 37, rows - 1]]))
+    want = oracle.router_logits(u16(x[torch.as_tensor(sample).cuda()].cpu()), u16(w.cpu()))
+    got = np_of(big)[sample]
+    assert np.abs(got - want).max() <= 1e-5 * np.abs(want).max() + 1e-6
+
+
 @pytest.mark.parametrize("mode,experts,topk", [("benchmark", 256, 6), ("reference", 384, 6), ("reference", 128, 3), ("benchmark", 16, 2)])
 def test_route_topk_bit_exact(mode, experts, topk):
     g = geometry(1024, experts, topk, 512, 512, mode)

@@ -516,8 +516,14 @@ int router_logits_wide_of(const ca_geometry& g, int rows, const void* x, const v
     if (rows < 1 || !x || !w || !out) return -1;
     if (rows <= 16) return router_logits_of(g, rows, x, w, out, stream);
     if (g.hidden % 64) return -4;
+    // 128-row workgroup tiles once they give every CU of the part (256) a workgroup; 64-row tiles below that
     const dim3 grid((rows + 127) / 128, (g.experts + 255) / 256);
-    ca_router_logits_mfma<<<grid, 512, 0, (hipStream_t)stream>>>((const uint16_t*)x, (const uint16_t*)w, (float*)out, rows, g.hidden, g.experts);
+    if (grid.x * grid.y >= 256) {
+        ca_router_logits_mfma<<<grid, 512, 0, (hipStream_t)stream>>>((const uint16_t*)x, (const uint16_t*)w, (float*)out, rows, g.hidden, g.experts);
+    } else {
+        const dim3 half((rows + 63) / 64, grid.y);
+        tf_router_logits_mfma_64<<<half, 512, 0, (hipStream_t)stream>>>((const uint16_t*)x, (const uint16_t*)w, (float*)out, rows, g.hidden, g.experts);
+    }
     return launch_status();
 }
 int shared_swiglu_of(const ca_geometry& g, int rows, const void* input, void* output, void* stream) {

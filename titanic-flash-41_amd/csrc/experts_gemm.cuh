@@ -427,85 +427,97 @@ inline int tf_launch_shared_fc1_gemm(const GemmArgs& a, int cus, hipStream_t s) 
 }
 
 // Gate product for many rows: logits[rows][experts] = x . w^T, BF16 inputs, FP32 accumulate on the matrix cores
-// (v_mfma_f32_32x32x16_bf16).  grid (ceil(rows / 128), ceil(experts / 256)), block 512: a workgroup keeps a 128 x 256 tile
-// of logits (wave (mr, nq): rows 64 mr .., experts 64 nq ..: 2 x 2 accumulators of 32 x 32), so the rows are read from HBM
-// once and the gate weight (2 MB) from L2 once per 128 rows.  Both operands go through LDS, 64 columns of K a step, double
-// buffered, loaded as whole 128-byte row pieces (eight lanes a row) and stored in matrix-instruction fragment order: the
-// 16-byte piece kc of row r of a 32-row tile sits in block (tile, kc / 2), half kc % 2, slot (r + 2 kc) % 32; the rotation
-// by 2 kc keeps both the stores (two rows x eight pieces a phase) and the fragment reads free of bank conflicts.
+// (v_mfma_f32_32x32x16_bf16).  grid (ceil(rows / (32 XT)), ceil(experts / 256)), block 512: a workgroup keeps a 32 XT x 256 tile
+// of logits, XT = 4 or 2 (wave (mr, nq): rows 16 XT mr .., experts 64 nq ..: XT / 2 x 2 accumulators of 32 x 32), so the rows
+// are read from HBM once and the gate weight (2 MB) from L2 once per 32 XT rows.  Both operands go through LDS, 64 columns of K
+// a step, double buffered, loaded as whole 128-byte row pieces (eight lanes a row) and stored in matrix-instruction fragment
+// order: the 16-byte piece kc of row r of a 32-row tile sits in block (tile, kc / 2), half kc % 2, slot (r + 2 kc) % 32; the
+// rotation by 2 kc keeps both the stores (two rows x eight pieces a phase) and the fragment reads free of bank conflicts.
+// Every logit is the same sum in the same order for either tile height.
 typedef __bf16 bf16x8 __attribute__((ext_vector_type(8)));
 typedef float v16f __attribute__((ext_vector_type(16)));
-extern "C" __global__ void __launch_bounds__(512) ca_router_logits_mfma(const uint16_t* x, const uint16_t* w, float* out, int rows,
-                                                                        int hidden, int experts) {
-    constexpr int X_TILES = 4, W_TILES = 8, STAGE = (X_TILES + W_TILES) * 4 * 1024;      // 32-row tiles; 4 KiB a tile and step
+template <int XT>
+__device__ __forceinline__ void tf_router_logits_tile(const uint16_t* x, const uint16_t* w, float* out, int rows, int hidden, int experts) {
+    static_assert(XT == 2 || XT == 4, "64 or 128 rows a workgroup");
+    constexpr int X_TILES = XT, W_TILES = 8, STAGE = (X_TILES + W_TILES) * 4 * 1024;      // 32-row tiles; 4 KiB a tile and step
+    constexpr int XA = XT / 2;                    // 32-row tiles of x a wave; also this thread's x pieces a step
+    constexpr int NP = XA + 4;                    // this thread's pieces of a step: x: 32 XT rows x 8 pieces (XA a thread); w: 256 rows x 8 (4 a thread)
     __shared__ __attribute__((aligned(16))) uint8_t s_ops[2][STAGE];
     const int tid = threadIdx.x, lane = tid & 63, wave = __builtin_amdgcn_readfirstlane(tid >> 6), mr = wave >> 2, nq = wave & 3;
     const int r32 = lane & 31, kg = lane >> 5;
-    const int row0 = blockIdx.x * 128, e0 = blockIdx.y * 256;
-    // this thread's pieces of a step: x: 128 rows x 8 pieces = 1,024 (2 a thread); w: 256 rows x 8 = 2,048 (4 a thread)
-    const uint16_t* src[6];
-    int dst[6];
+    const int row0 = blockIdx.x * (32 * XT), e0 = blockIdx.y * 256;
+    const uint16_t* src[NP];
+    int dst[NP];
 #pragma unroll
-    for (int i = 0; i < 6; ++i) {
-        const int c = tid + 512 * i, is_w = i >= 2, local = is_w ? c - 1024 : c, r = local >> 3, kc = local & 7;
+    for (int i = 0; i < NP; ++i) {
+        const int is_w = i >= XA, local = tid + 512 * (is_w ? i - XA : i), r = local >> 3, kc = local & 7;
         const int tile = (is_w ? X_TILES : 0) + (r >> 5);
         const long long source_row = is_w ? min(e0 + r, experts - 1) : min(row0 + r, rows - 1);
         src[i] = (is_w ? w : x) + source_row * hidden + kc * 8;
         dst[i] = ((tile * 4 + (kc >> 1)) * 64 + (kc & 1) * 32 + ((r + 2 * kc) & 31)) * 16;
     }
-    v16f acc[2][2];
+    v16f acc[XA][2];
 #pragma unroll
-    for (int a = 0; a < 2; ++a)
+    for (int a = 0; a < XA; ++a)
 #pragma unroll
         for (int b = 0; b < 2; ++b)
 #pragma unroll
             for (int i = 0; i < 16; ++i) acc[a][b][i] = 0.f;
     // operands of step s + 3 are requested while step s is multiplied: a ring of three register sets (indexed statically by
-    // unrolling four steps; hidden % 512 == 0), one LDS stage ahead of the products
+    // unrolling four steps; hidden % 256 == 0), one LDS stage ahead of the products
     constexpr int D = 4;
-    u4v regs[D][6];
+    u4v regs[D][NP];
     const int steps = hidden / 64;
 #pragma unroll
     for (int d = 0; d < D - 1; ++d)
 #pragma unroll
-        for (int i = 0; i < 6; ++i) regs[d][i] = *reinterpret_cast<const u4v*>(src[i] + (size_t)min(d, steps - 1) * 64);
+        for (int i = 0; i < NP; ++i) regs[d][i] = *reinterpret_cast<const u4v*>(src[i] + (size_t)min(d, steps - 1) * 64);
 #pragma unroll
-    for (int i = 0; i < 6; ++i) *reinterpret_cast<u4v*>(&s_ops[0][dst[i]]) = regs[0][i];
+    for (int i = 0; i < NP; ++i) *reinterpret_cast<u4v*>(&s_ops[0][dst[i]]) = regs[0][i];
     __syncthreads();
     for (int step0 = 0; step0 < steps; step0 += D) {
 #pragma unroll
         for (int u = 0; u < D; ++u) {
             const int step = step0 + u, stage = step & 1, ahead = min(step + D - 1, steps - 1);
 #pragma unroll
-            for (int i = 0; i < 6; ++i) regs[(u + D - 1) % D][i] = *reinterpret_cast<const u4v*>(src[i] + (size_t)ahead * 64);
+            for (int i = 0; i < NP; ++i) regs[(u + D - 1) % D][i] = *reinterpret_cast<const u4v*>(src[i] + (size_t)ahead * 64);
 #pragma unroll
             for (int sub = 0; sub < 4; ++sub) {
                 const int slot = (r32 + 4 * sub + 2 * kg) & 31;                 // (r + 2 kc) % 32 with kc = 2 sub + kg
-                u4v av[2], bv[2];
+                u4v av[XA], bv[2];
 #pragma unroll
-                for (int a = 0; a < 2; ++a) av[a] = *reinterpret_cast<const u4v*>(&s_ops[stage][(((2 * mr + a) * 4 + sub) * 64 + kg * 32 + slot) * 16]);
+                for (int a = 0; a < XA; ++a) av[a] = *reinterpret_cast<const u4v*>(&s_ops[stage][(((XA * mr + a) * 4 + sub) * 64 + kg * 32 + slot) * 16]);
 #pragma unroll
                 for (int b = 0; b < 2; ++b) bv[b] = *reinterpret_cast<const u4v*>(&s_ops[stage][(((X_TILES + 2 * nq + b) * 4 + sub) * 64 + kg * 32 + slot) * 16]);
 #pragma unroll
-                for (int a = 0; a < 2; ++a)
+                for (int a = 0; a < XA; ++a)
 #pragma unroll
                     for (int b = 0; b < 2; ++b)
                         acc[a][b] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(__builtin_bit_cast(bf16x8, av[a]), __builtin_bit_cast(bf16x8, bv[b]), acc[a][b], 0, 0, 0);
             }
 #pragma unroll
-            for (int i = 0; i < 6; ++i) *reinterpret_cast<u4v*>(&s_ops[stage ^ 1][dst[i]]) = regs[(u + 1) % D][i];
+            for (int i = 0; i < NP; ++i) *reinterpret_cast<u4v*>(&s_ops[stage ^ 1][dst[i]]) = regs[(u + 1) % D][i];
             __syncthreads();
         }
     }
 #pragma unroll
-    for (int a = 0; a < 2; ++a)
+    for (int a = 0; a < XA; ++a)
 #pragma unroll
         for (int b = 0; b < 2; ++b) {
             const int e = e0 + (2 * nq + b) * 32 + r32;
 #pragma unroll
             for (int i = 0; i < 16; ++i) {
-                const int row = row0 + (2 * mr + a) * 32 + 8 * (i >> 2) + 4 * kg + (i & 3);      // D[m][n = lane % 32]
+                const int row = row0 + (XA * mr + a) * 32 + 8 * (i >> 2) + 4 * kg + (i & 3);      // D[m][n = lane % 32]
                 if (row < rows && e < experts) out[(size_t)row * experts + e] = acc[a][b][i];
             }
         }
+}
+extern "C" __global__ void __launch_bounds__(512) ca_router_logits_mfma(const uint16_t* x, const uint16_t* w, float* out, int rows,
+                                                                        int hidden, int experts) {
+    tf_router_logits_tile<4>(x, w, out, rows, hidden, experts);
+}
+// 64 rows a workgroup: twice the workgroups for the same rows (for row counts whose 128-row tiles leave CUs without one).
+__global__ void __launch_bounds__(512) tf_router_logits_mfma_64(const uint16_t* x, const uint16_t* w, float* out, int rows, int hidden,
+                                                                 int experts) {
+    tf_router_logits_tile<2>(x, w, out, rows, hidden, experts);
 }
