@@ -160,6 +160,7 @@ def test_the_bf16_intermediate_is_only_a_tap_on_the_many_row_path():
     layer.keep_intermediate(False)
     layer.run(x.cuda())
     without = layer.taps()
-    for name in ["hq", "hs", "route_out", "out"]:
+    # the same switch drops the shared expert's BF16 taps (its projections before the activation and its activation)
+    for name in ["hq", "hs", "route_out", "shared_aq", "shared_as", "shared_down", "out"]:
         assert np.array_equal(with_tap[name], without[name]), name
     layer.close()

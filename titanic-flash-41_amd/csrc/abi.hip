@@ -425,7 +425,9 @@ int launch_dense(const Context& c, const uint64_t* p, const int32_t* sc, hipStre
 int launch_shared(const Context& c, const uint64_t* p, const int32_t* sc, hipStream_t s) {
     const ca_geometry& g = c.g;
     const int m = sc[0];
-    for (int i = 0; i < H_COUNT; ++i) if (!p[i] && i != H_UP_TAP && i != H_ACT_CODES && i != H_ACT_SCALES) return -1;
+    // many rows: the second projection reads the FP8 codes, so the BF16 activation is a tap like the projections before it
+    for (int i = 0; i < H_COUNT; ++i)
+        if (!p[i] && i != H_UP_TAP && i != H_ACT_CODES && i != H_ACT_SCALES && !(i == H_ACT && m > TF_STREAM_MAX_ROWS)) return -1;
     if (m < 1 || !supported_hidden(g.hidden) || !supported_k(g.shared_intermediate)) return -4;
     if (m <= TF_STREAM_MAX_ROWS) {
         StreamArgs a, b, none{};

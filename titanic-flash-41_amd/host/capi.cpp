@@ -120,7 +120,6 @@ long long tfh_checkpoint_contract(const char* prefix, const ca_geometry* geometr
 void tfh_layer_destroy(void* handle) { delete (Handle*)handle; }
 // The geometry the layer runs with (the caller's, with the expert widths padded to multiples of 512): the widths of the taps.
 void tfh_layer_geometry(void* handle, ca_geometry* out) { *out = ((Handle*)handle)->native->geometry(); }
-// Many rows: drop (0) or keep (1) the BF16 tap of the routed intermediate.
 // Test hooks of the front-end's in-launch hand-offs: the bound of its waits, and the host's reset of the `sync` region.
 int tfh_layer_spin_limit(void* handle, int limit, char* error, size_t error_len) {
     Handle* h = (Handle*)handle;
@@ -133,7 +132,15 @@ int tfh_layer_zero_sync(void* handle, char* error, size_t error_len) {
         tf::check(hipMemset((void*)h->workspace->at("sync_ptr"), 0, h->workspace->bytes_of("sync_ptr")), "zero sync region");
     });
 }
-void tfh_layer_keep_intermediate(void* handle, int on) { ((Handle*)handle)->workspace->keep_intermediate(on != 0); }
+// Many rows: drop (0) or keep (1) the BF16 taps of the routed intermediate and of the shared expert (its projections before
+// the activation, its activation): both second projections read the FP8 codes.
+void tfh_layer_keep_intermediate(void* handle, int on) {
+    Handle* h = (Handle*)handle;
+    h->workspace->keep_intermediate(on != 0);
+    h->layer->keep_intermediate(on != 0);
+    if (h->layer_b) h->layer_b->keep_intermediate(on != 0);
+    if (h->layer_pool) h->layer_pool->keep_intermediate(on != 0);
+}
 
 int tfh_layer_set_tokens(void* handle, const int64_t* ids, int live, const int32_t* padding, char* error, size_t error_len) {
     Handle* h = (Handle*)handle;

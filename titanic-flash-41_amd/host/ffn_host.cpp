@@ -565,8 +565,10 @@ void LayerFfn::run_shared(const Workspace& workspace, uint64_t input, const Stre
 }
 void LayerFfn::run_shared_quantized(uint64_t codes, uint64_t scales, const Stream& stream) {
     ensure(codes && scales, "prequantized normalized shared input requires both operands");
-    const uint64_t p[11] = {codes, scales, shared_w13_.values, shared_w13_.scales, shared_w2_.values, shared_w2_.scales, activation_.ptr(),
-                            activation_codes_.ptr(), activation_scales_.ptr(), shared_up_.ptr(), shared_down_.ptr()};
+    // many rows: the BF16 activation and the projections before it are taps (the second projection reads the codes)
+    const bool taps = keep_intermediate_ || rows_ <= 64;
+    const uint64_t p[11] = {codes, scales, shared_w13_.values, shared_w13_.scales, shared_w2_.values, shared_w2_.scales, taps ? activation_.ptr() : 0,
+                            activation_codes_.ptr(), activation_scales_.ptr(), taps ? shared_up_.ptr() : 0, shared_down_.ptr()};
     const int32_t s[1] = {(int32_t)rows_};
     native_->primitive(5, p, 11, s, 1, stream.raw(), "ffn.shared_expert");
 }

@@ -271,6 +271,9 @@ public:
     // Row transport of the sequence-parallel prefill on one rank (src/ffn.rs:789-878): the rows are routed, packed into wire rows
     // by the fused producer, (gathered: with one rank the rows are already all here), the shared quantizer's codes are decoded
     // from them, the routed experts run from the packed rows and the shared expert from the decoded codes.
+    // many rows: whether the shared expert also stores its BF16 taps (projections before the activation, the activation); the
+    // second projection reads the FP8 codes.  Few rows always keep them (there the BF16 activation is the hand-over).
+    void keep_intermediate(bool on) { keep_intermediate_ = on; }
     void enable_row_transport();
     bool row_transport_active() const { return packed_.len() != 0; }
     void run_row_transport(Workspace& workspace, uint64_t input, size_t input_len, const TokenRows& tokens, const Stream& stream);
@@ -287,6 +290,7 @@ private:
     Buffer<uint8_t> activation_codes_, activation_scales_;
     size_t rows_;
     Options options_;
+    bool keep_intermediate_ = true;
     std::unique_ptr<Stream> branch_stream_;
     std::unique_ptr<Event> input_ready_, output_ready_;
 };
