@@ -255,18 +255,22 @@ def measure(pkg, name, numerics, steps, warmup, profile_steps, overlap, operands
     step_flops = fc1_flops + fc2_flops + rows * (6 * H * S + 2 * H * E)
     max_load = float(np.mean([np.bincount(ids[ids >= 0].ravel(), minlength=E).max() for ids in ids_per_batch]))
 
-    # whole-layer throughput: one graph holds a pass over each of the input batches (as the reference's graph holds its forty
-    # layers' passes); a step is one pass.  Step counts that are no multiple of the batch count end with a shorter graph over
-    # the first batches, so exactly the steps asked for run, in the warm-up and in the timed region
-    full = layer.capture(xs)
-    tails = {}
+    # whole-layer throughput by graph replay (as the reference replays a graph of its forty layers' passes); a step is one pass,
+    # the input batches take turns.  A graph holds `per_graph` passes; a count that is no multiple of it ends with a graph of
+    # exactly the remainder, so exactly the steps asked for run, in the warm-up and in the timed region (a short count is one
+    # graph of its own: a second graph's first launch costs the region about 30 us)
+    per_graph = batches if wide else 16 * batches
+    graphs = {}
+
+    def graph_of(passes):
+        if passes not in graphs:
+            graphs[passes] = layer.capture([xs[i % batches] for i in range(passes)])
+        return graphs[passes]
 
     def launches(count):
-        order = [full] * (count // batches)
-        if count % batches:
-            if count % batches not in tails:
-                tails[count % batches] = layer.capture(xs[:count % batches])
-            order.append(tails[count % batches])
+        order = [graph_of(per_graph)] * (count // per_graph)
+        if count % per_graph:
+            order.append(graph_of(count % per_graph))
         return order
     warm_order, timed_order = launches(warmup), launches(steps)
     torch.cuda.synchronize()
@@ -307,11 +311,11 @@ def measure(pkg, name, numerics, steps, warmup, profile_steps, overlap, operands
                     "timing": "HIP events bound to the kernel's start and completion (hipExtLaunchKernelGGL) on its launch stream, eager passes of the layer's schedule"}
     record = {
         "value": value, "unit": "tokens/s", "steps": steps, "warmup": warmup, "ms_per_step": ms_per_step,
-        "steps_note": "%d steps after %d warm-up steps: replays of a %d-pass graph, a shorter graph for the remainder" % (steps, warmup, batches),
+        "steps_note": "%d steps after %d warm-up steps: replays of a %d-pass graph, a graph of exactly the remainder after them" % (steps, warmup, per_graph),
         "config": {"workload": name + ": " + cfg["workload"],
                    "numerics": ("sigmoid top-k renormalised, 128-wide activation blocks" if numerics == "benchmark" else
                                 "reference numerics: sqrt-softplus scores x 1.5, 32-wide activation blocks, 32 x 32 shared weight blocks"),
-                   "input_batches": batches, "distinct_experts_per_step": distinct, "schedule": "HIP graph replay (%d passes a graph)" % batches},
+                   "input_batches": batches, "distinct_experts_per_step": distinct, "schedule": "HIP graph replay (%d passes a graph)" % per_graph},
         "roofline": roofline,
         "step_tflops": step_flops / (ms_per_step * 1e-3) / 1e12, "busiest_expert_rows": max_load, "phys_tiles": tiles,
         "step_bytes": step_bytes, "step_gbs": step_bytes / (ms_per_step * 1e-3) / 1e9, "step_hbm_frac": step_bytes / (ms_per_step * 1e-3) / 1e9 / HBM_PEAK_GBS,
