@@ -452,11 +452,18 @@ __global__ void __launch_bounds__(256, 2) tf_phase2_stream(const StreamArgs rout
     if (routed.w) tf_plan_preload(routed, plan);
     const long long r_items = routed.w ? (long long)plan.tiles * (routed.hidden / 64) : 0;
     const long long s_items = shared.w ? (long long)tf_tiles(shared) * (shared.hidden / 32) : 0;
-    const long long total = r_items + s_items;
-    const long long lo = total * blockIdx.x / gridDim.x, hi = total * (blockIdx.x + 1) / gridDim.x;
+    // Equal cost shares of the list "routed items, then shared items", in quarter items.  Every item streams the same bytes; a
+    // shared item of an owner with more than eight rows counts a quarter more: its workgroup quantizes a row tile that is full
+    // or nearly so (four rounds of loads instead of one or two) for the four to six items it takes, and the launch ends with
+    // the slowest workgroup.  An item belongs to the workgroup whose cost range holds its start.
+    const long long cs = 4 + (shared.w && shared.dense_rows > 8 ? 1 : 0);
+    const long long r_cost = 4 * r_items, cost = r_cost + cs * s_items;
+    const long long lo = cost * blockIdx.x / gridDim.x, hi = cost * (blockIdx.x + 1) / gridDim.x;
+    const long long r_lo = min(r_items, (lo + 3) / 4), r_hi = min(r_items, (hi + 3) / 4);
+    const long long s_lo = lo > r_cost ? min(s_items, (lo - r_cost + cs - 1) / cs) : 0, s_hi = hi > r_cost ? min(s_items, (hi - r_cost + cs - 1) / cs) : 0;
     const int kmax = routed.w && (!shared.w || routed.k > shared.k) ? routed.k : shared.k;
-    if (lo < r_items) tf_fc2_items<false, KSR>(routed, (int)lo, (int)(hi < r_items ? hi : r_items), red, dyn, dyn + 16 * (size_t)kmax, plan);
-    if (hi > r_items) tf_fc2_items<true, KSS>(shared, (int)(lo > r_items ? lo - r_items : 0), (int)(hi - r_items), red, dyn, dyn + 16 * (size_t)kmax, plan);
+    if (r_lo < r_hi) tf_fc2_items<false, KSR>(routed, (int)r_lo, (int)r_hi, red, dyn, dyn + 16 * (size_t)kmax, plan);
+    if (s_lo < s_hi) tf_fc2_items<true, KSS>(shared, (int)s_lo, (int)s_hi, red, dyn, dyn + 16 * (size_t)kmax, plan);
 }
 
 // The experts' front-end with the shared expert's first projection in the same launch (few-row owners, hidden <= 5,120).
