@@ -421,7 +421,7 @@ __device__ __forceinline__ void tf_fc2_items(const StreamArgs& p, int item_first
 
 // Persistent launch of one phase over the routed experts and, optionally, the shared expert (`shared.w == nullptr`: routed
 // only; `routed.w == nullptr`: dense only).  Every item costs the same bytes (a shared FC1 item counts twice), so workgroup
-// b of G takes the cost range [b C / G, (b + 1) C / G) of the list "routed items, then shared items".  block = 64 WAVES:
+// b of G takes the cost range [b C / G, (b + 1) C / G) of the list "routed items, then shared items" (the second phase: shared first).  block = 64 WAVES:
 // four waves, two workgroups a CU, for K <= 4,096; eight waves, one workgroup a CU, above (a wave's share of K stays at
 // most eight k-steps: what the registers hold of the A tile and a unit of weights).
 template <int KSR, int KSS, int WAVES = 4>
@@ -452,18 +452,20 @@ __global__ void __launch_bounds__(256, 2) tf_phase2_stream(const StreamArgs rout
     if (routed.w) tf_plan_preload(routed, plan);
     const long long r_items = routed.w ? (long long)plan.tiles * (routed.hidden / 64) : 0;
     const long long s_items = shared.w ? (long long)tf_tiles(shared) * (shared.hidden / 32) : 0;
-    // Equal cost shares of the list "routed items, then shared items", in quarter items.  Every item streams the same bytes; a
+    // Equal cost shares of the list "shared items, then routed items", in quarter items.  Every item streams the same bytes; a
     // shared item of an owner with more than eight rows counts a quarter more: its workgroup quantizes a row tile that is full
     // or nearly so (four rounds of loads instead of one or two) for the four to six items it takes, and the launch ends with
-    // the slowest workgroup.  An item belongs to the workgroup whose cost range holds its start.
+    // the slowest workgroup.  An item belongs to the workgroup whose cost range holds its start.  (Dealing the last items out
+    // by an atomic counter instead, to whichever workgroup is done first, was measured: the device-scope atomics travel the
+    // same congested request path as the weights, and 512 of them at the workgroups' exits alone cost 1.5 us.)
     const long long cs = 4 + (shared.w && shared.dense_rows > 8 ? 1 : 0);
-    const long long r_cost = 4 * r_items, cost = r_cost + cs * s_items;
+    const long long s_cost = cs * s_items, cost = s_cost + 4 * r_items;
     const long long lo = cost * blockIdx.x / gridDim.x, hi = cost * (blockIdx.x + 1) / gridDim.x;
-    const long long r_lo = min(r_items, (lo + 3) / 4), r_hi = min(r_items, (hi + 3) / 4);
-    const long long s_lo = lo > r_cost ? min(s_items, (lo - r_cost + cs - 1) / cs) : 0, s_hi = hi > r_cost ? min(s_items, (hi - r_cost + cs - 1) / cs) : 0;
+    const long long s_lo = min(s_items, (lo + cs - 1) / cs), s_hi = min(s_items, (hi + cs - 1) / cs);
+    const long long r_lo = lo > s_cost ? min(r_items, (lo - s_cost + 3) / 4) : 0, r_hi = hi > s_cost ? min(r_items, (hi - s_cost + 3) / 4) : 0;
     const int kmax = routed.w && (!shared.w || routed.k > shared.k) ? routed.k : shared.k;
-    if (r_lo < r_hi) tf_fc2_items<false, KSR>(routed, (int)r_lo, (int)r_hi, red, dyn, dyn + 16 * (size_t)kmax, plan);
     if (s_lo < s_hi) tf_fc2_items<true, KSS>(shared, (int)s_lo, (int)s_hi, red, dyn, dyn + 16 * (size_t)kmax, plan);
+    if (r_lo < r_hi) tf_fc2_items<false, KSR>(routed, (int)r_lo, (int)r_hi, red, dyn, dyn + 16 * (size_t)kmax, plan);
 }
 
 // The experts' front-end with the shared expert's first projection in the same launch (few-row owners, hidden <= 5,120).
