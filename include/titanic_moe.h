@@ -159,6 +159,13 @@ int64_t ca_moe_dynamic_static_capacity(void);
  * context or a negative limit. */
 int32_t ca_primitives_spin_limit(void* context, int32_t limit);
 
+/* No counterpart in the reference.  Entry 5 (`ffn.shared_expert`) above 64 rows runs persistent workgroups, one a CU, which leave
+ * no room for other launches while they run.  A host that runs the router's small launches beside it on another stream (the
+ * dual-stream schedule of src/ffn.rs:1000-1040) sets `cus` (a multiple of 8, at most half the part's CUs; 0, the default: none)
+ * and the entry's first projection then leaves that many CUs without a workgroup.  The setting holds for the launches
+ * enqueued after it.  0, or -1 for a null context or a count outside that range. */
+int32_t ca_primitives_shared_reserve(void* context, int32_t cus);
+
 #ifdef __cplusplus
 }
 #endif

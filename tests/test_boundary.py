@@ -98,7 +98,7 @@ def test_contexts_carry_their_geometry_and_the_library_is_pinned(tmp_path):
     bad = native.Geometry(1000, 16, 2, 512, 512, 0, 1.0, 128, 128, 128, -1, 10.0)
     assert not lib.ca_primitives_open_geometry(ctypes.byref(bad), ctypes.byref(st)) and st.value == -4
     assert lib.ca_router_logits_in(None, 1, None, None, None, None) == -1 and lib.ca_ffn_add_in(None, 1, None, None, None, None) == -1
-    assert lib.ca_shared_swiglu_in(None, 1, None, None, None) == -1 and lib.ca_primitives_spin_limit(None, 1) == -1
+    assert lib.ca_shared_swiglu_in(None, 1, None, None, None) == -1 and lib.ca_primitives_spin_limit(None, 1) == -1 and lib.ca_primitives_shared_reserve(None, 8) == -1
     assert lib.ca_primitives_geometry(None, None) == -1
     # the host mirror refuses a kernel library whose SHA-256 differs from the manifest beside it (src/ffn.rs:70-74), before loading it
     shutil.copy(native.KERNEL_LIB, tmp_path / "libtitanic_moe_hip.so")

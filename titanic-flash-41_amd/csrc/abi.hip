@@ -49,6 +49,7 @@ struct Context {
     bool marking;
     bool kernel_marks;     // marks[5], marks[6]: begin and end of the FC1 + SwiGLU kernel itself
     int spin_limit;        // polls a wait inside the front-end launch may take before the waiter does the work itself
+    int shared_reserve;    // CUs the shared expert's many-row first projection leaves without a workgroup (0: none)
     int device;            // the device the context was opened on
     uint8_t* static_scratch;   // that device's copy of `scratch`
 };
@@ -442,7 +443,8 @@ int launch_shared(const Context& c, const uint64_t* p, const int32_t* sc, hipStr
     a.dense_rows = m; a.k = g.hidden; a.inter = g.shared_intermediate; a.hidden = g.hidden; a.act_block = g.act_block;
     a.limit = g.swiglu_limit; a.h_bf16 = (uint16_t*)p[H_ACT]; a.h_codes = (uint8_t*)p[H_ACT_CODES]; a.h_scales = (uint8_t*)p[H_ACT_SCALES];
     a.tap = (uint16_t*)p[H_UP_TAP];
-    int status = tf_grouped_dense_shape_ok(a, true) ? tf_launch_grouped_dense<TF_GEMM_FC1_SHARED>(a, c.cus, s) : tf_launch_shared_fc1_gemm(a, c.cus, s);
+    // a host that runs the router beside this entry on another stream may keep some CUs free for it (ca_primitives_shared_reserve)
+    int status = tf_grouped_dense_shape_ok(a, true) ? tf_launch_grouped_dense<TF_GEMM_FC1_SHARED>(a, c.cus - c.shared_reserve, s) : tf_launch_shared_fc1_gemm(a, c.cus, s);
     if (status) return status;
     GemmArgs b{};
     b.a_codes = (const uint8_t*)p[H_ACT_CODES]; b.a_scales = (const uint8_t*)p[H_ACT_SCALES];
@@ -672,7 +674,7 @@ void* ca_primitives_open_geometry(const ca_geometry* geometry, int32_t* status) 
         g_static_scratch[device] = at;
     }
     Context* c = new Context{};
-    c->g = *geometry; c->cus = cus; c->stream_wgs = cus * 2; c->spin_limit = 1 << 18;
+    c->g = *geometry; c->cus = cus; c->stream_wgs = cus * 2; c->spin_limit = 1 << 18; c->shared_reserve = 0;
     c->device = device; c->static_scratch = (uint8_t*)g_static_scratch[device];
     return c;
 }
@@ -697,6 +699,11 @@ int32_t ca_primitives_marks(void* context, void* const* events, size_t count) {
 int32_t ca_primitives_spin_limit(void* context, int32_t limit) {
     if (!context || limit < 0) return -1;
     ((Context*)context)->spin_limit = limit;
+    return 0;
+}
+int32_t ca_primitives_shared_reserve(void* context, int32_t cus) {
+    if (!context || cus < 0 || cus % 8 || cus * 2 > ((Context*)context)->cus) return -1;
+    ((Context*)context)->shared_reserve = cus;
     return 0;
 }
 int32_t ca_primitives_launch(void* context, int32_t index, const uint64_t* pointers, size_t np, const int32_t* scalars, size_t ns,

@@ -85,6 +85,7 @@ Native::Native(const std::string& library, const ca_geometry& geometry) : g_(geo
     shared_swiglu_ = symbol<decltype(shared_swiglu_)>(lib_, "ca_shared_swiglu_in");
     ffn_add_ = symbol<decltype(ffn_add_)>(lib_, "ca_ffn_add_in");
     spin_limit_ = symbol<decltype(spin_limit_)>(lib_, "ca_primitives_spin_limit");
+    shared_reserve_ = symbol<decltype(shared_reserve_)>(lib_, "ca_primitives_shared_reserve");
     kernel_launch_ = symbol<decltype(kernel_launch_)>(lib_, "ca_kernel_launch");
     close_ = symbol<decltype(close_)>(lib_, "ca_primitives_close");
     launch_ = symbol<decltype(launch_)>(lib_, "ca_primitives_launch");
@@ -131,6 +132,13 @@ void Native::ffn_add(int rows, uint64_t routed, uint64_t shared, uint64_t out, h
     ensure(ffn_add_(ctx_, rows, (const void*)routed, (const void*)shared, (void*)out, s) == 0, "FFN shared addition launch failed");   // src/ffn.rs:1071-1082
 }
 void Native::spin_limit(int limit) const { ensure(spin_limit_(ctx_, limit) == 0, "spin limit rejected"); }
+int Native::compute_units() const {
+    int device = 0, cus = 0;
+    check(hipGetDevice(&device), "current device");
+    check(hipDeviceGetAttribute(&cus, hipDeviceAttributeMultiprocessorCount, device), "compute unit count");
+    return cus;
+}
+void Native::shared_reserve(int cus) const { ensure(shared_reserve_(ctx_, cus) == 0, "shared expert CU reserve rejected"); }
 void Native::launch(const char* name, uint32_t grid_x, uint32_t grid_y, uint32_t block, uint32_t shared, void** args, hipStream_t s) const {
     const uint32_t grid[3] = {grid_x, grid_y, 1}, blk[3] = {block, 1, 1};
     const int status = kernel_launch_(name, grid, blk, shared, args, s);
@@ -550,6 +558,7 @@ LayerFfn::LayerFfn(std::shared_ptr<const Native> native, std::shared_ptr<Weights
     shared_w2_ = prepare_shared(*native, *weights, "ffn.shared_experts.w2", g.hidden, g.shared_intermediate);
     output_.zero();
     if (options_.overlap) {                                                                                    // :700-706 SharedBranch
+        compute_units_ = native->compute_units();
         branch_stream_ = std::make_unique<Stream>();
         input_ready_ = std::make_unique<Event>();
         output_ready_ = std::make_unique<Event>();
@@ -600,8 +609,15 @@ void LayerFfn::run_quantized_input(Workspace& workspace, uint64_t input, size_t 
     if (branch) {
         input_ready_->record(stream.raw());
         input_ready_->wait(branch_stream_->raw());
+        // The branch's first projection runs beside the router's launches (gate product, top-k, plan, quantizer: about 60 us +
+        // 8 ns a row, on few CUs) and takes about 20 ns a row with one workgroup on every CU, which leaves the router no CU until
+        // it ends.  Up to 6,144 rows a quarter of the CUs stays free for the router (the projection gets a third longer, the
+        // router runs under it); beyond, the projection outlasts the router by more than that costs.
+        const int reserve = rows_ > 64 && rows_ <= 6144 ? compute_units_ / 32 * 8 : 0;
+        if (reserve) native_->shared_reserve(reserve);
         if (quantized) run_shared_quantized(quantized->codes, quantized->scales, *branch_stream_);              // :1058-1064
         else run_shared(workspace, input, *branch_stream_);
+        if (reserve) native_->shared_reserve(0);
         output_ready_->record(branch_stream_->raw());
     }
     const std::optional<RouteOperands> route = router_.run_routed(input, input_len, tokens, fused, stream, options_.gate_front);

@@ -45,6 +45,9 @@ public:
     void marks(hipEvent_t* events, size_t count = 5) const;      // 5: between the launches; 7: + the FC1 kernel's own begin / end
     // polls a wait inside the front-end launch may take before the waiter does the work itself (0: no hand-off is waited for)
     void spin_limit(int limit) const;
+    // CUs the many-row shared expert's first projection leaves free (ca_primitives_shared_reserve); holds for later launches
+    void shared_reserve(int cus) const;
+    int compute_units() const;          // of the current device
     // the wire row "dual_quant_rows_v1" (src/ffn.rs:805-811 RowTransport's functions)
     void codec_encode(uint64_t routed, uint64_t scales, uint64_t shared, uint64_t packed, int rows, int k, hipStream_t s) const;
     void codec_decode(uint64_t packed, uint64_t shared, uint64_t row_scales, uint64_t mma_scales, int rows, int k, hipStream_t s) const;
@@ -59,6 +62,7 @@ private:
     int (*shared_swiglu_)(void*, int, const void*, void*, void*) = nullptr;
     int (*ffn_add_)(void*, int, const void*, const void*, void*, void*) = nullptr;
     int32_t (*spin_limit_)(void*, int32_t) = nullptr;
+    int32_t (*shared_reserve_)(void*, int32_t) = nullptr;
     int (*kernel_launch_)(const char*, const uint32_t*, const uint32_t*, uint32_t, void**, void*) = nullptr;
     void (*close_)(void*) = nullptr;
     int32_t (*launch_)(void*, int32_t, const uint64_t*, size_t, const int32_t*, size_t, void*) = nullptr;
@@ -291,6 +295,7 @@ private:
     size_t rows_;
     Options options_;
     bool keep_intermediate_ = true;
+    int compute_units_ = 0;
     std::unique_ptr<Stream> branch_stream_;
     std::unique_ptr<Event> input_ready_, output_ready_;
 };

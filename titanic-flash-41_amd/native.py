@@ -14,7 +14,7 @@ EXPORTS = ["ca_ffn_abi", "ca_ffn_configure", "ca_ffn_geometry", "ca_router_logit
            "ca_router_logits_wide", "ca_kernel_launch", "ca_kernel_count", "ca_kernel_name", "ca_moe_nibble_permute",
            "ca_primitives_abi", "ca_primitives_open", "ca_primitives_close", "ca_primitives_launch", "ca_primitives_launch2",
            "ca_primitives_entries", "ca_primitives_scratch_bytes", "ca_primitives_marks", "ca_encode", "ca_decode", "ca_local_live",
-           "ca_pack_bf16", "ca_primitives_spin_limit", "ca_primitives_open_geometry", "ca_primitives_geometry", "ca_router_logits_in",
+           "ca_pack_bf16", "ca_primitives_spin_limit", "ca_primitives_shared_reserve", "ca_primitives_open_geometry", "ca_primitives_geometry", "ca_router_logits_in",
            "ca_router_logits_wide_in", "ca_shared_swiglu_in", "ca_ffn_add_in", "ca_moe_dynamic_static", "ca_moe_dynamic_static_capacity",
            "ca_ffn_norm_quant", "ca_ffn_sum_residual", "ca_hc_combine_norm_quant", "ca_hc_post", "ca_ffn_sum_hc_post"]
 
@@ -77,6 +77,8 @@ def load():
     lib.ca_primitives_marks.argtypes = [vp, ctypes.POINTER(vp), ctypes.c_size_t]
     lib.ca_primitives_spin_limit.restype = i32
     lib.ca_primitives_spin_limit.argtypes = [vp, i32]
+    lib.ca_primitives_shared_reserve.restype = i32
+    lib.ca_primitives_shared_reserve.argtypes = [vp, i32]
     lib.ca_primitives_open_geometry.restype = vp
     lib.ca_primitives_open_geometry.argtypes = [ctypes.POINTER(Geometry), i32p]
     lib.ca_primitives_geometry.restype = i32
